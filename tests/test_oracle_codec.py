@@ -1,0 +1,223 @@
+"""Pins the CPU oracle's block-float codec (no GPU).
+
+Sources of truth, none of which is the oracle's own formula retyped:
+  * known answers recorded from the compiled reference (tests/golden/reference_known_answers.json);
+  * the invariants of tests/tt_metal/tt_metal/test_bfp8_conversion.cpp and test_bfp4_conversion.cpp;
+  * an exact-arithmetic statement of the quantiser: code = min(floor(|x| / ulp + 1/2), max), ulp =
+    2**(E - 127 - (W-1)), which holds because floor((floor(y) + a) / b) == floor((y + a) / b) for
+    integers a, b > 0 — the truncating pre-shift of the reference cannot change the result;
+  * exact rational values of unpacked codes: sign * man * 2**(E - 127 - (W-1)).
+"""
+import json
+import os
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from ttmi import workloads
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+KNOWN = json.load(open(os.path.join(HERE, "golden", "reference_known_answers.json")))
+BFP8, BFP4 = 3, 4
+W = {BFP8: 7, BFP4: 3}
+
+
+def f32_bits(x):
+    return np.asarray(x, dtype=np.float32).view(np.uint32)
+
+
+def bits_f32(b):
+    return np.asarray(b, dtype=np.uint32).view(np.float32)
+
+
+def exact_value(bits: int) -> Fraction:
+    """Magnitude the reference's packer *sees*: hidden one present even when the exponent field is 0."""
+    e = (bits >> 23) & 0xFF
+    f = bits & 0x7FFFFF
+    return Fraction((1 << 23) | f) * Fraction(2) ** (e - 150)
+
+
+def exact_code(bits: int, shared: int, fmt: int) -> int:
+    if bits & 0x7FFFFFFF == 0:
+        return 0
+    w = W[fmt]
+    ulp = Fraction(2) ** (shared - 127 - (w - 1))
+    q = (exact_value(bits) / ulp + Fraction(1, 2)).__floor__()
+    q = min(q, (1 << w) - 1)
+    sign = (bits >> 31) if q else 0
+    return (sign << w) | q
+
+
+def test_tile_sizes(oracle):
+    # tt_backend_api_types.hpp:113-116, constants.hpp:20-21
+    assert oracle.lib().oracle_tile_size_bytes(BFP8) == 1088
+    assert oracle.lib().oracle_tile_size_bytes(BFP4) == 576
+
+
+def test_known_edge_rows_bfp8(oracle):
+    for case in KNOWN["edge_single_value_rows"]["cases"]:
+        bits = int(case["bits"], 16)
+        row = np.zeros(1024, dtype=np.uint32)
+        row[0] = bits
+        words = oracle.pack_fp32_vec_as_bfp_tiles(BFP8, row.view(np.float32), False)
+        assert words[0] & 0xFF == int(case["exp"], 16), case
+        assert words[16] & 0xFF == int(case["code"], 16), case
+        assert words[16] >> 8 == 0 and not words[17:].any()
+        back = oracle.unpack_bfp_tiles_into_float_vec(BFP8, words, False).view(np.uint32)
+        assert back[0] == int(case["unpacked"], 16), case
+        assert not back[1:].any()
+
+
+def test_known_row_with_max_one(oracle):
+    k = KNOWN["row_with_max_one"]
+    row = np.zeros(1024, dtype=np.float32)
+    row[: len(k["values"])] = k["values"]
+    words = oracle.pack_fp32_vec_as_bfp_tiles(BFP8, row, False)
+    codes = [(int(words[16]) >> (8 * i)) & 0xFF for i in range(3)]
+    assert codes == [int(c, 16) for c in k["codes"]]
+
+
+@pytest.mark.parametrize("fmt,key", [(BFP8, "first_mantissa_word_bfp8"), (BFP4, "first_mantissa_word_bfp4")])
+def test_arange_tile_known_words_and_reference_invariants(oracle, fmt, key):
+    """test_bfp8_conversion.cpp:29-74 / test_bfp4_conversion.cpp:29-74 re-run on the oracle."""
+    k = KNOWN["arange_tile"]
+    x = np.arange(1024, dtype=np.float32)
+    tiled = oracle.tilize_nchw_4faces(x.reshape(1, 1, 32, 32))
+    rm_in = oracle.pack_fp32_vec_as_bfp_tiles(fmt, x, True)
+    tile_in = oracle.pack_fp32_vec_as_bfp_tiles(fmt, tiled, False)
+    assert rm_in[0] == int(k["first_exponent_word"], 16)
+    assert rm_in[16] == int(k[key], 16)
+    assert np.array_equal(rm_in, tile_in)  # :51
+    rm_out = oracle.unpack_bfp_tiles_into_float_vec(fmt, rm_in, True)
+    tile_out = oracle.unpack_bfp_tiles_into_float_vec(fmt, tile_in, False)
+    rtol = 0.01 if fmt == BFP8 else 0.15
+    # is_close(a, b, rtol, atol) of bfloat16.hpp:370-383: |a-b| <= atol + rtol*max(|a|,|b|) style bound; 8.0 dominates here
+    assert np.all(np.abs(rm_out - x) <= 8.0 + rtol * np.abs(x))
+    assert np.all(np.abs(tile_out - tiled) <= 8.0 + rtol * np.abs(tiled))
+    assert np.array_equal(rm_out, oracle.untilize_nchw_4faces(tile_out, (1, 1, 32, 32)).reshape(-1))  # :73
+    assert np.array_equal(tile_out, oracle.tilize_nchw_4faces(rm_out.reshape(1, 1, 32, 32)))  # :74
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_element_converter_every_exponent_pair_exact_arithmetic(oracle, fmt):
+    """Every (own exponent, shared exponent >= own) pair with boundary mantissas, both signs."""
+    w = W[fmt]
+    half = 1 << (23 - w)  # half of an output ulp at gap 0, in fp32 fraction units
+    fracs = sorted({0, 1, half - 1, half, half + 1, 2 * half - 1, 2 * half, 2 * half + 1, 3 * half, 0x400000,
+                    0x7FFFFF - half, 0x7FFFFF - half + 1, 0x7FFFFF})
+    conv = oracle.lib().oracle_convert_u32_to_bfp
+    bad = 0
+    for own in range(256):
+        for shared in list(range(own, min(own + 30, 256))) + [255]:
+            if shared < own:
+                continue
+            for f in fracs:
+                for s in (0, 1):
+                    bits = (s << 31) | (own << 23) | f
+                    if conv(bits, shared, fmt) != exact_code(bits, shared, fmt):
+                        bad += 1
+    assert bad == 0
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_element_converter_random_exact_arithmetic(oracle, fmt):
+    rng = np.random.default_rng(7)
+    conv = oracle.lib().oracle_convert_u32_to_bfp
+    bits = rng.integers(0, 1 << 32, size=40000, dtype=np.uint64)
+    gaps = rng.integers(0, 34, size=bits.size)
+    for b, g in zip(bits.tolist(), gaps.tolist()):
+        own = (b >> 23) & 0xFF
+        shared = min(own + g, 255)
+        assert conv(b, shared, fmt) == exact_code(b, shared, fmt)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_shared_exponent_is_row_max_of_exponent_fields(oracle, fmt):
+    rng = np.random.default_rng(11)
+    x = rng.integers(0, 1 << 32, size=64 * 16, dtype=np.uint64).astype(np.uint32)
+    words = oracle.pack_fp32_vec_as_bfp_tiles(fmt, x.view(np.float32), False)
+    exps = words[:16].view(np.uint8)  # little endian: byte k of word w is row 4w+k
+    want = ((x >> 23) & 0xFF).reshape(64, 16).max(axis=1)
+    assert np.array_equal(exps, want.astype(np.uint8))
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_unpack_every_code_and_exponent_exact_value(oracle, fmt):
+    w = W[fmt]
+    dec = oracle.lib().oracle_bfp_code_to_u32
+    for shared in range(256):
+        for code in range(1 << (w + 1)):
+            got = dec(code, shared, fmt)
+            sign, man = code >> w, code & ((1 << w) - 1)
+            if man == 0:
+                assert got == sign << 31  # 0x80 / 0x8 -> -0.0f (bfloat8.hpp:232-244)
+                continue
+            sc = (w - 1) - (man.bit_length() - 1)
+            if shared - sc >= 1 and shared - sc <= 254:
+                val = Fraction(float(bits_f32(got)))
+                assert val == (-1) ** sign * Fraction(man) * Fraction(2) ** (shared - 127 - (w - 1))
+            else:
+                # exponent field <= 0 or 255: release-mode behaviour of bfloat8.hpp:244-249 (no assert): the
+                # int32 exponent is shifted into place with 32-bit wrap and OR-ed with sign and mantissa
+                frac = ((man << (sc + 1)) & ((1 << w) - 1)) << (23 - w)
+                assert got == ((sign << 31) | (((shared - sc) << 23) & 0xFFFFFFFF) | frac) & 0xFFFFFFFF
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_unpacked_values_fit_bf16_and_repack_is_identity(oracle, fmt):
+    x = workloads.stress_mixture((1, 1, 64, 256), seed=5)
+    words = oracle.pack_fp32_vec_as_bfp_tiles(fmt, x, False)
+    vals = oracle.unpack_bfp_tiles_into_float_vec(fmt, words, False)
+    assert not (vals.view(np.uint32) & 0xFFFF).any()  # at most 7 significant bits
+    assert np.array_equal(oracle.pack_fp32_vec_as_bfp_tiles(fmt, vals, False), words)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_unpack_error_bound_against_input(oracle, fmt):
+    """|unpack(pack(x)) - x| <= half an ulp of the row's shared exponent (plus saturation at the top code)."""
+    w = W[fmt]
+    x = workloads.normal_tensor((1, 1, 64, 64), seed=3)
+    flat = oracle.tilize_nchw_4faces(x)
+    words = oracle.pack_fp32_vec_as_bfp_tiles(fmt, flat, False)
+    vals = oracle.unpack_bfp_tiles_into_float_vec(fmt, words, False)
+    e = ((flat.view(np.uint32) >> 23) & 0xFF).reshape(-1, 16).max(axis=1).astype(np.int64)
+    ulp = np.exp2((e - 127 - (w - 1)).astype(np.float64))
+    err = np.abs(vals.astype(np.float64) - flat.astype(np.float64)).reshape(-1, 16)
+    assert np.all(err <= ulp[:, None])  # half ulp rounding, one ulp where the top code saturates
+    assert np.mean(err <= 0.5 * ulp[:, None]) > 0.95
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("shape", [(1, 1, 32, 32), (2, 3, 64, 96), (1, 1, 7, 3), (1, 2, 33, 65), (1, 1, 100, 48)])
+def test_from_torch_sequence_equals_single_pass(oracle, fmt, shape):
+    """The reference's pack(chunks) -> unpack -> tilize -> pack equals pack(tilize(pad(x))) and to_torch inverts it."""
+    count = int(np.prod(shape))
+    x = workloads.stress_mixture((1, 1, 1, -(-count // 16) * 16), seed=9).reshape(-1)[:count]
+    x = np.ascontiguousarray(x).reshape(shape)
+    full = oracle.from_torch_bfp_tiles(fmt, x)
+    single = oracle.pack_fp32_vec_as_bfp_tiles(fmt, oracle.tilize_nchw_4faces(x), False)
+    assert np.array_equal(full, single)
+    back = oracle.to_torch_bfp_tiles(fmt, full, shape)
+    hp, wp = -(-shape[2] // 32) * 32, -(-shape[3] // 32) * 32
+    direct = oracle.untilize_nchw_4faces(oracle.unpack_bfp_tiles_into_float_vec(fmt, full, False), (shape[0], shape[1], hp, wp))
+    assert np.array_equal(back.view(np.uint32), direct[:, :, : shape[2], : shape[3]].view(np.uint32))
+
+
+def test_reference_tolerances_test_to_and_from_torch(oracle):
+    """tests/ttnn/unit_tests/test_to_and_from_torch.py:22-42: 7x3 -> bfloat8_b/4_b TILE -> back."""
+    rng = np.random.default_rng(0)
+    x = workloads.bf16_bits_to_f32(workloads.f32_to_bf16_bits_rne(rng.random((7, 3), dtype=np.float32)))
+    b8 = oracle.to_torch_bfp_tiles(BFP8, oracle.from_torch_bfp_tiles(BFP8, x), (7, 3))
+    assert np.allclose(x, b8, atol=1e-2)
+    b4 = oracle.to_torch_bfp_tiles(BFP4, oracle.from_torch_bfp_tiles(BFP4, x), (7, 3))
+    assert np.corrcoef(x.reshape(-1), b4.reshape(-1))[0, 1] > 0.9
+
+
+def test_reference_tolerances_test_tensor(oracle):
+    """tests/tt_eager/python_api_testing/unit_testing/misc/test_tensor.py:26-91: (2,3,64,96), atol 1e-2 / 0.2."""
+    rng = np.random.default_rng(1)
+    x = rng.random((2, 3, 64, 96), dtype=np.float32)
+    b8 = oracle.to_torch_bfp_tiles(BFP8, oracle.from_torch_bfp_tiles(BFP8, x), x.shape)
+    b4 = oracle.to_torch_bfp_tiles(BFP4, oracle.from_torch_bfp_tiles(BFP4, x), x.shape)
+    assert np.allclose(x, b8, atol=1e-2) and np.allclose(x, b4, atol=0.2)
