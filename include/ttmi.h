@@ -1,0 +1,120 @@
+/*
+ * ttmi — block-float tensors on MI355X (gfx950): the C ABI.
+ *
+ * Every entry point is extern "C", takes plain pointers and sizes, returns an
+ * int status (TTMI_OK == 0) and never throws.  ttmi_last_error() gives the
+ * message of the last failure on the calling thread.  Unless a name says
+ * "host", pointers are DEVICE pointers (hipMalloc'd memory of the current
+ * device) and `stream` is a hipStream_t passed as void* (NULL = the null
+ * stream).  Launches are asynchronous on that stream.
+ *
+ * Each declaration cites the tt-metal interface it stands in for (paths
+ * relative to the tt-metal checkout).  The reference binds these through
+ * pybind11 (tt_eager/tt_lib/csrc/tt_lib_bindings_tensor_pytensor.cpp and
+ * ttnn/cpp/pybind11/operations/matmul.hpp); this C layer is what such a
+ * binding would call.
+ */
+#ifndef TTMI_H
+#define TTMI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTMI_API __attribute__((visibility("default")))
+
+/* status codes */
+enum {
+    TTMI_OK = 0,
+    TTMI_ERR_INVALID_ARGUMENT = 1, /* what TT_FATAL / TT_THROW reject in the reference */
+    TTMI_ERR_HIP = 2,              /* a HIP runtime call failed */
+    TTMI_ERR_UNSUPPORTED = 3
+};
+
+/* tt_eager/tensor/types.hpp:26-34 DataType — same numeric values */
+enum { TTMI_BFLOAT16 = 0, TTMI_FLOAT32 = 1, TTMI_UINT32 = 2, TTMI_BFLOAT8_B = 3, TTMI_BFLOAT4_B = 4, TTMI_UINT16 = 6 };
+
+/* tt_eager/tensor/types.hpp:24 Layout — same numeric values */
+enum { TTMI_ROW_MAJOR = 0, TTMI_TILE = 1 };
+
+/* fused activation of ttnn.linear (ttnn/ttnn/operations/matmul.py:59-63) */
+enum { TTMI_ACT_NONE = 0, TTMI_ACT_RELU = 1, TTMI_ACT_GELU = 2, TTMI_ACT_SILU = 3 };
+
+TTMI_API const char *ttmi_last_error(void);
+TTMI_API const char *ttmi_version(void);
+
+/* tt_metal/common/tt_backend_api_types.hpp:109-132 tile_size(DataFormat): bytes of one 32x32 tile
+ * (1088 bfloat8_b, 576 bfloat4_b, 2048 bfloat16/uint16, 4096 float32/uint32); 0 for an unknown dtype. */
+TTMI_API uint32_t ttmi_tile_size(int dtype);
+
+/* tt_eager/tensor/tensor_utils.hpp:33-49 compute_buffer_size: bytes of a [batch, h, w] tensor in TILE layout
+ * after h and w are rounded up to 32 (ttnn/ttnn/operations/core.py:793 pads with zeros). */
+TTMI_API size_t ttmi_tiled_size_bytes(int dtype, uint32_t batch, uint32_t h, uint32_t w);
+
+/* tt_metal/common/bfloat8.hpp:102 pack_fp32_vec_as_bfp8_tiles and bfloat4.hpp:23 pack_fp32_vec_as_bfp4_tiles
+ * (is_exp_a = false).  src: n_tiles*1024 fp32, each 1024-chunk a row-major 32x32 block (row_major_input != 0)
+ * or already in 4-face order.  dst: n_tiles * tile_size/4 words.  fmt: TTMI_BFLOAT8_B | TTMI_BFLOAT4_B. */
+TTMI_API int ttmi_pack_fp32_vec_as_bfp_tiles(int fmt, const float *src, size_t n_tiles, int row_major_input, uint32_t *dst,
+                                    void *stream);
+
+/* bfloat8.hpp:175 unpack_bfp8_tiles_into_float_vec and bfloat4.hpp:33 unpack_bfp4_tiles_into_float_vec
+ * (is_exp_a = false): inverse of the above, fp32 out. */
+TTMI_API int ttmi_unpack_bfp_tiles_into_float_vec(int fmt, const uint32_t *words, size_t n_tiles, int row_major_output,
+                                         float *dst, void *stream);
+
+/* The whole host sequence of ttnn.from_torch(dtype=bfloat8_b|bfloat4_b, layout=TILE_LAYOUT) in one pass
+ * (ttnn/ttnn/operations/core.py:276-309, tt_lib_bindings_tensor_pytensor.cpp:78-151,
+ * tt_eager/tensor/tensor_impl.cpp:179-197): zero-pad h, w to 32, tilize to 4-face tiles, pack.
+ * src: [batch, h, w] row-major, src_dtype TTMI_FLOAT32 or TTMI_BFLOAT16; consecutive rows are `row_stride`
+ * elements apart (pass w for a dense tensor) and consecutive [h, w] slices batch_stride elements apart
+ * (pass h*row_stride).  dst: ttmi_tiled_size_bytes(fmt, batch, h, w) bytes. */
+TTMI_API int ttmi_pack_rowmajor_as_bfp_tiles(int fmt, const void *src, int src_dtype, uint32_t batch, uint32_t h, uint32_t w,
+                                    size_t row_stride, size_t batch_stride, uint32_t *dst, void *stream);
+
+/* The whole host sequence of ttnn.to_torch for a block-float tensor (core.py:336-394, tensor_impl.cpp:179-197,
+ * tt_lib_bindings_tensor_pytensor.cpp:382-393): unpack, untilize, drop the tile padding.
+ * words: tiles of the padded tensor.  dst: dense [batch, h, w] row-major, dst_dtype TTMI_FLOAT32 (what the
+ * reference returns) or TTMI_BFLOAT16 (exact: unpacked values carry at most 7 significant bits). */
+TTMI_API int ttmi_unpack_bfp_tiles_as_rowmajor(int fmt, const uint32_t *words, uint32_t batch, uint32_t h, uint32_t w,
+                                      void *dst, int dst_dtype, void *stream);
+
+/* tt_metal/common/test_tiles.hpp:177 convert_layout(LIN_ROW_MAJOR -> TILED32_4FACES), which is what
+ * Tensor::to(Layout::TILE) runs (tt_eager/tensor/tensor_impl.hpp:158-165), and
+ * tt_metal/common/tilize_untilize.hpp:9 tilize.  elem_size 2 or 4.  src [batch, h, w] dense row-major;
+ * dst holds the zero-padded tensor in tile order. */
+TTMI_API int ttmi_tilize(const void *src, uint32_t elem_size, uint32_t batch, uint32_t h, uint32_t w, void *dst, void *stream);
+
+/* test_tiles.hpp:177 convert_layout(TILED32_4FACES -> LIN_ROW_MAJOR) (tensor_impl.hpp:167-171) and
+ * tilize_untilize.hpp:68 untilize.  src: tiles of the padded tensor; dst: dense [batch, h, w] (padding dropped). */
+TTMI_API int ttmi_untilize(const void *src, uint32_t elem_size, uint32_t batch, uint32_t h, uint32_t w, void *dst,
+                  void *stream);
+
+/* Bytes of scratch ttmi_matmul_bfp wants for these sizes (0 when none).  No reference counterpart: the
+ * reference's op allocates its circular buffers inside the program factory
+ * (tt_eager/tt_dnn/op_library/bmm/multi_core_reuse_mcast_1d_optimized/bmm_op_multi_core_reuse_mcast_1d_optimized.cpp:48-52). */
+TTMI_API size_t ttmi_matmul_bfp_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
+
+/* C[b, m, n] = act(A[b, m, k] . B[(b | 0), k, n] + bias[n]) with block-float weights:
+ * tt::operations::primary::matmul (tt_eager/tt_dnn/op_library/bmm/bmm_op.hpp:318-346, validate
+ * bmm_op.cpp:828-1049) as reached from ttnn.matmul / ttnn.linear (ttnn/cpp/ttnn/operations/matmul.hpp:44-214)
+ * and tt_lib.tensor.matmul / bmm (bmm_op.hpp:388-456).
+ *   a        bf16, [batch, m, k]; a_layout TTMI_ROW_MAJOR (dense) or TTMI_TILE (4-face tiles, tile (mt, kt) of
+ *            slice b at index (b*Mt + mt)*Kt + kt; m, k multiples of 32)
+ *   b        packed tiles, b_fmt TTMI_BFLOAT8_B | TTMI_BFLOAT4_B, tile (kt, nt) at index kt*Nt + nt, k and n
+ *            multiples of 32; b_batch is `batch` (bmm) or 1 (weights broadcast over the batch: bcast_batch)
+ *   bias     NULL or bf16 [n] (row-broadcast add, matmul.hpp:117-214)
+ *   c        c_dtype TTMI_BFLOAT16 (round to nearest even) or TTMI_FLOAT32; c_layout as for a
+ *   workspace NULL (the library keeps a per-device buffer of its own, allocated on first use) or at least
+ *            ttmi_matmul_bfp_workspace_bytes() bytes of device memory, 256-byte aligned
+ * fp32 accumulation throughout. */
+TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch,
+                    uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
+                    int c_dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTMI_H */

@@ -1,0 +1,179 @@
+"""GPU parity of the block-float codec kernels against the CPU oracle — bit exact, through the C ABI."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+from ttmi import capi, workloads  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+BFP8, BFP4 = capi.BFLOAT8_B, capi.BFLOAT4_B
+HERE = os.path.dirname(os.path.abspath(__file__))
+KNOWN = json.load(open(os.path.join(HERE, "golden", "reference_known_answers.json")))
+
+
+def dev(a: np.ndarray):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def words_np(t) -> np.ndarray:
+    return t.cpu().numpy().view(np.uint32)
+
+
+def special_values(shape, seed):
+    """fp32 patterns the packer treats specially: +-0, subnormals, Inf, NaN, huge and tiny exponents."""
+    rng = np.random.default_rng(seed)
+    n = int(np.prod(shape))
+    bits = rng.integers(0, 1 << 32, size=n, dtype=np.uint64).astype(np.uint32)
+    pool = np.array([0x00000000, 0x80000000, 0x00000001, 0x80000001, 0x00400000, 0x007FFFFF, 0x00800000, 0x7F800000,
+                     0xFF800000, 0x7FC00000, 0xFFC00001, 0x7F7FFFFF, 0x3F7FFFFF, 0x3F800000, 0xBF800000, 0x3EFFFFFF],
+                    dtype=np.uint32)
+    pick = rng.random(n) < 0.5
+    bits[pick] = pool[rng.integers(0, pool.size, size=int(pick.sum()))]
+    zero_rows = rng.random(n // 16 + 1) < 0.2
+    for r in np.nonzero(zero_rows)[0]:
+        bits[r * 16:(r + 1) * 16] &= 0x80000000
+    return bits[:n].view(np.float32).reshape(shape)
+
+
+SHAPES = [(1, 1, 32, 32), (2, 3, 64, 96), (1, 1, 7, 3), (1, 2, 33, 65), (1, 1, 100, 48), (1, 1, 32, 288), (3, 1, 1, 1),
+          (1, 1, 64, 4100)]
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_from_torch_and_to_torch_paths_bit_exact(oracle, fmt, shape):
+    for x in (workloads.normal_tensor(shape, seed=21), special_values(shape, seed=22)):
+        want = oracle.from_torch_bfp_tiles(fmt, x)
+        got = capi.pack_tensor(fmt, dev(x))
+        assert np.array_equal(words_np(got), want)
+        back = capi.unpack_tensor(fmt, got, shape)
+        want_back = oracle.to_torch_bfp_tiles(fmt, want, shape)
+        assert np.array_equal(back.cpu().numpy().view(np.uint32), want_back.view(np.uint32))
+        # bf16 destination is exact: same upper halves, lower halves were zero
+        back16 = capi.unpack_tensor(fmt, got, shape, dtype=torch.bfloat16)
+        assert np.array_equal(back16.view(torch.int16).cpu().numpy().view(np.uint16), (want_back.view(np.uint32) >> 16).astype(np.uint16))
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("shape", [(1, 1, 64, 96), (2, 1, 5, 40), (1, 1, 32, 24)])
+def test_bf16_source_bit_exact(oracle, fmt, shape):
+    bits = workloads.f32_to_bf16_bits_rne(workloads.stress_mixture((1, 1, 1, -(-int(np.prod(shape)) // 16) * 16), seed=23).reshape(-1)[: int(np.prod(shape))]).reshape(shape)
+    x32 = workloads.bf16_bits_to_f32(bits)
+    want = oracle.from_torch_bfp_tiles(fmt, x32)
+    got = capi.pack_tensor(fmt, dev(bits.view(np.int16)).view(torch.bfloat16))
+    assert np.array_equal(words_np(got), want)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("row_major", [True, False])
+@pytest.mark.parametrize("n_tiles", [1, 7, 8, 19])
+def test_chunk_api_mirrors_reference_packers(oracle, fmt, row_major, n_tiles):
+    x = special_values((n_tiles * 1024,), seed=30 + n_tiles)
+    want = oracle.pack_fp32_vec_as_bfp_tiles(fmt, x, row_major)
+    got = capi.pack_chunks(fmt, dev(x), row_major)
+    assert np.array_equal(words_np(got), want)
+    want_f = oracle.unpack_bfp_tiles_into_float_vec(fmt, want, row_major)
+    got_f = capi.unpack_chunks(fmt, got, row_major)
+    assert np.array_equal(got_f.cpu().numpy().view(np.uint32), want_f.view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_unpack_foreign_codes_every_code_and_exponent(oracle, fmt):
+    """Tiles no packer would write (0x80 -> -0.0f, shift count above the exponent): every code x exponent."""
+    w = 7 if fmt == BFP8 else 3
+    n_codes = 2 << w
+    tiles = []
+    for e0 in range(0, 256, 64):
+        t = np.zeros(capi.TILE_BYTES[fmt], dtype=np.uint8)
+        t[:64] = np.arange(e0, e0 + 64, dtype=np.uint8)
+        codes = np.arange(1024) % n_codes
+        for rep in range(n_codes // 16):
+            c = (np.arange(1024) + rep * 16) % n_codes
+            tt = t.copy()
+            if fmt == BFP8:
+                tt[64:] = c.astype(np.uint8)
+            else:
+                tt[64:] = (c[0::2] | (c[1::2] << 4)).astype(np.uint8)
+            tiles.append(tt)
+        del codes
+    words = np.concatenate(tiles).view(np.uint32)
+    want = oracle.unpack_bfp_tiles_into_float_vec(fmt, words, False)
+    got = capi.unpack_chunks(fmt, dev(words.view(np.int32)), False)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_known_answers_on_gpu():
+    for case in KNOWN["edge_single_value_rows"]["cases"]:
+        row = np.zeros(1024, dtype=np.uint32)
+        row[0] = int(case["bits"], 16)
+        got = capi.pack_chunks(BFP8, dev(row.view(np.float32)), False)
+        w = words_np(got)
+        assert w[0] & 0xFF == int(case["exp"], 16) and w[16] == int(case["code"], 16), case
+        back = capi.unpack_chunks(BFP8, got, False).cpu().numpy().view(np.uint32)
+        assert back[0] == int(case["unpacked"], 16) and not back[1:].any(), case
+    k = KNOWN["arange_tile"]
+    x = np.arange(1024, dtype=np.float32)
+    w8 = words_np(capi.pack_chunks(BFP8, dev(x), True))
+    w4 = words_np(capi.pack_chunks(BFP4, dev(x), True))
+    assert w8[0] == int(k["first_exponent_word"], 16) and w8[16] == int(k["first_mantissa_word_bfp8"], 16)
+    assert w4[0] == int(k["first_exponent_word"], 16) and w4[16] == int(k["first_mantissa_word_bfp4"], 16)
+    # test_bfp8_conversion.cpp:51: row-major chunk input equals tilized input
+    tiled = capi.tilize(dev(x.reshape(1, 1, 32, 32)))
+    assert torch.equal(capi.pack_chunks(BFP8, tiled, False).cpu(), torch.from_numpy(w8.view(np.int32)))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.uint16])
+@pytest.mark.parametrize("shape", [(2, 3, 64, 96), (1, 1, 5, 40), (1, 2, 33, 65), (1, 1, 32, 1024), (1, 1, 1, 1)])
+def test_tilize_untilize_match_oracle(oracle, dtype, shape):
+    rng = np.random.default_rng(40)
+    x = rng.integers(0, 60000, size=shape).astype(dtype)
+    want = oracle.tilize_nchw_4faces(x)
+    t = dev(x.view(np.int16) if dtype == np.uint16 else x)
+    got = capi.tilize(t)
+    assert np.array_equal(got.cpu().numpy().view(dtype), want)
+    back = capi.untilize(got, shape)
+    assert np.array_equal(back.cpu().numpy().view(dtype), x)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_config_roundtrip_1k_full_size(oracle, fmt):
+    """fp32 [1,1,1024,1024] ~ N(0,1): the host round trip the reference runs on CPU, every packed byte compared."""
+    x = workloads.roundtrip_1k()
+    got = capi.pack_tensor(fmt, dev(x))
+    want = oracle.from_torch_bfp_tiles(fmt, x)
+    assert np.array_equal(words_np(got), want)
+    back = capi.unpack_tensor(fmt, got, x.shape)
+    assert np.array_equal(back.cpu().numpy().view(np.uint32), oracle.to_torch_bfp_tiles(fmt, want, x.shape).view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", [BFP4, BFP8])
+def test_config_stress_4k_full_size(oracle, fmt):
+    """fp32 [1,1,4096,4096] mixed distribution, bit exact against the oracle, plus size-independent properties."""
+    x = workloads.stress_mixture()
+    d = dev(x)
+    got = capi.pack_tensor(fmt, d)
+    want = oracle.pack_fp32_vec_as_bfp_tiles(fmt, oracle.tilize_nchw_4faces(x), False)
+    assert np.array_equal(words_np(got), want)
+    back = capi.unpack_tensor(fmt, got, x.shape)
+    # idempotence: pack(unpack(pack(x))) == pack(x); unpacked values fit bf16
+    assert torch.equal(capi.pack_tensor(fmt, back), got)
+    assert not (back.view(torch.int32) & 0xFFFF).any().item()
+    want_back = oracle.untilize_nchw_4faces(oracle.unpack_bfp_tiles_into_float_vec(fmt, want, False), x.shape)
+    assert np.array_equal(back.cpu().numpy().view(np.uint32), want_back.view(np.uint32))
+
+
+def test_strided_source_and_empty_inputs(oracle):
+    x = workloads.normal_tensor((2, 40, 80), seed=50)
+    big = np.zeros((2, 48, 96), dtype=np.float32)
+    big[:, :40, :80] = x
+    d = dev(big)
+    out = torch.empty(capi.lib().ttmi_tiled_size_bytes(BFP8, 2, 40, 80) // 4, dtype=torch.int32, device="cuda")
+    capi.check(capi.lib().ttmi_pack_rowmajor_as_bfp_tiles(BFP8, d.data_ptr(), capi.FLOAT32, 2, 40, 80, 96, 48 * 96, out.data_ptr(), None))
+    torch.cuda.synchronize()
+    assert np.array_equal(words_np(out), oracle.from_torch_bfp_tiles(BFP8, x))
+    # empty tensors are accepted and launch nothing
+    assert capi.lib().ttmi_pack_rowmajor_as_bfp_tiles(BFP8, None, capi.FLOAT32, 0, 32, 32, 32, 1024, None, None) == 0
+    assert capi.lib().ttmi_unpack_bfp_tiles_into_float_vec(BFP4, None, 0, 0, None, None) == 0

@@ -1,0 +1,180 @@
+"""GPU parity of the block-float-weight GEMM against an fp32/fp64 CPU matmul on oracle-unpacked weights.
+
+Tolerance (stated by the task): PCC >= 0.9999 and, per element,
+    |c - ref| <= 2**-8 * |ref| + 2 * K * 2**-24 * sum_k |a_k| |w_k|
+(one bf16 rounding of the output, doubled, plus the classical fp32 summation bound).
+"""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+from ttmi import capi, workloads  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+BFP8, BFP4 = capi.BFLOAT8_B, capi.BFLOAT4_B
+FMT = {"bfp8_b": BFP8, "bfp4_b": BFP4}
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def bf16_dev(bits_u16):
+    return dev(bits_u16.view(np.int16)).view(torch.bfloat16)
+
+
+def comp_pcc(golden, calculated):
+    """models/utility_functions.py:544-597 comp_pcc, for finite inputs."""
+    g = golden.astype(np.float64).reshape(-1)
+    c = calculated.astype(np.float64).reshape(-1)
+    if np.array_equal(g, c):
+        return 1.0
+    return float(np.corrcoef(g, c)[0, 1])
+
+
+def check_against_reference(c_f32, a_f32, w_f32, k, bf16_out=True, rows=None):
+    a64, w64 = a_f32.astype(np.float64), w_f32.astype(np.float64)
+    ref = np.matmul(a64, w64)
+    mag = np.matmul(np.abs(a64), np.abs(w64))
+    bound = (2.0 ** -8 if bf16_out else 2.0 ** -22) * np.abs(ref) + 2.0 * k * 2.0 ** -24 * mag + 1e-37
+    got = c_f32.astype(np.float64)
+    worst = float(np.max(np.abs(got - ref) / bound))
+    assert worst <= 1.0, f"elementwise bound exceeded by factor {worst}"
+    pcc = comp_pcc(ref, got)
+    assert pcc >= 0.9999, pcc
+    return pcc
+
+
+def pack_weights(oracle, w_f32, fmt):
+    """[..., K, N] fp32 -> (device packed words by the GPU packer, oracle-unpacked fp32 [..., K, N])."""
+    words = capi.pack_tensor(fmt, dev(w_f32))
+    want = oracle.from_torch_bfp_tiles(fmt, w_f32)
+    assert np.array_equal(words.cpu().numpy().view(np.uint32), want)
+    return words, oracle.to_torch_bfp_tiles(fmt, want, w_f32.shape)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("m,k,n", [(32, 32, 32), (32, 64, 128), (32, 160, 96), (7, 96, 160), (64, 256, 288), (45, 512, 64)])
+def test_small_shapes_row_major(oracle, fmt, m, k, n):
+    a_bits = workloads.activations_bf16(m, k, seed=60)
+    w = workloads.weights_f32(k, n, seed=61)
+    words, w_unpacked = pack_weights(oracle, w, fmt)
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n)
+    torch.cuda.synchronize()
+    check_against_reference(c.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+    c32 = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n, out_dtype=torch.float32)
+    check_against_reference(c32.cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k, bf16_out=False)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_identity_weights_return_the_activations(oracle, fmt):
+    """tests/tt_metal/tt_metal/unit_tests/.../test_matmul_single_tile_bfp8b.cpp:121-129,168: x @ I == x, exactly."""
+    m, k = 64, 96
+    a_bits = workloads.activations_bf16(m, k, seed=62)
+    words, w_unpacked = pack_weights(oracle, np.eye(k, dtype=np.float32), fmt)
+    assert np.array_equal(w_unpacked, np.eye(k, dtype=np.float32))
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, k)
+    assert np.array_equal(c.view(torch.int16).cpu().numpy().view(np.uint16)[0], a_bits)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_integer_valued_problem_is_exact(oracle, fmt):
+    """Small integers: every product and partial sum is exact in fp32, so any summation order gives the same bits."""
+    rng = np.random.default_rng(63)
+    m, k, n = 32, 288, 160
+    lim = 64 if fmt == BFP8 else 4
+    a = rng.integers(-8, 9, size=(m, k)).astype(np.float32)
+    w = rng.integers(-lim + 1, lim, size=(k, n)).astype(np.float32)
+    w[:, ::16] = lim - 1 if fmt == BFP4 else 64.0      # every face row shares one exponent, so all values are kept exactly
+    words, w_unpacked = pack_weights(oracle, w, fmt)
+    assert np.array_equal(w_unpacked, w)
+    c = capi.matmul_bfp(bf16_dev(workloads.f32_to_bf16_bits_rne(a)), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n, out_dtype=torch.float32)
+    assert np.array_equal(c.cpu().numpy()[0], a @ w)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_tile_layout_in_and_out(oracle, fmt):
+    m, k, n = 64, 128, 192
+    a_bits = workloads.activations_bf16(m, k, seed=64)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=65), fmt)
+    a_tiles = capi.tilize(bf16_dev(a_bits))
+    c_tiles = capi.matmul_bfp(a_tiles, capi.TILE, words, fmt, 1, 1, m, k, n, c_layout=capi.TILE)
+    c_rm = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n)
+    assert torch.equal(capi.untilize(c_tiles, (1, m, n)).view(torch.int16), c_rm.view(torch.int16))
+    check_against_reference(c_rm.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+
+
+@pytest.mark.parametrize("b_batch", [1, 3])
+def test_batched_and_broadcast_weights(oracle, b_batch):
+    batch, m, k, n = 3, 40, 96, 64
+    a_bits = workloads.activations_bf16(m, k, seed=66, batch=batch)
+    w = workloads.weights_f32(k, n, seed=67, batch=b_batch)
+    words, w_unpacked = pack_weights(oracle, w, BFP8)
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, batch, b_batch, m, k, n)
+    a = workloads.bf16_bits_to_f32(a_bits)
+    for b in range(batch):
+        check_against_reference(c[b].float().cpu().numpy(), a[b], w_unpacked[b if b_batch > 1 else 0], k)
+
+
+@pytest.mark.parametrize("activation", [capi.ACT_NONE, capi.ACT_RELU, capi.ACT_GELU, capi.ACT_SILU])
+def test_linear_bias_and_activation(oracle, activation):
+    """ttnn.linear golden (ttnn/ttnn/operations/matmul.py:419-438): a @ w + bias, then the activation."""
+    m, k, n = 32, 256, 128
+    a_bits = workloads.activations_bf16(m, k, seed=68)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=69), BFP8)
+    bias_bits = workloads.f32_to_bf16_bits_rne(workloads.normal_tensor((n,), seed=70))
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n, bias=bf16_dev(bias_bits),
+                        activation=activation, out_dtype=torch.float32)
+    x = torch.from_numpy(workloads.bf16_bits_to_f32(a_bits).astype(np.float64) @ w_unpacked.astype(np.float64)
+                         + workloads.bf16_bits_to_f32(bias_bits).astype(np.float64))
+    ref = {capi.ACT_NONE: lambda t: t, capi.ACT_RELU: torch.relu, capi.ACT_GELU: torch.nn.functional.gelu,
+           capi.ACT_SILU: torch.nn.functional.silu}[activation](x)
+    assert torch.allclose(c[0].cpu().double(), ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("env_split", ["1", "3"])
+def test_forced_k_split_paths_agree(oracle, env_split, monkeypatch):
+    monkeypatch.setenv("TTMI_MATMUL_KSPLIT", env_split)
+    m, k, n = 32, 1024, 160
+    a_bits = workloads.activations_bf16(m, k, seed=71)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=72), BFP8)
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    check_against_reference(c.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+
+
+@pytest.mark.parametrize("name,m,k,n,fmt,batch", workloads.DECODE_FALCON + workloads.DECODE_MISTRAL)
+def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch):
+    a_bits = workloads.activations_bf16(m, k, seed=80)
+    w = workloads.weights_f32(k, n, seed=81)
+    words = capi.pack_tensor(FMT[fmt], dev(w))
+    w_unpacked = oracle.untilize_nchw_4faces(
+        oracle.unpack_bfp_tiles_into_float_vec(FMT[fmt], words.cpu().numpy().view(np.uint32), False), (1, 1, k, n))[0, 0]
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, FMT[fmt], 1, 1, m, k, n)
+    pcc = check_against_reference(c.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+    print(name, "pcc", pcc)
+
+
+def test_prefill_shape_full_size_sampled_rows(oracle):
+    """[2048,4096] x BFP8 [4096,14336]: all rows computed on the GPU, 48 sampled rows checked in fp64."""
+    name, m, k, n, fmt, _ = workloads.PREFILL[0]
+    a_bits = workloads.activations_bf16(m, k, seed=82)
+    w = workloads.weights_f32(k, n, seed=83)
+    words = capi.pack_tensor(BFP8, dev(w))
+    w_unpacked = capi.unpack_tensor(BFP8, words, (k, n)).cpu().numpy()
+    assert np.array_equal(oracle.pack_fp32_vec_as_bfp_tiles(BFP8, oracle.tilize_nchw_4faces(w_unpacked[None, None]), False),
+                          words.cpu().numpy().view(np.uint32))
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    rows = np.random.default_rng(84).choice(m, size=48, replace=False)
+    check_against_reference(c[0][torch.from_numpy(rows).cuda()].float().cpu().numpy(),
+                            workloads.bf16_bits_to_f32(a_bits)[rows], w_unpacked, k)
+
+
+def test_bert_like_bmm_full_size(oracle):
+    name, m, k, n, fmt, batch = workloads.PREFILL[1]
+    a_bits = workloads.activations_bf16(m, k, seed=85, batch=batch)
+    w = workloads.weights_f32(k, n, seed=86, batch=batch)
+    words, w_unpacked = pack_weights(oracle, w, BFP8)
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, batch, batch, m, k, n)
+    a = workloads.bf16_bits_to_f32(a_bits)
+    for b in (0, 5, 11):
+        check_against_reference(c[b].float().cpu().numpy(), a[b], w_unpacked[b], k)

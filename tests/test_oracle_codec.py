@@ -221,3 +221,64 @@ def test_reference_tolerances_test_tensor(oracle):
     b8 = oracle.to_torch_bfp_tiles(BFP8, oracle.from_torch_bfp_tiles(BFP8, x), x.shape)
     b4 = oracle.to_torch_bfp_tiles(BFP4, oracle.from_torch_bfp_tiles(BFP4, x), x.shape)
     assert np.allclose(x, b8, atol=1e-2) and np.allclose(x, b4, atol=0.2)
+
+
+def _special_bits(n, seed):
+    rng = np.random.default_rng(seed)
+    bits = rng.integers(0, 1 << 32, size=n, dtype=np.uint64).astype(np.uint32)
+    pool = np.array([0, 0x80000000, 1, 0x80000001, 0x00400000, 0x007FFFFF, 0x00800000, 0x00FFFFFF, 0x01000000,
+                     0x01800001, 0x02000000, 0x03000000, 0x03400000, 0x7F800000, 0x7FC00000, 0x3F800000], dtype=np.uint32)
+    pick = rng.random(n) < 0.85
+    bits[pick] = pool[rng.integers(0, pool.size, size=int(pick.sum()))]
+    tiny = np.repeat(rng.random(-(-n // 16)) < 0.4, 16)[:n]      # runs whose exponent fields all stay below 8, or below 2
+    bits[tiny] &= np.repeat(np.where(rng.random(-(-n // 16)) < 0.5, 0x83FFFFFF, 0x80FFFFFF), 16).astype(np.uint32)[:n][tiny]
+    return bits
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("shape", [(1, 1, 32, 32), (1, 2, 33, 65), (1, 1, 7, 3), (2, 1, 64, 48)])
+def test_from_torch_sequence_on_tiny_exponents_follows_the_zeroing_rule(oracle, fmt, shape):
+    """Rows whose shared exponent is below the mantissa width are NOT fixed points of pack/unpack/pack.
+
+    A code whose mantissa is the single bit 2**(W-1-E) unpacks to exponent field 0 with a zero fraction (bfloat8.hpp:
+    240-249), i.e. to +-0, so the second pack of tt_eager/tensor/tensor_impl.cpp:179-197 writes code 0.  The full
+    sequence therefore equals one pass followed by that rule — which is what the fused GPU kernel implements.
+    Subnormal inputs are frequent here on purpose (zero padding makes all-tiny face rows likely)."""
+    w = W[fmt]
+    x = _special_bits(int(np.prod(shape)), 17).view(np.float32).reshape(shape)
+    full = oracle.from_torch_bfp_tiles(fmt, x)
+    single = oracle.pack_fp32_vec_as_bfp_tiles(fmt, oracle.tilize_nchw_4faces(x), False).copy()
+    wpt = 272 if fmt == BFP8 else 144
+    tiles = single.reshape(-1, wpt)
+    exps = tiles[:, :16].copy().view(np.uint8).reshape(-1, 64).astype(np.int64)          # [tile, face row]
+    per_word = 32 // (w + 1)
+    shifts = (np.arange(per_word) * (w + 1)).astype(np.uint32)
+    codes = (tiles[:, 16:, None] >> shifts) & ((2 << w) - 1)                       # [tile, word, slot]
+    codes = codes.reshape(tiles.shape[0], 64, 16)                                  # [tile, face row, column]
+    man = codes & ((1 << w) - 1)
+    lone_bit = np.where(exps < w, 1 << np.clip(w - 1 - exps, 0, 31), -1)[:, :, None]
+    changed = int(np.count_nonzero(man == lone_bit))
+    codes = np.where(man == lone_bit, 0, codes).reshape(tiles.shape[0], -1, per_word).astype(np.uint32)
+    tiles[:, 16:] = np.bitwise_or.reduce(codes << shifts, axis=2)
+    assert np.array_equal(tiles.reshape(-1), full)
+    assert changed > 0 or x.size < 1024  # the corner is actually exercised
+    # after the sequence the data IS a fixed point: a further unpack/pack changes nothing, and to_torch's own
+    # double pass equals one plain unpack
+    vals = oracle.unpack_bfp_tiles_into_float_vec(fmt, full, False)
+    assert np.array_equal(oracle.pack_fp32_vec_as_bfp_tiles(fmt, vals, False), full)
+    hp, wp = -(-shape[2] // 32) * 32, -(-shape[3] // 32) * 32
+    direct = oracle.untilize_nchw_4faces(vals, (shape[0], shape[1], hp, wp))[:, :, : shape[2], : shape[3]]
+    assert np.array_equal(oracle.to_torch_bfp_tiles(fmt, full, shape).view(np.uint32), np.ascontiguousarray(direct).view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_to_torch_sequence_on_foreign_sign_only_codes(oracle, fmt):
+    """Codes 0x80 / 0x8 (never written by a packer) unpack to -0.0f, but ttnn.to_torch's unpack -> pack -> unpack gives +0.0f."""
+    w = W[fmt]
+    words = np.zeros(272 if fmt == BFP8 else 144, dtype=np.uint32)
+    words[:16] = 0x7F7F7F7F
+    words[16] = (1 << w) | (0x41 << 8 if fmt == BFP8 else 0x5 << 4)
+    plain = oracle.unpack_bfp_tiles_into_float_vec(fmt, words, False).view(np.uint32)
+    assert plain[0] == 0x80000000
+    seq = oracle.to_torch_bfp_tiles(fmt, words, (32, 32)).view(np.uint32)
+    assert seq[0, 0] == 0 and seq[0, 1] == plain[1] and plain[1] != 0

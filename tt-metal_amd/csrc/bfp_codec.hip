@@ -1,0 +1,465 @@
+// Block-float codec kernels for gfx950: fused pad + tilize + pack, and unpack + untilize.
+//
+// Arithmetic follows tt-metal's host codecs bit for bit:
+//   shared exponent   tt_metal/common/blockfloat_common.hpp:19-47   (max raw exponent field of a 16-element face row)
+//   element -> code   tt_metal/common/bfloat8.hpp:23-87, blockfloat_common.hpp:67-147
+//   tile layout       bfloat8.hpp:102-173 (64 exponent bytes, then faces 0..3 row by row, element 0 in the low bits)
+//   code -> element   bfloat8.hpp:229-249, tt_metal/common/bfloat4.hpp:113-146
+//   tilize order      tt_metal/common/test_tiles.hpp:24-65,123-158
+//
+// Work decomposition (HBM-bound, nothing is read twice):
+//   a lane owns 16 bytes of one face row (4 fp32 or 8 bf16), LPR = 4 or 2 neighbouring lanes own the row;
+//   a wavefront covers 1 KiB of contiguous source per step, a 256-thread block covers 32 rows x TPB tiles;
+//   the row's shared exponent is a DPP quad-permute max over the LPR lanes;
+//   packed tiles are assembled in LDS and leave (or enter) the block as one contiguous run of 16-byte accesses.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ttmi_internal.h"
+
+namespace ttmi {
+
+enum SrcMode { SRC_TENSOR = 0, SRC_TILE_ROWMAJOR = 1, SRC_TILE_FACES = 2 };
+
+struct CodecShape {
+    uint32_t batch, h, w;       // logical extent (SRC_TENSOR); unused for tile-chunk modes
+    uint32_t ht, wt;            // tiles per column / row of the padded tensor
+    uint32_t col_groups;        // ceil(wt / TPB)
+    uint64_t n_tiles;           // total tiles
+    uint64_t row_stride;        // elements between rows of the row-major tensor
+    uint64_t batch_stride;      // elements between [h, w] slices
+};
+
+template <int W> struct Fmt;
+template <> struct Fmt<7> { static constexpr int tile_bytes = 1088, row_bytes = 16, face_bytes = 256; };
+template <> struct Fmt<3> { static constexpr int tile_bytes = 576, row_bytes = 8, face_bytes = 128; };
+
+// max over the 2 or 4 lanes that share a face row (lanes are aligned quads / pairs)
+template <int LPR> __device__ __forceinline__ uint32_t row_max(uint32_t v) {
+    uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, true);
+    v = v > o ? v : o;
+    if (LPR == 4) {
+        o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E /* quad_perm:[2,3,0,1] */, 0xf, 0xf, true);
+        v = v > o ? v : o;
+    }
+    return v;
+}
+
+template <int W> __device__ __forceinline__ uint32_t to_code(uint32_t bits, uint32_t shared) {
+    const uint32_t mag = bits & 0x7fffffffu;
+    const uint32_t gap = shared - (mag >> 23);
+    uint32_t m = (bits & 0x007fffffu) | 0x00800000u;   // hidden one, also for a zero exponent field
+    m = gap > 31u ? 0u : (m >> gap);                   // truncating pre-shift
+    m = (m + (1u << (23 - W))) >> (24 - W);            // round half up
+    m = m > ((1u << W) - 1u) ? ((1u << W) - 1u) : m;   // saturate, no carry into the exponent
+    const uint32_t code = m ? (((bits >> 31) << W) | m) : 0u;
+    return mag ? code : 0u;
+}
+
+template <int W> __device__ __forceinline__ uint32_t from_code(uint32_t code, uint32_t shared) {
+    const uint32_t man = code & ((1u << W) - 1u);
+    const uint32_t sign = ((code >> W) & 1u) << 31;
+    const int sc = __clz((int)man) - (32 - W);
+    const uint32_t frac = (man << (sc + 1)) & ((1u << W) - 1u);
+    const uint32_t ex = (uint32_t)((int)shared - sc);
+    const uint32_t bits = sign | (ex << 23) | (frac << (23 - W));
+    return man ? bits : sign;
+}
+
+// Which (tile-in-block, face, row-in-face, lane-in-row) a lane handles at step `it`, and where its 16 source
+// bytes live.  ELEM = bytes per source element.
+template <int ELEM> struct Item {
+    static constexpr int LPR = ELEM;               // lanes per face row: 4 (fp32) or 2 (bf16)
+    static constexpr int EPL = 16 / ELEM;          // elements per lane: 4 or 8
+    static constexpr int TPB = 32 / LPR;           // tiles per block: 8 or 16
+    int t, face, i, q;
+    __device__ __forceinline__ Item(int mode, int wave, int it, int lane) {
+        const int step = wave * 8 + it;            // 0..31: one KiB of source each
+        q = lane % LPR;
+        if (mode == SRC_TENSOR) {                  // the wave walks along one tensor row
+            const int r = step;
+            t = lane / (2 * LPR);
+            face = (r >> 4) * 2 + ((lane / LPR) & 1);
+            i = r & 15;
+        } else {                                   // the wave walks through the block's contiguous chunks
+            if (ELEM == 4) {                       // tile = 4 KiB = 4 steps
+                t = step >> 2;
+                const int part = step & 3;
+                if (mode == SRC_TILE_FACES) { face = part; i = lane >> 2; }
+                else { const int r = part * 8 + (lane >> 3); face = (r >> 4) * 2 + ((lane >> 2) & 1); i = r & 15; }
+            } else {                               // tile = 2 KiB = 2 steps
+                t = step >> 1;
+                const int part = step & 1;
+                if (mode == SRC_TILE_FACES) { face = part * 2 + (lane >> 5); i = (lane >> 1) & 15; }
+                else { const int r = part * 16 + (lane >> 2); face = (r >> 4) * 2 + ((lane >> 1) & 1); i = r & 15; }
+            }
+        }
+    }
+};
+
+template <int ELEM> __device__ __forceinline__ void expand(const uint4 raw, uint32_t (&bits)[16 / ELEM]) {
+    if (ELEM == 4) {
+        bits[0] = raw.x; bits[1] = raw.y; bits[2] = raw.z; bits[3] = raw.w;
+    } else {
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { bits[2 * k] = w[k] << 16; bits[2 * k + 1] = w[k] & 0xffff0000u; }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// pack: MODE selects how the source is addressed; ALIGNED means every lane may use one 16-byte load.
+// ---------------------------------------------------------------------------------------------------------
+template <int W, int ELEM, int MODE, bool ALIGNED>
+__global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                   const CodecShape s) {
+    using F = Fmt<W>;
+    using I = Item<ELEM>;
+    constexpr int TPB = I::TPB, EPL = I::EPL, LPR = I::LPR;
+    __shared__ __attribute__((aligned(16))) uint8_t stage[TPB * F::tile_bytes];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint64_t tile0;          // first tile of this block in the output
+    uint32_t n_valid;        // tiles of this block that exist
+    uint32_t row0 = 0, col0 = 0;
+    const uint8_t *slice = src;
+    if (MODE == SRC_TENSOR) {
+        const uint32_t cg = blockIdx.x % s.col_groups;
+        const uint64_t rest = blockIdx.x / s.col_groups;
+        const uint32_t tr = (uint32_t)(rest % s.ht);
+        const uint64_t b = rest / s.ht;
+        tile0 = (b * s.ht + tr) * s.wt + (uint64_t)cg * TPB;
+        n_valid = min((uint32_t)TPB, s.wt - cg * TPB);
+        row0 = tr * 32; col0 = cg * TPB * 32;
+        slice = src + b * s.batch_stride * ELEM;
+    } else {
+        tile0 = (uint64_t)blockIdx.x * TPB;
+        n_valid = (uint32_t)min((uint64_t)TPB, s.n_tiles - tile0);
+    }
+
+    uint4 raw[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const I at(MODE, wave, it, lane);
+        raw[it] = make_uint4(0, 0, 0, 0);
+        if (at.t >= (int)n_valid) continue;
+        if (MODE == SRC_TENSOR) {
+            const uint32_t r = row0 + (at.face >> 1) * 16 + at.i;
+            const uint32_t c = col0 + at.t * 32 + (at.face & 1) * 16 + at.q * EPL;
+            if (r >= s.h || c >= s.w) continue;
+            const uint8_t *p = slice + ((uint64_t)r * s.row_stride + c) * ELEM;
+            if (ALIGNED) {
+                raw[it] = *reinterpret_cast<const uint4 *>(p);
+            } else {
+                uint32_t tmp[4] = {0, 0, 0, 0};
+                for (int e = 0; e < EPL; ++e)
+                    if (c + e < s.w) {
+                        if (ELEM == 4) tmp[e] = reinterpret_cast<const uint32_t *>(p)[e];
+                        else tmp[e >> 1] |= (uint32_t) reinterpret_cast<const uint16_t *>(p)[e] << (16 * (e & 1));
+                    }
+                raw[it] = make_uint4(tmp[0], tmp[1], tmp[2], tmp[3]);
+            }
+        } else {
+            const uint64_t chunk = (tile0 + at.t) * 1024 * ELEM;
+            const int within = MODE == SRC_TILE_FACES ? (at.face * 256 + at.i * 16 + at.q * EPL)
+                                                      : (((at.face >> 1) * 16 + at.i) * 32 + (at.face & 1) * 16 + at.q * EPL);
+            raw[it] = *reinterpret_cast<const uint4 *>(src + chunk + (uint64_t)within * ELEM);
+        }
+    }
+
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const I at(MODE, wave, it, lane);
+        uint32_t bits[EPL];
+        expand<ELEM>(raw[it], bits);
+        uint32_t top = 0;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) { const uint32_t f = bits[e] & 0x7f800000u; top = f > top ? f : top; }
+        const uint32_t shared = row_max<LPR>(top) >> 23;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            uint32_t code = to_code<W>(bits[e], shared);
+            // from_torch runs pack -> unpack -> tilize -> pack (tt_eager/tensor/tensor_impl.cpp:179-197).  A code
+            // whose mantissa is the single bit 2^(W-1-E) unpacks to exponent field 0 with a zero fraction, i.e.
+            // to +-0, and the second pack turns that into code 0; every other code survives the round trip.
+            if (MODE == SRC_TENSOR && shared < (uint32_t)W && (code & ((1u << W) - 1u)) == (1u << ((W - 1 - shared) & 31u))) code = 0;
+            const int sh = (W + 1) * e;
+            if (sh < 32) lo |= code << sh; else hi |= code << (sh - 32);
+        }
+        if (at.t < (int)n_valid) {
+            uint8_t *tile = stage + at.t * F::tile_bytes;
+            if (at.q == 0) tile[at.face * 16 + at.i] = (uint8_t)shared;
+            uint8_t *row = tile + 64 + at.face * F::face_bytes + at.i * F::row_bytes;
+            constexpr int lane_bytes = EPL * (W + 1) / 8;          // 4, 8 (bfp8) or 2, 4 (bfp4)
+            if (lane_bytes == 2) reinterpret_cast<uint16_t *>(row)[at.q] = (uint16_t)lo;
+            else if (lane_bytes == 4) reinterpret_cast<uint32_t *>(row)[at.q] = lo;
+            else reinterpret_cast<uint2 *>(row)[at.q] = make_uint2(lo, hi);
+        }
+    }
+    __syncthreads();
+    const uint32_t n16 = n_valid * (F::tile_bytes / 16);
+    uint4 *out = reinterpret_cast<uint4 *>(dst + tile0 * F::tile_bytes);
+    const uint4 *in = reinterpret_cast<const uint4 *>(stage);
+    for (uint32_t k = threadIdx.x; k < n16; k += 256) out[k] = in[k];
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// unpack: the inverse walk.  ELEM is the destination element size (4 = fp32, 2 = bf16).
+// ---------------------------------------------------------------------------------------------------------
+template <int W, int ELEM, int MODE, bool ALIGNED>
+__global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                     const CodecShape s) {
+    using F = Fmt<W>;
+    using I = Item<ELEM>;
+    constexpr int TPB = I::TPB, EPL = I::EPL;
+    __shared__ __attribute__((aligned(16))) uint8_t stage[TPB * F::tile_bytes];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint64_t tile0;
+    uint32_t n_valid;
+    uint32_t row0 = 0, col0 = 0;
+    uint8_t *slice = dst;
+    if (MODE == SRC_TENSOR) {
+        const uint32_t cg = blockIdx.x % s.col_groups;
+        const uint64_t rest = blockIdx.x / s.col_groups;
+        const uint32_t tr = (uint32_t)(rest % s.ht);
+        const uint64_t b = rest / s.ht;
+        tile0 = (b * s.ht + tr) * s.wt + (uint64_t)cg * TPB;
+        n_valid = min((uint32_t)TPB, s.wt - cg * TPB);
+        row0 = tr * 32; col0 = cg * TPB * 32;
+        slice = dst + b * s.batch_stride * ELEM;
+    } else {
+        tile0 = (uint64_t)blockIdx.x * TPB;
+        n_valid = (uint32_t)min((uint64_t)TPB, s.n_tiles - tile0);
+    }
+    {
+        const uint32_t n16 = n_valid * (F::tile_bytes / 16);
+        const uint4 *in = reinterpret_cast<const uint4 *>(src + tile0 * F::tile_bytes);
+        uint4 *out = reinterpret_cast<uint4 *>(stage);
+        for (uint32_t k = threadIdx.x; k < n16; k += 256) out[k] = in[k];
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const I at(MODE, wave, it, lane);
+        if (at.t >= (int)n_valid) continue;
+        const uint8_t *tile = stage + at.t * F::tile_bytes;
+        const uint32_t shared = tile[at.face * 16 + at.i];
+        const uint8_t *row = tile + 64 + at.face * F::face_bytes + at.i * F::row_bytes;
+        constexpr int lane_bytes = EPL * (W + 1) / 8;
+        uint32_t lo, hi = 0;
+        if (lane_bytes == 2) lo = reinterpret_cast<const uint16_t *>(row)[at.q];
+        else if (lane_bytes == 4) lo = reinterpret_cast<const uint32_t *>(row)[at.q];
+        else { const uint2 v = reinterpret_cast<const uint2 *>(row)[at.q]; lo = v.x; hi = v.y; }
+        uint32_t bits[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const int sh = (W + 1) * e;
+            const uint32_t code = (sh < 32 ? (lo >> sh) : (hi >> (sh - 32))) & ((2u << W) - 1u);
+            bits[e] = from_code<W>(code, shared);
+            // to_torch runs unpack -> untilize -> pack -> unpack: a sign-only value (code 0x80 / 0x8, which no
+            // packer writes) is packed to code 0 on the way and comes out as +0.0f
+            if (MODE == SRC_TENSOR && (bits[e] & 0x7fffffffu) == 0) bits[e] = 0;
+        }
+        uint4 v;
+        if (ELEM == 4) v = make_uint4(bits[0], bits[1], bits[2], bits[3]);
+        else v = make_uint4((bits[0] >> 16) | (bits[1 % EPL] & 0xffff0000u), (bits[2 % EPL] >> 16) | (bits[3 % EPL] & 0xffff0000u),
+                            (bits[4 % EPL] >> 16) | (bits[5 % EPL] & 0xffff0000u), (bits[6 % EPL] >> 16) | (bits[7 % EPL] & 0xffff0000u));
+        if (MODE == SRC_TENSOR) {
+            const uint32_t r = row0 + (at.face >> 1) * 16 + at.i;
+            const uint32_t c = col0 + at.t * 32 + (at.face & 1) * 16 + at.q * EPL;
+            if (r >= s.h || c >= s.w) continue;
+            uint8_t *p = slice + ((uint64_t)r * s.row_stride + c) * ELEM;
+            if (ALIGNED) {
+                *reinterpret_cast<uint4 *>(p) = v;
+            } else {
+                for (int e = 0; e < EPL; ++e)
+                    if (c + e < s.w) {
+                        if (ELEM == 4) reinterpret_cast<uint32_t *>(p)[e] = bits[e];
+                        else reinterpret_cast<uint16_t *>(p)[e] = (uint16_t)(bits[e] >> 16);
+                    }
+            }
+        } else {
+            const uint64_t chunk = (tile0 + at.t) * 1024 * ELEM;
+            const int within = MODE == SRC_TILE_FACES ? (at.face * 256 + at.i * 16 + at.q * EPL)
+                                                      : (((at.face >> 1) * 16 + at.i) * 32 + (at.face & 1) * 16 + at.q * EPL);
+            *reinterpret_cast<uint4 *>(dst + chunk + (uint64_t)within * ELEM) = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// tilize / untilize: pure permutation with zero padding (TO_TILES) or cropping.
+// ---------------------------------------------------------------------------------------------------------
+template <int ELEM, bool TO_TILES, bool ALIGNED>
+__global__ __launch_bounds__(256) void relayout_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                       const CodecShape s) {
+    using I = Item<ELEM>;
+    constexpr int TPB = I::TPB, EPL = I::EPL;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t cg = blockIdx.x % s.col_groups;
+    const uint64_t rest = blockIdx.x / s.col_groups;
+    const uint32_t tr = (uint32_t)(rest % s.ht);
+    const uint64_t b = rest / s.ht;
+    const uint64_t tile0 = (b * s.ht + tr) * s.wt + (uint64_t)cg * TPB;
+    const uint32_t n_valid = min((uint32_t)TPB, s.wt - cg * TPB);
+    const uint8_t *rm_c = (TO_TILES ? src : dst) + b * s.batch_stride * ELEM;
+    uint8_t *tiles = const_cast<uint8_t *>(TO_TILES ? dst : src);
+
+    uint4 v[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const I at(SRC_TENSOR, wave, it, lane);
+        v[it] = make_uint4(0, 0, 0, 0);
+        if (at.t >= (int)n_valid) continue;
+        const uint32_t r = tr * 32 + (at.face >> 1) * 16 + at.i;
+        const uint32_t c = (cg * TPB + at.t) * 32 + (at.face & 1) * 16 + at.q * EPL;
+        uint8_t *tp = tiles + ((tile0 + at.t) * 1024 + at.face * 256 + at.i * 16 + at.q * EPL) * ELEM;
+        uint8_t *rp = const_cast<uint8_t *>(rm_c) + ((uint64_t)r * s.row_stride + c) * ELEM;
+        if (TO_TILES) {
+            if (r < s.h && c < s.w) {
+                if (ALIGNED) v[it] = *reinterpret_cast<const uint4 *>(rp);
+                else {
+                    uint8_t tmp[16] = {0};
+                    for (int e = 0; e < EPL * ELEM; ++e) if (c + e / ELEM < s.w) tmp[e] = rp[e];
+                    v[it] = *reinterpret_cast<uint4 *>(tmp);
+                }
+            }
+            *reinterpret_cast<uint4 *>(tp) = v[it];
+        } else {
+            if (r >= s.h || c >= s.w) continue;
+            v[it] = *reinterpret_cast<const uint4 *>(tp);
+            if (ALIGNED) *reinterpret_cast<uint4 *>(rp) = v[it];
+            else {
+                const uint8_t *tmp = reinterpret_cast<const uint8_t *>(&v[it]);
+                for (int e = 0; e < EPL * ELEM; ++e) if (c + e / ELEM < s.w) rp[e] = tmp[e];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// host launchers
+// ---------------------------------------------------------------------------------------------------------
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <int W, int ELEM, int MODE>
+static void launch_pack(bool aligned, const void *src, void *dst, const CodecShape &s, uint32_t blocks, hipStream_t st) {
+    if (aligned) hipLaunchKernelGGL((pack_kernel<W, ELEM, MODE, true>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+    else hipLaunchKernelGGL((pack_kernel<W, ELEM, MODE, false>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+}
+template <int W, int ELEM, int MODE>
+static void launch_unpack(bool aligned, const void *src, void *dst, const CodecShape &s, uint32_t blocks, hipStream_t st) {
+    if (aligned) hipLaunchKernelGGL((unpack_kernel<W, ELEM, MODE, true>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+    else hipLaunchKernelGGL((unpack_kernel<W, ELEM, MODE, false>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+}
+
+static int tensor_shape(CodecShape &s, uint32_t batch, uint32_t h, uint32_t w, size_t row_stride, size_t batch_stride,
+                        int elem, uint64_t &blocks) {
+    s.batch = batch; s.h = h; s.w = w;
+    s.ht = (h + 31) / 32; s.wt = (w + 31) / 32;
+    const uint32_t tpb = 32 / elem;
+    s.col_groups = (s.wt + tpb - 1) / tpb;
+    s.n_tiles = (uint64_t)batch * s.ht * s.wt;
+    s.row_stride = row_stride; s.batch_stride = batch_stride;
+    blocks = (uint64_t)batch * s.ht * s.col_groups;
+    if (blocks > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "tensor too large for one launch: %llu blocks", (unsigned long long)blocks);
+    return TTMI_OK;
+}
+
+int codec_pack_chunks(int fmt, const float *src, size_t n_tiles, int row_major_input, uint32_t *dst, hipStream_t st) {
+    if (n_tiles == 0) return TTMI_OK;
+    if (!aligned16(src) || !aligned16(dst)) return fail(TTMI_ERR_INVALID_ARGUMENT, "pack: src and dst must be 16-byte aligned");
+    CodecShape s{};
+    s.n_tiles = n_tiles;
+    const uint64_t blocks = (n_tiles + 7) / 8;
+    if (blocks > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "pack: too many tiles");
+    if (fmt == TTMI_BFLOAT8_B) {
+        if (row_major_input) launch_pack<7, 4, SRC_TILE_ROWMAJOR>(true, src, dst, s, (uint32_t)blocks, st);
+        else launch_pack<7, 4, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st);
+    } else {
+        if (row_major_input) launch_pack<3, 4, SRC_TILE_ROWMAJOR>(true, src, dst, s, (uint32_t)blocks, st);
+        else launch_pack<3, 4, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st);
+    }
+    return check_launch("pack_kernel");
+}
+
+int codec_unpack_chunks(int fmt, const uint32_t *words, size_t n_tiles, int row_major_output, float *dst, hipStream_t st) {
+    if (n_tiles == 0) return TTMI_OK;
+    if (!aligned16(words) || !aligned16(dst)) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpack: src and dst must be 16-byte aligned");
+    CodecShape s{};
+    s.n_tiles = n_tiles;
+    const uint64_t blocks = (n_tiles + 7) / 8;
+    if (blocks > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpack: too many tiles");
+    if (fmt == TTMI_BFLOAT8_B) {
+        if (row_major_output) launch_unpack<7, 4, SRC_TILE_ROWMAJOR>(true, words, dst, s, (uint32_t)blocks, st);
+        else launch_unpack<7, 4, SRC_TILE_FACES>(true, words, dst, s, (uint32_t)blocks, st);
+    } else {
+        if (row_major_output) launch_unpack<3, 4, SRC_TILE_ROWMAJOR>(true, words, dst, s, (uint32_t)blocks, st);
+        else launch_unpack<3, 4, SRC_TILE_FACES>(true, words, dst, s, (uint32_t)blocks, st);
+    }
+    return check_launch("unpack_kernel");
+}
+
+int codec_pack_tensor(int fmt, const void *src, int elem, uint32_t batch, uint32_t h, uint32_t w, size_t row_stride,
+                      size_t batch_stride, uint32_t *dst, hipStream_t st) {
+    if ((uint64_t)batch * h * w == 0) return TTMI_OK;
+    if (!aligned16(dst)) return fail(TTMI_ERR_INVALID_ARGUMENT, "pack: dst must be 16-byte aligned");
+    CodecShape s{};
+    uint64_t blocks;
+    if (int rc = tensor_shape(s, batch, h, w, row_stride, batch_stride, elem, blocks)) return rc;
+    const size_t per16 = 16 / elem;
+    const bool al = aligned16(src) && w % per16 == 0 && row_stride % per16 == 0 && batch_stride % per16 == 0;
+    if (fmt == TTMI_BFLOAT8_B) {
+        if (elem == 4) launch_pack<7, 4, SRC_TENSOR>(al, src, dst, s, (uint32_t)blocks, st);
+        else launch_pack<7, 2, SRC_TENSOR>(al, src, dst, s, (uint32_t)blocks, st);
+    } else {
+        if (elem == 4) launch_pack<3, 4, SRC_TENSOR>(al, src, dst, s, (uint32_t)blocks, st);
+        else launch_pack<3, 2, SRC_TENSOR>(al, src, dst, s, (uint32_t)blocks, st);
+    }
+    return check_launch("pack_kernel");
+}
+
+int codec_unpack_tensor(int fmt, const uint32_t *words, uint32_t batch, uint32_t h, uint32_t w, void *dst, int elem,
+                        hipStream_t st) {
+    if ((uint64_t)batch * h * w == 0) return TTMI_OK;
+    if (!aligned16(words)) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpack: words must be 16-byte aligned");
+    CodecShape s{};
+    uint64_t blocks;
+    if (int rc = tensor_shape(s, batch, h, w, w, (size_t)h * w, elem, blocks)) return rc;
+    const size_t per16 = 16 / elem;
+    const bool al = aligned16(dst) && w % per16 == 0;
+    if (fmt == TTMI_BFLOAT8_B) {
+        if (elem == 4) launch_unpack<7, 4, SRC_TENSOR>(al, words, dst, s, (uint32_t)blocks, st);
+        else launch_unpack<7, 2, SRC_TENSOR>(al, words, dst, s, (uint32_t)blocks, st);
+    } else {
+        if (elem == 4) launch_unpack<3, 4, SRC_TENSOR>(al, words, dst, s, (uint32_t)blocks, st);
+        else launch_unpack<3, 2, SRC_TENSOR>(al, words, dst, s, (uint32_t)blocks, st);
+    }
+    return check_launch("unpack_kernel");
+}
+
+int codec_relayout(bool to_tiles, const void *src, uint32_t elem, uint32_t batch, uint32_t h, uint32_t w, void *dst,
+                   hipStream_t st) {
+    if ((uint64_t)batch * h * w == 0) return TTMI_OK;
+    CodecShape s{};
+    uint64_t blocks;
+    if (int rc = tensor_shape(s, batch, h, w, w, (size_t)h * w, (int)elem, blocks)) return rc;
+    if (!aligned16(to_tiles ? dst : src)) return fail(TTMI_ERR_INVALID_ARGUMENT, "tilize/untilize: the tiled buffer must be 16-byte aligned");
+    const size_t per16 = 16 / elem;
+    const bool al = aligned16(to_tiles ? src : dst) && w % per16 == 0;
+#define TTMI_RELAYOUT(E, T, A) hipLaunchKernelGGL((relayout_kernel<E, T, A>), dim3((uint32_t)blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s)
+    if (elem == 4) {
+        if (to_tiles) { if (al) TTMI_RELAYOUT(4, true, true); else TTMI_RELAYOUT(4, true, false); }
+        else { if (al) TTMI_RELAYOUT(4, false, true); else TTMI_RELAYOUT(4, false, false); }
+    } else {
+        if (to_tiles) { if (al) TTMI_RELAYOUT(2, true, true); else TTMI_RELAYOUT(2, true, false); }
+        else { if (al) TTMI_RELAYOUT(2, false, true); else TTMI_RELAYOUT(2, false, false); }
+    }
+#undef TTMI_RELAYOUT
+    return check_launch("relayout_kernel");
+}
+
+}  // namespace ttmi

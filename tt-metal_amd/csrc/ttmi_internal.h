@@ -1,0 +1,37 @@
+// Internal declarations shared by the HIP translation units of libttmi.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "ttmi.h"
+
+namespace ttmi {
+
+// Records a message for ttmi_last_error() on this thread and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// hipGetLastError() after a launch -> status.
+int check_launch(const char *what);
+int check_hip(hipError_t e, const char *what);
+
+int codec_pack_chunks(int fmt, const float *src, size_t n_tiles, int row_major_input, uint32_t *dst, hipStream_t st);
+int codec_unpack_chunks(int fmt, const uint32_t *words, size_t n_tiles, int row_major_output, float *dst, hipStream_t st);
+int codec_pack_tensor(int fmt, const void *src, int elem, uint32_t batch, uint32_t h, uint32_t w, size_t row_stride,
+                      size_t batch_stride, uint32_t *dst, hipStream_t st);
+int codec_unpack_tensor(int fmt, const uint32_t *words, uint32_t batch, uint32_t h, uint32_t w, void *dst, int elem,
+                        hipStream_t st);
+int codec_relayout(bool to_tiles, const void *src, uint32_t elem, uint32_t batch, uint32_t h, uint32_t w, void *dst,
+                   hipStream_t st);
+
+struct MatmulArgs {
+    const void *a; int a_layout;
+    const uint32_t *b; int b_fmt;
+    uint32_t batch, b_batch, m, k, n;
+    const void *bias; int activation;
+    void *c; int c_layout, c_dtype;
+    void *workspace; size_t workspace_bytes;
+};
+size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
+int matmul_bfp(const MatmulArgs &args, hipStream_t st);
+
+}  // namespace ttmi

@@ -1,0 +1,189 @@
+"""ctypes view of the C ABI in ``include/ttmi.h`` plus thin helpers that pass torch device pointers.
+
+There is no CPU fallback: if ``lib/libttmi.so`` is missing or a call fails, a RuntimeError is raised.
+torch is used for device memory and streams only.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libttmi.so")
+
+BFLOAT16, FLOAT32, UINT32, BFLOAT8_B, BFLOAT4_B, UINT16 = 0, 1, 2, 3, 4, 6
+ROW_MAJOR, TILE = 0, 1
+ACT_NONE, ACT_RELU, ACT_GELU, ACT_SILU = 0, 1, 2, 3
+TILE_BYTES = {BFLOAT8_B: 1088, BFLOAT4_B: 576, BFLOAT16: 2048, UINT16: 2048, FLOAT32: 4096, UINT32: 4096}
+
+# every symbol include/ttmi.h declares
+SYMBOLS = (
+    "ttmi_last_error", "ttmi_version", "ttmi_tile_size", "ttmi_tiled_size_bytes",
+    "ttmi_pack_fp32_vec_as_bfp_tiles", "ttmi_unpack_bfp_tiles_into_float_vec",
+    "ttmi_pack_rowmajor_as_bfp_tiles", "ttmi_unpack_bfp_tiles_as_rowmajor",
+    "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
+)
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is not built: run `python tt-metal_amd/build.py` (needs hipcc); there is no CPU fallback"
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        vp, u32, i32, sz = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int, ctypes.c_size_t
+        L.ttmi_last_error.restype = ctypes.c_char_p
+        L.ttmi_last_error.argtypes = []
+        L.ttmi_version.restype = ctypes.c_char_p
+        L.ttmi_version.argtypes = []
+        L.ttmi_tile_size.restype = u32
+        L.ttmi_tile_size.argtypes = [i32]
+        L.ttmi_tiled_size_bytes.restype = sz
+        L.ttmi_tiled_size_bytes.argtypes = [i32, u32, u32, u32]
+        L.ttmi_pack_fp32_vec_as_bfp_tiles.restype = i32
+        L.ttmi_pack_fp32_vec_as_bfp_tiles.argtypes = [i32, vp, sz, i32, vp, vp]
+        L.ttmi_unpack_bfp_tiles_into_float_vec.restype = i32
+        L.ttmi_unpack_bfp_tiles_into_float_vec.argtypes = [i32, vp, sz, i32, vp, vp]
+        L.ttmi_pack_rowmajor_as_bfp_tiles.restype = i32
+        L.ttmi_pack_rowmajor_as_bfp_tiles.argtypes = [i32, vp, i32, u32, u32, u32, sz, sz, vp, vp]
+        L.ttmi_unpack_bfp_tiles_as_rowmajor.restype = i32
+        L.ttmi_unpack_bfp_tiles_as_rowmajor.argtypes = [i32, vp, u32, u32, u32, vp, i32, vp]
+        L.ttmi_tilize.restype = i32
+        L.ttmi_tilize.argtypes = [vp, u32, u32, u32, u32, vp, vp]
+        L.ttmi_untilize.restype = i32
+        L.ttmi_untilize.argtypes = [vp, u32, u32, u32, u32, vp, vp]
+        L.ttmi_matmul_bfp_workspace_bytes.restype = sz
+        L.ttmi_matmul_bfp_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
+        L.ttmi_matmul_bfp.restype = i32
+        L.ttmi_matmul_bfp.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, sz, vp]
+        _lib = L
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise RuntimeError(lib().ttmi_last_error().decode())
+
+
+def _stream():
+    import torch
+
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t):
+    if not t.is_cuda:
+        raise RuntimeError("ttmi kernels need device tensors (no CPU fallback)")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _torch_dtype_code(t):
+    import torch
+
+    if t.dtype == torch.float32:
+        return FLOAT32
+    if t.dtype == torch.bfloat16:
+        return BFLOAT16
+    raise RuntimeError(f"unsupported source dtype {t.dtype}")
+
+
+def padded(x: int) -> int:
+    return (x + 31) // 32 * 32
+
+
+# ---- torch-pointer helpers (device tensors in, device tensors out) -------------------------------------
+
+def pack_chunks(fmt: int, src, row_major_input: bool):
+    """src: cuda fp32, numel a multiple of 1024 -> cuda int32 words (mirrors pack_fp32_vec_as_bfp{8,4}_tiles)."""
+    import torch
+
+    assert src.dtype == torch.float32 and src.is_contiguous() and src.numel() % 1024 == 0
+    n_tiles = src.numel() // 1024
+    out = torch.empty(n_tiles * TILE_BYTES[fmt] // 4, dtype=torch.int32, device=src.device)
+    check(lib().ttmi_pack_fp32_vec_as_bfp_tiles(fmt, _dev(src), n_tiles, int(row_major_input), _dev(out), _stream()))
+    return out
+
+
+def unpack_chunks(fmt: int, words, row_major_output: bool):
+    import torch
+
+    assert words.dtype == torch.int32 and words.is_contiguous()
+    n_tiles = words.numel() * 4 // TILE_BYTES[fmt]
+    out = torch.empty(n_tiles * 1024, dtype=torch.float32, device=words.device)
+    check(lib().ttmi_unpack_bfp_tiles_into_float_vec(fmt, _dev(words), n_tiles, int(row_major_output), _dev(out), _stream()))
+    return out
+
+
+def _bhw(t):
+    h, w = t.shape[-2], t.shape[-1]
+    batch = 1
+    for s in t.shape[:-2]:
+        batch *= s
+    return batch, h, w
+
+
+def pack_tensor(fmt: int, src):
+    """[..., H, W] cuda fp32/bf16 (dense) -> packed words of the padded, tilized tensor."""
+    import torch
+
+    src = src.contiguous()
+    batch, h, w = _bhw(src)
+    nbytes = lib().ttmi_tiled_size_bytes(fmt, batch, h, w)
+    out = torch.empty(nbytes // 4, dtype=torch.int32, device=src.device)
+    check(lib().ttmi_pack_rowmajor_as_bfp_tiles(fmt, _dev(src), _torch_dtype_code(src), batch, h, w, w, h * w, _dev(out), _stream()))
+    return out
+
+
+def unpack_tensor(fmt: int, words, shape, dtype=None):
+    import torch
+
+    dtype = dtype or torch.float32
+    out = torch.empty(tuple(shape), dtype=dtype, device=words.device)
+    batch, h, w = _bhw(out)
+    check(lib().ttmi_unpack_bfp_tiles_as_rowmajor(fmt, _dev(words), batch, h, w, _dev(out), _torch_dtype_code(out), _stream()))
+    return out
+
+
+def tilize(src):
+    """[..., H, W] dense cuda tensor with 2- or 4-byte elements -> flat tile-order tensor of the padded shape."""
+    import torch
+
+    src = src.contiguous()
+    batch, h, w = _bhw(src)
+    out = torch.empty(batch * padded(h) * padded(w), dtype=src.dtype, device=src.device)
+    check(lib().ttmi_tilize(_dev(src), src.element_size(), batch, h, w, _dev(out), _stream()))
+    return out
+
+
+def untilize(tiles, shape):
+    import torch
+
+    out = torch.empty(tuple(shape), dtype=tiles.dtype, device=tiles.device)
+    batch, h, w = _bhw(out)
+    assert tiles.numel() == batch * padded(h) * padded(w)
+    check(lib().ttmi_untilize(_dev(tiles), tiles.element_size(), batch, h, w, _dev(out), _stream()))
+    return out
+
+
+def matmul_bfp(a, a_layout: int, b_words, b_fmt: int, batch: int, b_batch: int, m: int, k: int, n: int, *,
+               bias=None, activation: int = ACT_NONE, c_layout: int = ROW_MAJOR, out_dtype=None, workspace=None):
+    """a: cuda bf16 (dense [batch,m,k] or tile order); b_words: packed weights; returns C (dense or tile order)."""
+    import torch
+
+    out_dtype = out_dtype or torch.bfloat16
+    mp = padded(m) if c_layout == TILE else m
+    c = torch.empty(batch * mp * n, dtype=out_dtype, device=a.device)
+    ws_ptr, ws_bytes = None, 0
+    if workspace is not None:
+        ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
+    check(lib().ttmi_matmul_bfp(
+        _dev(a), a_layout, _dev(b_words), b_fmt, batch, b_batch, m, k, n,
+        _dev(bias) if bias is not None else None, activation, _dev(c), c_layout, _torch_dtype_code(c),
+        ws_ptr, ws_bytes, _stream()))
+    if c_layout == ROW_MAJOR:
+        return c.view(batch, m, n)
+    return c
