@@ -32,6 +32,9 @@ def special_values(shape, seed):
                     dtype=np.uint32)
     pick = rng.random(n) < 0.5
     bits[pick] = pool[rng.integers(0, pool.size, size=int(pick.sum()))]
+    # runs of 16 whose exponent fields all stay below 8 (or below 2): rows that are not fixed points of pack/unpack/pack
+    tiny = np.repeat(rng.random(n // 16 + 1) < 0.3, 16)[:n]
+    bits[tiny] &= np.repeat(np.where(rng.random(n // 16 + 1) < 0.5, 0x83FFFFFF, 0x80FFFFFF), 16).astype(np.uint32)[:n][tiny]
     zero_rows = rng.random(n // 16 + 1) < 0.2
     for r in np.nonzero(zero_rows)[0]:
         bits[r * 16:(r + 1) * 16] &= 0x80000000

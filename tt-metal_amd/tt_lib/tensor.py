@@ -1,0 +1,342 @@
+"""``tt_lib.tensor`` for the block-float path: DataType / Layout / StorageType, Tensor, matmul, bmm.
+
+Mirrors the pybind surface of tt_eager/tt_lib/csrc/tt_lib_bindings_tensor_pytensor.cpp:746-1300 and
+tt_lib_bindings_tensor_custom_bmm_ops.cpp:50-81.  Every conversion and the matmul run as HIP kernels behind
+the C ABI (include/ttmi.h); torch only carries memory.  Host-storage tensors keep their bytes in CPU memory
+exactly as the reference lays them out (packed uint32 words for block-float), device-storage tensors in HBM.
+"""
+from __future__ import annotations
+
+import enum
+from typing import Optional, Sequence
+
+import torch
+
+from ttmi import capi
+
+
+class DataType(enum.IntEnum):  # tt_eager/tensor/types.hpp:26-34
+    BFLOAT16 = 0
+    FLOAT32 = 1
+    UINT32 = 2
+    BFLOAT8_B = 3
+    BFLOAT4_B = 4
+    UINT16 = 6
+    INVALID = 7
+
+
+class Layout(enum.IntEnum):  # tt_eager/tensor/types.hpp:24
+    ROW_MAJOR = 0
+    TILE = 1
+    INVALID = 2
+
+
+class StorageType(enum.IntEnum):  # tt_eager/tensor/types.hpp:36-41
+    OWNED = 0
+    DEVICE = 1
+    BORROWED = 2
+    MULTI_DEVICE = 3
+
+
+class BufferType(enum.IntEnum):
+    DRAM = 0
+    L1 = 1
+
+
+class TensorMemoryLayout(enum.IntEnum):
+    INTERLEAVED = 0
+    SINGLE_BANK = 1
+    HEIGHT_SHARDED = 2
+    WIDTH_SHARDED = 3
+    BLOCK_SHARDED = 4
+
+
+class MathFidelity(enum.IntEnum):
+    LoFi = 0
+    HiFi2 = 2
+    HiFi3 = 3
+    HiFi4 = 4
+
+
+class MemoryConfig:
+    """Accepted for signature compatibility; every buffer lives in HBM."""
+
+    def __init__(self, memory_layout=TensorMemoryLayout.INTERLEAVED, buffer_type=BufferType.DRAM, shard_spec=None):
+        self.memory_layout, self.buffer_type, self.shard_spec = memory_layout, buffer_type, shard_spec
+
+    def __eq__(self, other):
+        return isinstance(other, MemoryConfig) and (self.memory_layout, self.buffer_type) == (other.memory_layout, other.buffer_type)
+
+    def __repr__(self):
+        return f"MemoryConfig({self.memory_layout.name}, {self.buffer_type.name})"
+
+
+class Device:
+    """One MI355X.  tt_lib.device.CreateDevice(id) in the reference opens a Tensix chip; here it selects a HIP device."""
+
+    def __init__(self, device_id: int = 0):
+        capi.lib()  # fail loudly when the HIP library is not built
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU visible: the block-float path has no CPU fallback")
+        self.device_id = device_id
+        self.torch_device = torch.device("cuda", device_id)
+
+    def id(self):
+        return self.device_id
+
+    def __repr__(self):
+        return f"Device(id={self.device_id}, MI355X)"
+
+
+_BFP = (DataType.BFLOAT8_B, DataType.BFLOAT4_B)
+_TORCH = {DataType.BFLOAT16: torch.bfloat16, DataType.FLOAT32: torch.float32, DataType.UINT32: torch.int32, DataType.UINT16: torch.int16}
+
+
+def _pad32(x: int) -> int:
+    return (x + 31) // 32 * 32
+
+
+def _run_on_gpu(buf: torch.Tensor, fn, device: Optional[torch.device] = None):
+    """Runs fn(cuda tensor) -> cuda tensor; host buffers are staged through the GPU and copied back."""
+    if buf.is_cuda:
+        return fn(buf)
+    capi.lib()
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU visible: block-float conversions run as HIP kernels and have no CPU fallback")
+    return fn(buf.to(device or "cuda")).cpu()
+
+
+class Tensor:
+    """Eager tensor: legacy shape (with tile padding), dtype, layout, storage.
+
+    Buffer conventions (identical to the reference's byte layout):
+      ROW_MAJOR bf16/fp32/ints   dense torch tensor of the padded shape
+      TILE      bf16/fp32/ints   flat torch tensor, 32x32 tiles of four 16x16 faces (test_tiles.hpp:24-65)
+      block-float                flat int32 words; TILE = packed tiles of the tilized tensor, ROW_MAJOR = the
+                                 row-major data packed in consecutive 1024-element chunks
+                                 (tt_lib_bindings_tensor_pytensor.cpp:145-151)
+    """
+
+    def __init__(self, data, data_type: Optional[DataType] = None, device: Optional[Device] = None,
+                 layout: Optional[Layout] = None, mem_config: Optional[MemoryConfig] = None, *, _raw=None):
+        if _raw is not None:
+            self._buf, self._shape, self._padded, self._dtype, self._layout, self._device = _raw
+            return
+        if not isinstance(data, torch.Tensor):
+            raise RuntimeError("tt_lib.tensor.Tensor: expected a torch.Tensor")
+        t = data.contiguous()
+        if data_type is None:  # pytensor.cpp:38-62
+            data_type = {torch.float32: DataType.FLOAT32, torch.float16: DataType.BFLOAT16, torch.bfloat16: DataType.BFLOAT16,
+                         torch.int16: DataType.UINT16, torch.int32: DataType.UINT32, torch.int64: DataType.UINT32}.get(t.dtype)
+            if data_type is None:
+                raise RuntimeError(f"Unsupported DataType: {t.dtype}")
+        data_type = DataType(data_type)
+        self._shape = tuple(int(s) for s in t.shape)
+        self._padded = self._shape
+        self._dtype, self._layout, self._device = data_type, Layout.ROW_MAJOR, None
+        if data_type in _BFP:  # pytensor.cpp:78-85,145-157: cast to fp32, pack sequential 1024-chunks, declare ROW_MAJOR
+            if t.numel() % 1024:
+                raise RuntimeError("TT_ASSERT: fp32_vec.size() % num_float_in_tile == 0 (block-float tensors hold whole tiles)")
+            src = t.to(torch.float32).reshape(-1)
+            self._buf = _run_on_gpu(src, lambda d: capi.pack_chunks(int(data_type), d, False))
+        else:
+            self._buf = t.to(_TORCH[data_type]).clone()
+        if layout is not None and Layout(layout) != Layout.ROW_MAJOR:
+            converted = self.to(Layout(layout))
+            self._buf, self._padded, self._layout = converted._buf, converted._padded, converted._layout
+        if device is not None:
+            self._buf, self._device = self._buf.to(device.torch_device), device
+
+    # ---- metadata -----------------------------------------------------------------------------------
+    @property
+    def shape(self):
+        import ttnn
+
+        return ttnn.Shape(self._shape, self._padded)
+
+    def get_legacy_shape(self):
+        return self.shape.with_tile_padding()
+
+    def shape_without_padding(self):
+        return self._shape
+
+    @property
+    def dtype(self):
+        return self._dtype
+
+    def get_dtype(self):
+        return self._dtype
+
+    @property
+    def layout(self):
+        return self._layout
+
+    def get_layout(self):
+        return self._layout
+
+    def storage_type(self):
+        # block-float tensors always own a copy (tests/tt_eager/.../test_tensor.py:55-57)
+        return StorageType.DEVICE if self._device is not None else StorageType.OWNED
+
+    def device(self):
+        return self._device
+
+    def is_allocated(self):
+        return self._buf is not None
+
+    def deallocate(self, force: bool = False):
+        self._buf = None
+
+    def volume(self):
+        v = 1
+        for s in self._padded:
+            v *= s
+        return v
+
+    def __repr__(self):
+        return f"Tensor(shape={self.shape}, dtype={self._dtype.name}, layout={self._layout.name}, storage={self.storage_type().name})"
+
+    def _like(self, buf, shape=None, padded=None, dtype=None, layout=None, device="keep"):
+        return Tensor(None, _raw=(buf, shape if shape is not None else self._shape, padded if padded is not None else self._padded,
+                                  dtype if dtype is not None else self._dtype, layout if layout is not None else self._layout,
+                                  self._device if device == "keep" else device))
+
+    # ---- movement -----------------------------------------------------------------------------------
+    def to(self, target, mem_config: Optional[MemoryConfig] = None):
+        if isinstance(target, Device):
+            return self._like(self._buf.to(target.torch_device), device=target)
+        target = Layout(target)
+        if target == self._layout:
+            return self
+        batch, h, w = self._bhw(self._padded)
+        dev = self._device.torch_device if self._device else None
+        if target == Layout.TILE:
+            if self._padded[-1] % 32 or (len(self._padded) > 1 and self._padded[-2] % 32):
+                raise RuntimeError("TT_ASSERT: Unsupported shape for tensor conversion (height and width must be multiples of 32)")
+            if self._dtype in _BFP:  # tensor_impl.cpp:179-197: unpack -> tilize as fp32 -> pack
+                fmt = int(self._dtype)
+                fn = lambda d: capi.pack_chunks(fmt, capi.tilize(capi.unpack_chunks(fmt, d, False).view(batch, h, w)), False)
+            else:
+                fn = lambda d: capi.tilize(d.view(batch, h, w))
+            return self._like(_run_on_gpu(self._buf, fn, dev), layout=Layout.TILE)
+        if self._dtype in _BFP:
+            fmt = int(self._dtype)
+            fn = lambda d: capi.pack_chunks(fmt, capi.untilize(capi.unpack_chunks(fmt, d, False), (batch, h, w)).reshape(-1), False)
+            return self._like(_run_on_gpu(self._buf, fn, dev), layout=Layout.ROW_MAJOR)
+        fn = lambda d: capi.untilize(d, (batch, h, w)).view(self._padded)
+        return self._like(_run_on_gpu(self._buf, fn, dev), layout=Layout.ROW_MAJOR)
+
+    def cpu(self, blocking: bool = True):
+        return self._like(self._buf.cpu(), device=None)
+
+    def reshape(self, *shape):
+        if len(shape) == 1 and not isinstance(shape[0], int):
+            shape = shape[0]
+        import ttnn
+
+        if isinstance(shape, ttnn.Shape):
+            logical, padded = tuple(shape), tuple(shape.with_tile_padding())
+        else:
+            logical = padded = tuple(int(s) for s in shape)
+        v = 1
+        for s in padded:
+            v *= s
+        if v != self.volume():
+            raise RuntimeError(f"TT_ASSERT: reshape changes the volume ({self.volume()} -> {v})")
+        buf = self._buf
+        if self._layout == Layout.ROW_MAJOR and self._dtype not in _BFP:
+            buf = buf.reshape(padded)
+        elif self._layout == Layout.TILE and (padded[-2:] != self._padded[-2:]):
+            raise RuntimeError("reshape of a TILE tensor must keep the last two padded dimensions")
+        return self._like(buf, shape=logical, padded=padded)
+
+    def to_torch(self):
+        """pytensor.cpp:354-412: block-float comes back as float32 (sequential unpack), others in their own dtype."""
+        if self._device is not None:
+            raise RuntimeError("Tensor must be on host to be converted to torch (call .cpu() first)")
+        if self._dtype in _BFP:
+            fmt = int(self._dtype)
+            return _run_on_gpu(self._buf, lambda d: capi.unpack_chunks(fmt, d, False)).view(self._padded)
+        if self._layout == Layout.TILE:
+            return self._buf.clone().view(self._padded)
+        return self._buf.clone().view(self._padded)
+
+    @staticmethod
+    def _bhw(shape):
+        shape = tuple(shape)
+        if len(shape) > 4:
+            raise RuntimeError(f"Rank {len(shape)} is not supported!")  # tensor_impl.hpp:143-155
+        h = shape[-2] if len(shape) > 1 else 1
+        w = shape[-1]
+        batch = 1
+        for s in shape[:-2]:
+            batch *= s
+        return batch, h, w
+
+
+def _matmul(a: Tensor, b: Tensor, *, bcast_batch: bool, bias: Optional[Tensor] = None, activation: int = capi.ACT_NONE,
+            output_dtype: Optional[DataType] = None, op: str = "matmul") -> Tensor:
+    """Shared body of matmul / bmm / primary.matmul (validation of bmm_op.cpp:518-539,828-1049)."""
+    for t, name in ((a, "input_tensor_a"), (b, "input_tensor_b")):
+        if t.storage_type() != StorageType.DEVICE:
+            raise RuntimeError(f"TT_FATAL: Operands to {op} need to be on device! ({name})")
+        if t.layout != Layout.TILE:
+            raise RuntimeError(f"TT_FATAL: Inputs to {op} must be tilized ({name})")
+    pa, pb = tuple(a._padded), tuple(b._padded)
+    if len(pa) < 2 or len(pb) < 2 or len(pa) > 4 or len(pb) > 4:
+        raise RuntimeError(f"TT_FATAL: {op} supports ranks 2 to 4")
+    if pa[-1] != pb[-2]:
+        raise RuntimeError("TT_FATAL: The width of the first tensor must be equal to the height of the second tensor "
+                           f"(a.shape[-1] = {pa[-1]}, b.shape[-2] = {pb[-2]})")
+    if b.dtype not in _BFP:
+        raise RuntimeError(f"{op}: this build accelerates block-float weights (BFLOAT8_B / BFLOAT4_B); got {b.dtype.name}")
+    if a.dtype not in (DataType.BFLOAT16, DataType.BFLOAT8_B, DataType.BFLOAT4_B):
+        raise RuntimeError(f"TT_FATAL: Unsupported data format for input a: {a.dtype.name}")  # bmm_op.cpp:839
+    batch_a = 1
+    for s in pa[:-2]:
+        batch_a *= s
+    batch_b = 1
+    for s in pb[:-2]:
+        batch_b *= s
+    if bcast_batch:
+        if batch_b != 1:
+            raise RuntimeError("TT_FATAL: matmul (batch bcast variant) expects input tensors of shapes BCMK*11KN=BCMN")  # bmm_op.cpp:529
+    elif batch_b != batch_a:
+        raise RuntimeError("TT_FATAL: bmm (non-bcast matmul) expects input tensors of shapes BCMK*BCKN=BCMN")  # bmm_op.cpp:533
+    m, k, n = pa[-2], pa[-1], pb[-1]
+    a_buf = a._buf
+    if a.dtype in _BFP:  # block-float activations: exact expansion to bf16 tiles in front of the GEMM
+        a_buf = capi.tilize(capi.unpack_tensor(int(a.dtype), a._buf, (batch_a, m, k), dtype=torch.bfloat16))
+    bias_buf = None
+    if bias is not None:
+        if bias.storage_type() != StorageType.DEVICE:
+            raise RuntimeError("TT_FATAL: bias must be on device")
+        if bias._padded[-1] != n:
+            raise RuntimeError("TT_FATAL: bias width must match the output width")
+        bb = bias
+        if bb.dtype in _BFP:
+            raise RuntimeError("bias must be BFLOAT16")
+        # bias is a [.., 32, N] tile row in the reference; row 0 carries the values (matmul.hpp:117-140)
+        row = capi.untilize(bb._buf, (1, bb._padded[-2] if len(bb._padded) > 1 else 1, n)) if bb.layout == Layout.TILE else bb._buf.view(-1, n)
+        bias_buf = row.reshape(-1, n)[0].contiguous().to(torch.bfloat16)
+    out_dtype = DataType(output_dtype) if output_dtype is not None else (a.dtype if a.dtype == DataType.BFLOAT16 else DataType.BFLOAT16)
+    if out_dtype != DataType.BFLOAT16:
+        raise RuntimeError(f"{op}: output dtype {out_dtype.name} is not supported yet (BFLOAT16 only)")
+    with torch.cuda.device(a._device.torch_device):
+        c = capi.matmul_bfp(a_buf, capi.TILE, b._buf, int(b.dtype), batch_a, batch_b, m, k, n, bias=bias_buf,
+                            activation=activation, c_layout=capi.TILE, out_dtype=torch.bfloat16)
+    logical = tuple(a._shape[:-1]) + (b._shape[-1],)
+    padded = pa[:-1] + (n,)
+    return Tensor(None, _raw=(c, logical, padded, DataType.BFLOAT16, Layout.TILE, a._device))
+
+
+def matmul(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None, kernel_config=None,
+           untilize_out: bool = False) -> Tensor:
+    """tt_lib.tensor.matmul: [B, C, M, K] x [1, 1, K, N] (tt_lib_bindings_tensor_custom_bmm_ops.cpp:50-65, bmm_op.hpp:388)."""
+    return _matmul(input_a, input_b, bcast_batch=True, op="matmul")
+
+
+def bmm(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None, kernel_config=None,
+        untilize_out: bool = False) -> Tensor:
+    """tt_lib.tensor.bmm: [B, C, M, K] x [B, C, K, N] (tt_lib_bindings_tensor_custom_bmm_ops.cpp:66-81, bmm_op.hpp:425)."""
+    return _matmul(input_a, input_b, bcast_batch=False, op="bmm")
