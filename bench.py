@@ -1,0 +1,273 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-float hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--legs all|primary|none]
+
+A "step" is one pass of the primary workload over one batch of synthetic input with everything resident in HBM:
+by default the Falcon-7B decode MLP (bf16 [32,4544] x BFP8_B [4544,18176], then [32,18176] x BFP8_B [18176,4544]).
+Each step uses the next of several distinct copies of the weights (footprint > 512 MiB), so the 256 MiB
+Infinity Cache cannot serve the weight stream.  One JSON line is printed; `legs` carries the other workloads
+(pack / unpack GB/s, Mistral decode GEMMs, prefill GEMM, BERT-like bmm), each with its own roofline fraction.
+
+Times come from HIP events recorded on the stream the kernels are launched on (torch's current stream).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "tt-metal_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+ROTATE_BYTES = 512 << 20
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="decode_falcon",
+                    choices=["decode_falcon", "decode_mistral", "prefill", "pack_bfp4_4k", "pack_bfp8_1k"])
+    ap.add_argument("--legs", default="all", choices=["all", "primary", "none"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from ttmi import capi, workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the block-float path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    capi.lib()
+    FMT = {"bfp8_b": capi.BFLOAT8_B, "bfp4_b": capi.BFLOAT4_B}
+
+    def dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    def bf16_dev(bits):
+        return dev(bits.view(np.int16)).view(torch.bfloat16)
+
+    def time_loop(fn, steps, warmup):
+        """fn(i) launches step i.  Returns average milliseconds per step over `steps` timed steps."""
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(steps):
+            fn(warmup + i)
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / steps
+
+    def copies_for(nbytes):
+        return max(2, -(-ROTATE_BYTES // nbytes))
+
+    def hbm_roofline(nbytes, ms):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+
+    def mfma_roofline(flops, ms):
+        tf = flops / (ms * 1e-3) / 1e12
+        return {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}
+
+    # ------------------------------------------------------------------------------------------------
+    # GEMM workloads
+    # ------------------------------------------------------------------------------------------------
+    def gemm_leg(spec, steps, warmup, seed):
+        name, m, k, n, fmt, batch = spec
+        b = batch or 1
+        w = workloads.weights_f32(k, n, seed, batch=batch)
+        words = capi.pack_tensor(FMT[fmt], dev(w))
+        del w
+        a_shape_batch = batch
+        a = bf16_dev(workloads.activations_bf16(m, k, seed + 1, batch=a_shape_batch))
+        nbytes = workloads.gemm_bytes(m, k, n, fmt, batch)
+        flops = workloads.gemm_flops(m, k, n, batch)
+        hbm_bound = m <= 64
+        ncopies = copies_for(words.numel() * 4) if hbm_bound else 2
+        wcopies = [words] + [words.clone() for _ in range(ncopies - 1)]
+        acopies = [a] + [a.clone() for _ in range(ncopies - 1)]
+        # pre-built argument lists: the timed loop is nothing but C-ABI calls on torch's current stream
+        L = capi.lib()
+        stream = torch.cuda.current_stream().cuda_stream
+        c = torch.empty((b, m, n), dtype=torch.bfloat16, device="cuda")
+        calls = [(acopies[j].data_ptr(), capi.ROW_MAJOR, wcopies[j].data_ptr(), FMT[fmt], b, b, m, k, n, None, capi.ACT_NONE,
+                  c.data_ptr(), capi.ROW_MAJOR, capi.BFLOAT16, None, 0, stream) for j in range(ncopies)]
+
+        def run(i):
+            capi.check(L.ttmi_matmul_bfp(*calls[i % ncopies]))
+
+        ms = time_loop(run, steps, warmup)
+        roof = hbm_roofline(nbytes, ms) if hbm_bound else mfma_roofline(flops, ms)
+        leg = {"workload": name, "shape": [b, m, k, n], "weights": fmt, "ms": round(ms, 5),
+               "tflops": round(flops / (ms * 1e-3) / 1e12, 2), "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1),
+               "algorithmic_bytes": nbytes, "flops": flops, "weight_copies_rotated": ncopies, "roofline": roof}
+        return leg, (wcopies, acopies, FMT[fmt], b, m, k, n)
+
+    def codec_leg(name, x_np, fmt, steps, warmup):
+        x = dev(x_np)
+        nbytes_in = x.numel() * 4
+        words = capi.pack_tensor(fmt, x)
+        nbytes = nbytes_in + words.numel() * 4
+        ncopies = copies_for(nbytes_in)
+        xs = [x] + [x.clone() for _ in range(ncopies - 1)]
+        ws = [words] + [words.clone() for _ in range(ncopies - 1)]
+        L = capi.lib()
+        stream = torch.cuda.current_stream().cuda_stream
+        batch, h, w = capi._bhw(x)
+        out_words = torch.empty_like(words)
+        out_x = torch.empty_like(x)
+        pack_calls = [(fmt, t.data_ptr(), capi.FLOAT32, batch, h, w, w, h * w, out_words.data_ptr(), stream) for t in xs]
+        unpack_calls = [(fmt, t.data_ptr(), batch, h, w, out_x.data_ptr(), capi.FLOAT32, stream) for t in ws]
+
+        ms_p = time_loop(lambda i: capi.check(L.ttmi_pack_rowmajor_as_bfp_tiles(*pack_calls[i % ncopies])), steps, warmup)
+        ms_u = time_loop(lambda i: capi.check(L.ttmi_unpack_bfp_tiles_as_rowmajor(*unpack_calls[i % ncopies])), steps, warmup)
+        # same loop on one buffer: the working set sits in the Infinity Cache ("hot")
+        ms_p_hot = time_loop(lambda i: capi.check(L.ttmi_pack_rowmajor_as_bfp_tiles(*pack_calls[0])), steps, warmup)
+        legs = []
+        for op, ms, hot in (("pack", ms_p, ms_p_hot), ("unpack", ms_u, None)):
+            leg = {"workload": f"{name}_{op}", "shape": list(x.shape), "ms": round(ms, 5), "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                   "algorithmic_bytes": nbytes, "buffers_rotated": ncopies, "roofline": hbm_roofline(nbytes, ms)}
+            if hot is not None:
+                leg["gbs_cache_resident"] = round(nbytes / (hot * 1e-3) / 1e9, 1)
+            legs.append(leg)
+        return legs
+
+    t0 = time.time()
+    legs = []
+    primary = None
+    primary_state = None
+    steps, warmup = args.steps, args.warmup
+
+    def note(msg):
+        print(f"[bench {time.time() - t0:6.1f}s] {msg}", file=sys.stderr, flush=True)
+
+    gemm_sets = {"decode_falcon": workloads.DECODE_FALCON, "decode_mistral": workloads.DECODE_MISTRAL, "prefill": workloads.PREFILL}
+    order = [args.workload] + ([w for w in ("decode_falcon", "decode_mistral", "prefill", "pack_bfp4_4k", "pack_bfp8_1k")
+                               if w != args.workload] if args.legs == "all" else [])
+    results = {}
+    for wl in order:
+        note(f"workload {wl}")
+        sub_steps = steps if wl == args.workload else max(10, min(steps, 30))
+        if wl in gemm_sets:
+            sub = []
+            for idx, spec in enumerate(gemm_sets[wl]):
+                big = spec[1] > 64
+                leg, state = gemm_leg(spec, max(5, sub_steps // 5) if big else sub_steps, 2 if big else warmup, 1234 + 10 * idx)
+                sub.append(leg)
+                if wl == args.workload and idx == 0:
+                    primary_state = state
+                else:
+                    del state
+                torch.cuda.empty_cache()
+            results[wl] = sub
+        else:
+            fmt = capi.BFLOAT4_B if wl == "pack_bfp4_4k" else capi.BFLOAT8_B
+            x = workloads.stress_mixture() if wl == "pack_bfp4_4k" else workloads.roundtrip_1k()
+            results[wl] = codec_leg(wl, x, fmt, sub_steps, warmup)
+            torch.cuda.empty_cache()
+
+    prim = results[args.workload]
+    total_ms = sum(l["ms"] for l in prim)
+    if args.workload in gemm_sets:
+        total_flops = sum(l["flops"] for l in prim)
+        value, unit = total_flops / (total_ms * 1e-3) / 1e12, "TFLOP/s"
+        metric = "bfp_weight_matmul_tflops"
+        dtype = "bf16"
+    else:
+        total_bytes = sum(l["algorithmic_bytes"] for l in prim)
+        value, unit = total_bytes / (total_ms * 1e-3) / 1e9, "GB/s"
+        metric = "bfp_pack_unpack_gbs"
+        dtype = "u32"
+    dominant = max(prim, key=lambda l: l["ms"])
+
+    # ------------------------------------------------------------------------------------------------
+    # CPU baseline: the oracle (a port of the reference's host path) timed on this host, bounded sample
+    # ------------------------------------------------------------------------------------------------
+    cpu = None
+    if not args.no_cpu_baseline:
+        note("cpu baseline")
+        from oracle import bfp_oracle as oracle
+
+        oracle.build()
+        if args.workload in gemm_sets:
+            name, m, k, n, fmt, batch = gemm_sets[args.workload][0]
+            n_s = min(n, 2048)
+            w = workloads.weights_f32(k, n_s, 999)
+            t = time.time()
+            words = oracle.from_torch_bfp_tiles(FMT[fmt], w)
+            t_pack = time.time() - t
+            t = time.time()
+            w_un = oracle.to_torch_bfp_tiles(FMT[fmt], words, (k, n_s))
+            t_unpack = time.time() - t
+            a = torch.from_numpy(workloads.bf16_bits_to_f32(workloads.activations_bf16(m, k, 998)))
+            wt = torch.from_numpy(w_un)
+            threads = torch.get_num_threads()
+            torch.matmul(a, wt)
+            reps, t = 0, time.time()
+            while time.time() - t < 8.0:
+                torch.matmul(a, wt)
+                reps += 1
+            t_mm = (time.time() - t) / reps
+            # single-thread gold loop (tests/tt_metal/tt_metal/test_gold_impls.hpp:237-290) on a slice
+            n_g = 256
+            t = time.time()
+            oracle.gold_bmm(oracle.bf16_truncate(a.numpy()), oracle.bf16_truncate(w_un[:, :n_g]), 1, m, k, n_g)
+            t_gold = time.time() - t
+            cpu = {"value": round(2.0 * m * k * n_s / t_mm / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                   "sample": f"torch.matmul fp32 [{m},{k}]x[{k},{n_s}] on oracle-unpacked {fmt} weights ({n_s} of {n} columns, {reps} reps); "
+                             f"oracle from_torch sequence on that slice, 1 thread",
+                   "gold_bmm_1thread_tflops": round(2.0 * m * k * n_g / t_gold / 1e12, 5),
+                   "from_torch_pack_melem_s_1thread": round(k * n_s / t_pack / 1e6, 1),
+                   "to_torch_unpack_melem_s_1thread": round(k * n_s / t_unpack / 1e6, 1)}
+        else:
+            fmt = capi.BFLOAT4_B if args.workload == "pack_bfp4_4k" else capi.BFLOAT8_B
+            x = (workloads.stress_mixture((1, 1, 2048, 4096)) if args.workload == "pack_bfp4_4k" else workloads.roundtrip_1k())
+            t = time.time()
+            words = oracle.from_torch_bfp_tiles(fmt, x)
+            t_pack = time.time() - t
+            t = time.time()
+            oracle.to_torch_bfp_tiles(fmt, words, x.shape)
+            t_unpack = time.time() - t
+            nb = x.size * 4 + words.size * 4
+            cpu = {"value": round(2 * nb / (t_pack + t_unpack) / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                   "sample": f"oracle from_torch + to_torch host sequences on fp32 {list(x.shape)}",
+                   "from_torch_pack_melem_s_1thread": round(x.size / t_pack / 1e6, 1),
+                   "to_torch_unpack_melem_s_1thread": round(x.size / t_unpack / 1e6, 1)}
+
+    line = {
+        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(total_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic",
+        "config": {"workload": args.workload, "parts": [l["workload"] for l in prim],
+                   "note": "weights rotate over distinct copies (>512 MiB) so the Infinity Cache cannot serve them"},
+        "roofline": dict(dominant["roofline"], kernel=dominant["workload"]),
+        "cpu_baseline": cpu,
+        "legs": [l for wl in order for l in results[wl]],
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -132,14 +132,31 @@ def test_linear_bias_and_activation(oracle, activation):
     assert torch.allclose(c[0].cpu().double(), ref, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("env_split", ["1", "3"])
-def test_forced_k_split_paths_agree(oracle, env_split, monkeypatch):
-    monkeypatch.setenv("TTMI_MATMUL_KSPLIT", env_split)
-    m, k, n = 32, 1024, 160
+@pytest.mark.parametrize("workgroups", ["1", "3", "7", "64", "4096"])
+def test_any_number_of_workgroups_gives_the_same_bits(oracle, workgroups, monkeypatch):
+    """The k range of an output may be shared between workgroups in any way; partial sums are added in a fixed order."""
+    m, k, n = 40, 1024, 288
     a_bits = workloads.activations_bf16(m, k, seed=71)
     words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=72), BFP8)
+    monkeypatch.setenv("TTMI_MATMUL_WGS", workgroups)
     c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    again = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    assert torch.equal(c.view(torch.int16), again.view(torch.int16))
     check_against_reference(c.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+
+
+def test_caller_workspace(oracle):
+    m, k, n = 32, 2048, 256
+    a_bits = workloads.activations_bf16(m, k, seed=73)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=74), BFP4)
+    need = capi.lib().ttmi_matmul_bfp_workspace_bytes(1, m, k, n, BFP4)
+    assert need > 0
+    ws = torch.full((need,), 0x5A, dtype=torch.uint8, device="cuda")   # dirty on purpose
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP4, 1, 1, m, k, n, workspace=ws)
+    check_against_reference(c.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+    small = torch.empty(need - 256, dtype=torch.uint8, device="cuda")
+    with pytest.raises(RuntimeError, match="workspace"):
+        capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP4, 1, 1, m, k, n, workspace=small)
 
 
 @pytest.mark.parametrize("name,m,k,n,fmt,batch", workloads.DECODE_FALCON + workloads.DECODE_MISTRAL)

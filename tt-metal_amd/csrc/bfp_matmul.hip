@@ -20,21 +20,27 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "ttmi_internal.h"
 
 namespace ttmi {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // first-class 16-byte value: stays in registers
 
 struct MatmulDev {
     const uint8_t *a;        // bf16
     const uint8_t *b;        // packed tiles
     const uint16_t *bias;    // bf16 [n] or null
     uint8_t *c;              // output (bf16 or fp32)
-    float *partial;          // [ksplit][batch*m][n] when ksplit > 1
+    float *slots;            // 2 slots of 32x128 fp32 per workgroup, for outputs shared between workgroups
+    uint32_t *counters;      // one arrival counter per output group (all zero between launches)
     uint32_t batch, b_batch, m, k, n;
-    uint32_t mt, kt, nt, ngroups, ksplit, kt_per_split;
+    uint32_t mt, kt, nt, ngroups;
+    uint32_t workgroups;     // P
+    uint64_t units;          // U = batch * mt * ngroups * kt
     int a_tiled, c_tiled, c_f32, activation;
 };
 
@@ -55,7 +61,9 @@ constexpr int WAVES = 4;
 constexpr int EXP_AREA = GROUP_TILES * 64;           // exponent bytes of the 4 staged tiles
 constexpr int REDUCE_BYTES = WAVES * 48 * 64 * 4;    // 48 fp32 per lane handed over per wavefront
 
-template <int W> constexpr int stage_bytes() { return EXP_AREA + GROUP_TILES * Wfmt<W>::tile_stride; }
+// exponent area + padded mantissa area + a 64-byte dump slot for lanes with nothing to park
+template <int W> constexpr int stage_data_bytes() { return EXP_AREA + GROUP_TILES * Wfmt<W>::tile_stride; }
+template <int W> constexpr int stage_bytes() { return stage_data_bytes<W>() + 64; }
 
 __device__ __forceinline__ float apply_activation(float x, int act) {
     switch (act) {
@@ -73,232 +81,343 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
 }
 
 // Eight weights of one output column, k rows 8g..8g+7, as the bf16 B operand of one MFMA.
-//   words[jj]  mantissa word of k row 8g+jj that contains this column's code
-//   scale[jj]  2^(E - bias_exp) of that row
-//   sel        which code inside the word (byte 0..3 for W=7, nibble 0..7 for W=3)
-template <int W>
-__device__ __forceinline__ bf16x8 weights_operand(const uint32_t (&words)[8], const float (&scale)[8], int sel) {
+//   words[jj]  mantissa word of k row 8g+jj that contains this column's code (W=3: already shifted so that the
+//              codes of interest sit in the low 16 bits)
+//   mags[jj]   the same word with the sign bits cleared and, for W=3, split so every code sits alone in a byte
+//   ex[jj]     E - bias_exp of that row
+//   SEL        which code inside the word (byte 0..3)
+// Per pair of rows: 2 x v_cvt_f32_ubyteN, 2 x v_ldexp_f32, v_perm_b32 (keep the upper halves = exact bf16),
+// v_perm_b32 (fetch the two sign bytes) and v_and_or_b32.
+// v_cvt_f32_ubyteN: byte N of a word as float, one instruction (the compiler otherwise extracts the field first)
+template <int SEL> __device__ __forceinline__ float byte_to_float(uint32_t word) {
+    float r;
+    if (SEL == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(word));
+    else if (SEL == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(word));
+    else if (SEL == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(word));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(word));
+    return r;
+}
+
+template <int SEL>
+__device__ __forceinline__ bf16x8 weights_operand8(const uint32_t (&words)[8], const uint32_t (&mags)[8], const float (&scale)[8]) {
     uint32_t packed[4];
+    constexpr uint32_t sign_sel = ((4u + SEL) << 24) | (0x0cu << 16) | ((uint32_t)SEL << 8) | 0x0cu;
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-        uint32_t half[2];
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const uint32_t code = words[2 * p + s] >> ((W + 1) * sel);
-            const float mag = (float)(code & ((1u << W) - 1u)) * scale[2 * p + s];
-            half[s] = (__float_as_uint(mag) >> 16) | (((code >> W) & 1u) << 15);
-        }
-        packed[p] = half[0] | (half[1] << 16);
+        const uint32_t v0 = __float_as_uint(byte_to_float<SEL>(mags[2 * p]) * scale[2 * p]);
+        const uint32_t v1 = __float_as_uint(byte_to_float<SEL>(mags[2 * p + 1]) * scale[2 * p + 1]);
+        const uint32_t both = __builtin_amdgcn_perm(v1, v0, 0x07060302u);
+        const uint32_t signs = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], sign_sel);
+        packed[p] = (signs & 0x80008000u) | both;
     }
     return __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
 }
 
+// Partial sums that other workgroups read travel through device-coherent accesses: relaxed atomic stores and loads
+// at agent scope go past the per-XCD L2 (which is not coherent across XCDs), so no cache write-back or invalidate
+// is needed — a full agent-scope fence here costs more than the whole GEMM.
+__device__ __forceinline__ void slot_store(float4 *to, const float4 v) {
+    uint64_t *q = reinterpret_cast<uint64_t *>(to);
+    __hip_atomic_store(q, ((uint64_t)__float_as_uint(v.y) << 32) | __float_as_uint(v.x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(q + 1, ((uint64_t)__float_as_uint(v.w) << 32) | __float_as_uint(v.z), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float4 slot_load(const float4 *from) {
+    uint64_t *q = reinterpret_cast<uint64_t *>(const_cast<float4 *>(from));
+    const uint64_t lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return make_float4(__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)), __uint_as_float((uint32_t)hi),
+                       __uint_as_float((uint32_t)(hi >> 32)));
+}
+
+// First unit of workgroup i when U units are dealt out evenly and contiguously to P workgroups.
+__host__ __device__ __forceinline__ uint64_t range_start(uint64_t units, uint32_t workgroups, uint32_t i) {
+    return units * i / workgroups;
+}
+
+// Work decomposition ("stream-K"): a unit is (output group, k-tile), an output group being one 32-row band of
+// one batch slice times 128 columns; units are numbered with the k-tile fastest and dealt out contiguously and
+// evenly to P workgroups (P = what the chip holds at once), so every workgroup streams the same number of
+// packed bytes whatever K, N and P are.  A workgroup whose range covers all k-tiles of an output group stores
+// that output directly.  Otherwise it writes its fp32 partial sums to a slot of its own and bumps the group's
+// arrival counter; the workgroup that arrives last adds the slots in workgroup order (so the result does not
+// depend on who was last), applies the epilogue, stores, and resets the counter.
 template <int W>
 __global__ __launch_bounds__(256) void matmul_stream_kernel(const MatmulDev p) {
     using F = Wfmt<W>;
     constexpr int STAGE = stage_bytes<W>();
+    constexpr uint32_t STAGE_DATA = stage_data_bytes<W>();
     constexpr int LDS_BYTES = REDUCE_BYTES > WAVES * STAGE ? REDUCE_BYTES : WAVES * STAGE;
     constexpr int NLOAD = (GROUP_TILES * F::chunks + 63) / 64;
     __shared__ __attribute__((aligned(16))) uint8_t lds[LDS_BYTES];
+    __shared__ uint32_t arrival;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 31, g = lane >> 5;
     const int t_of_lane = c >> 3, fc = (c >> 2) & 1, q = c & 3;
 
-    uint32_t idx = blockIdx.x;
-    const uint32_t ks = idx % p.ksplit; idx /= p.ksplit;
-    const uint32_t ng = idx % p.ngroups; idx /= p.ngroups;
-    const uint32_t mt = idx % p.mt;
-    const uint32_t bb = idx / p.mt;
-    const uint32_t nt0 = ng * GROUP_TILES;
-    const uint32_t n_valid = min((uint32_t)GROUP_TILES, p.nt - nt0);
-    const uint32_t kt_begin = ks * p.kt_per_split;
-    const uint32_t kt_end = min(p.kt, kt_begin + p.kt_per_split);
-
-    const uint8_t *wbase = p.b + (uint64_t)(p.b_batch == 1 ? 0 : bb) * p.kt * p.nt * F::tile_bytes;
-    uint8_t *my_stage = lds + wave * STAGE;
-    uint8_t *my_mant = my_stage + EXP_AREA;
+    // ---- addressing that does not depend on the segment ---------------------------------------------------
+    // The 4 adjacent tiles of a k-tile are one contiguous run of GROUP_TILES*chunks 16-byte chunks.  Load l of a
+    // lane takes chunk l*64+lane and parks it at a fixed LDS address; lanes with nothing to park in the last
+    // round write to a dump slot behind the stage.
+    uint32_t chunk_of[NLOAD], dst_off[NLOAD];
+#pragma unroll
+    for (int l = 0; l < NLOAD; ++l) {
+        const uint32_t gch = l * 64 + lane;
+        chunk_of[l] = gch;
+        const uint32_t t = gch / F::chunks, r = gch % F::chunks;
+        if (gch >= (uint32_t)(GROUP_TILES * F::chunks)) dst_off[l] = STAGE_DATA + (lane & 3) * 16;
+        else if (r < 4) dst_off[l] = t * 64 + r * 16;
+        else {
+            const uint32_t rr = r - 4, per_face = 16 / F::rows_per_chunk;
+            dst_off[l] = EXP_AREA + t * F::tile_stride + (rr / per_face) * F::face_stride + (rr % per_face) * 16;
+        }
+        dst_off[l] += wave * STAGE;
+    }
+    // per-lane LDS offsets of the two 16-row halves (offsets, not pointers, so the accesses stay LDS instructions)
+    uint32_t exp_off[2], mant_off[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int face = 2 * h + fc;
+        exp_off[h] = wave * STAGE + t_of_lane * 64 + face * 16 + g * 8;
+        mant_off[h] = wave * STAGE + EXP_AREA + t_of_lane * F::tile_stride + face * F::face_stride + (g * 8) * F::row_bytes +
+                      (W == 7 ? q * 4 : (q >> 1) * 4);
+    }
+    const uint64_t w_step = (uint64_t)WAVES * p.nt * F::tile_bytes;      // bytes between the k-tiles of one wavefront
+    const uint32_t a_half = p.a_tiled ? 512 : 32, a_step = p.a_tiled ? WAVES * 2048 : WAVES * 64;
 
     f32x16 acc[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+    u32x4 inflight[NLOAD], a_next[2];
+    uint32_t src_off[NLOAD];
+    const uint8_t *wptr, *aptr;
 
-    const uint32_t chunks_valid = n_valid * F::chunks;
-    uint4 inflight[NLOAD];
-    auto fetch = [&](uint32_t kt) {
-        const uint4 *src = reinterpret_cast<const uint4 *>(wbase + ((uint64_t)kt * p.nt + nt0) * F::tile_bytes);
+    auto fetch = [&]() {
+#if defined(TTMI_PROBE) && TTMI_PROBE >= 3
+        a_next[0] = (uint32_t)(uintptr_t)aptr; a_next[1] = a_next[0] + 1u;
+#else
+        a_next[0] = *reinterpret_cast<const u32x4 *>(aptr);
+        a_next[1] = *reinterpret_cast<const u32x4 *>(aptr + a_half);
+#endif
 #pragma unroll
-        for (int l = 0; l < NLOAD; ++l) {
-            const uint32_t gch = l * 64 + lane;
-            inflight[l] = gch < chunks_valid ? src[gch] : make_uint4(0, 0, 0, 0);
-        }
+#if defined(TTMI_PROBE) && (TTMI_PROBE == 2 || TTMI_PROBE == 3)
+        for (int l = 0; l < NLOAD; ++l) inflight[l] = a_next[0] + (uint32_t)l;
+#else
+        for (int l = 0; l < NLOAD; ++l) inflight[l] = *reinterpret_cast<const u32x4 *>(wptr + src_off[l]);
+#endif
+        aptr += a_step;
+        wptr += w_step;
     };
     auto stash = [&]() {
 #pragma unroll
-        for (int l = 0; l < NLOAD; ++l) {
-            const uint32_t gch = l * 64 + lane;
-            if (gch >= GROUP_TILES * F::chunks) continue;
-            const uint32_t t = gch / F::chunks, r = gch % F::chunks;
-            uint8_t *to;
-            if (r < 4) to = my_stage + t * 64 + r * 16;
-            else {
-                const uint32_t rr = r - 4;                       // 16-byte chunk inside the mantissa area
-                const uint32_t per_face = 16 / F::rows_per_chunk;
-                to = my_mant + t * F::tile_stride + (rr / per_face) * F::face_stride + (rr % per_face) * 16;
-            }
-            *reinterpret_cast<uint4 *>(to) = inflight[l];
+        for (int l = 0; l < NLOAD; ++l) *reinterpret_cast<u32x4 *>(lds + dst_off[l]) = inflight[l];
+    };
+    auto half_step = [&](const u32x4 a_regs, int h) {
+#if defined(TTMI_PROBE) && (TTMI_PROBE == 1 || TTMI_PROBE == 4)
+        acc[0][0] += __uint_as_float(a_regs.x + lds[exp_off[h]]); return;
+#endif
+        const bf16x8 aop = __builtin_bit_cast(bf16x8, a_regs);
+        // scale of row jj = 2^(E - bias_exp).  Writing the exponent field directly needs E - bias_exp + 127 >= 1;
+        // a wavefront that meets a smaller exponent (magnitudes below ~2^-120) takes v_ldexp_f32 instead.
+        uint32_t e[8];
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) e[jj] = lds[exp_off[h] + jj];
+        const uint32_t e_min = min(min(min(e[0], e[1]), min(e[2], e[3])), min(min(e[4], e[5]), min(e[6], e[7])));
+        float scale[8];
+        if (__builtin_expect(__ballot(e_min < (uint32_t)(F::bias_exp - 126)) != 0, 0)) {
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) scale[jj] = __builtin_amdgcn_ldexpf(1.0f, (int)e[jj] - F::bias_exp);
+        } else {
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float((e[jj] << 23) - ((uint32_t)(F::bias_exp - 127) << 23));
         }
+        uint32_t words[8], mags[8];
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+            if (W == 7) {
+                words[jj] = *reinterpret_cast<const uint32_t *>(lds + mant_off[h] + jj * 16);
+                mags[jj] = words[jj] & 0x7f7f7f7fu;
+            } else {
+                // four 4-bit codes -> one code per byte; sign bit moved from bit 3 to bit 7 of its byte
+                uint32_t v = (*reinterpret_cast<const uint32_t *>(lds + mant_off[h] + jj * 8) >> (16 * (q & 1))) & 0xffffu;
+                v = (v | (v << 8)) & 0x00ff00ffu;
+                v = (v | (v << 4)) & 0x0f0f0f0fu;
+                words[jj] = v << 4;
+                mags[jj] = v & 0x07070707u;
+            }
+        }
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aop, weights_operand8<0>(words, mags, scale), acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aop, weights_operand8<1>(words, mags, scale), acc[1], 0, 0, 0);
+        acc[2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aop, weights_operand8<2>(words, mags, scale), acc[2], 0, 0, 0);
+        acc[3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aop, weights_operand8<3>(words, mags, scale), acc[3], 0, 0, 0);
     };
 
-    const uint32_t m_row = mt * 32 + c;       // activation row this lane feeds to the MFMA
-    uint32_t kt = kt_begin + wave;
-    if (kt < kt_end) fetch(kt);
-    for (; kt < kt_end; kt += WAVES) {
-        stash();
-        if (kt + WAVES < kt_end) fetch(kt + WAVES);
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            // activations: rows m, k = kt*32 + h*16 + g*8 .. +7
-            uint4 araw = make_uint4(0, 0, 0, 0);
-            if (p.a_tiled) {
-                const uint8_t *at = p.a + (((uint64_t)bb * p.mt + mt) * p.kt + kt) * 2048 + ((c >> 4) * 2 + h) * 512 +
-                                    (c & 15) * 32 + g * 16;
-                araw = *reinterpret_cast<const uint4 *>(at);
-            } else if (m_row < p.m) {
-                const uint8_t *at = p.a + (((uint64_t)bb * p.m + m_row) * p.k + kt * 32 + h * 16 + g * 8) * 2;
-                araw = *reinterpret_cast<const uint4 *>(at);
-            }
-            const bf16x8 aop = __builtin_bit_cast(bf16x8, araw);
+#if defined(TTMI_PROBE) && TTMI_PROBE == 5
+    if (p.units) return;
+#endif
+    const uint32_t me = blockIdx.x;
+    uint64_t unit = range_start(p.units, p.workgroups, me);
+    const uint64_t unit_end = range_start(p.units, p.workgroups, me + 1);
+    const uint64_t my_first_og = unit / p.kt;
 
-            const int face = 2 * h + fc;
-            const uint2 e2 = *reinterpret_cast<const uint2 *>(my_stage + t_of_lane * 64 + face * 16 + g * 8);
-            float scale[8];
-#pragma unroll
-            for (int jj = 0; jj < 8; ++jj) {
-                const uint32_t e = ((jj < 4 ? e2.x : e2.y) >> (8 * (jj & 3))) & 0xffu;
-                scale[jj] = ldexpf(1.0f, (int)e - F::bias_exp);
-            }
-            uint32_t words[8];
-            const uint8_t *rows = my_mant + t_of_lane * F::tile_stride + face * F::face_stride + (g * 8) * F::row_bytes;
-#pragma unroll
-            for (int jj = 0; jj < 8; ++jj) {
-                if (W == 7) words[jj] = *reinterpret_cast<const uint32_t *>(rows + jj * 16 + q * 4);
-                else words[jj] = *reinterpret_cast<const uint32_t *>(rows + jj * 8 + (q >> 1) * 4) >> (16 * (q & 1));
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const bf16x8 bop = weights_operand<W>(words, scale, j);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aop, bop, acc[j], 0, 0, 0);
-            }
-        }
-    }
+    while (unit < unit_end) {
+        // ---- one segment: output group og, k-tiles [k_begin, k_end) ---------------------------------------
+        const uint64_t og = unit / p.kt;
+        const uint32_t k_begin = (uint32_t)(unit - og * p.kt);
+        const uint32_t k_end = (uint32_t)min((uint64_t)p.kt, k_begin + (unit_end - unit));
+        unit += k_end - k_begin;
+        const uint32_t ng = (uint32_t)(og % p.ngroups);
+        const uint32_t mt = (uint32_t)((og / p.ngroups) % p.mt);
+        const uint32_t bb = (uint32_t)(og / ((uint64_t)p.ngroups * p.mt));
+        const uint32_t nt0 = ng * GROUP_TILES;
+        const uint32_t n_valid = min((uint32_t)GROUP_TILES, p.nt - nt0);
 
-    // hand over: wavefront w keeps accumulator registers 4w..4w+3 of all four MFMAs (rows 8w + 4g + 0..3)
-    __syncthreads();
-    float *red = reinterpret_cast<float *>(lds);
+        // tiles past the matrix edge repeat the last chunk that exists and are never stored; rows past M repeat
+        // the last row and are never stored
+        const uint32_t chunks_valid = n_valid * F::chunks;
 #pragma unroll
-    for (int ow = 0; ow < WAVES; ++ow) {
-        if (ow == wave) continue;
-        const int slot = ow < wave ? ow : ow - 1;     // 3 slots per source wavefront
+        for (int l = 0; l < NLOAD; ++l) src_off[l] = min(chunk_of[l], chunks_valid - 1) * 16;
+        wptr = p.b + ((uint64_t)(p.b_batch == 1 ? 0 : bb) * p.kt * p.nt + (uint64_t)(k_begin + wave) * p.nt + nt0) * F::tile_bytes;
+        const uint32_t m_row = min(mt * 32 + c, p.m - 1);
+        // activations of one k-tile for this lane: row m, k = kt*32 + h*16 + g*8 .. +7 for h = 0, 1
+        if (p.a_tiled) aptr = p.a + (((uint64_t)bb * p.mt + mt) * p.kt + k_begin + wave) * 2048 + (c >> 4) * 1024 + (c & 15) * 32 + g * 16;
+        else aptr = p.a + (((uint64_t)bb * p.m + m_row) * p.k + (k_begin + wave) * 32 + g * 8) * 2;
+
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                red[(((wave * 3 + slot) * 16) + j * 4 + r) * 64 + lane] = acc[j][ow * 4 + r];
-    }
-    __syncthreads();
-    float mine[4][4];   // [r][j]
+            for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+
+        uint32_t kt = k_begin + wave;
+        if (kt < k_end) fetch();
+        for (; kt < k_end; kt += WAVES) {
+            // what was requested one iteration ago lands in LDS / registers; the next k-tile is requested before
+            // any arithmetic starts, so its latency hides behind the dequantisation and the MFMAs below
+            stash();
+            const u32x4 a_cur0 = a_next[0], a_cur1 = a_next[1];
+            if (kt + WAVES < k_end) fetch();
+            half_step(a_cur0, 0);
+            half_step(a_cur1, 1);
+        }
+
+#if defined(TTMI_PROBE) && TTMI_PROBE == 6
+        if (p.units) { if (acc[0][0] == 1.2345f) p.c[0] = 1; return; }
+#endif
+        // ---- hand over: wavefront w keeps accumulator registers 4w..4w+3 of all four MFMAs (rows 8w+4g+0..3) ----
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(lds);
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+        for (int ow = 0; ow < WAVES; ++ow) {
+            if (ow == wave) continue;
+            const int slot = ow < wave ? ow : ow - 1;     // 3 slots per source wavefront
 #pragma unroll
-        for (int r = 0; r < 4; ++r) mine[r][j] = acc[j][wave * 4 + r];
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-    for (int sw = 0; sw < WAVES; ++sw) {
-        if (sw == wave) continue;
-        const int slot = wave < sw ? wave : wave - 1;
+                for (int r = 0; r < 4; ++r)
+                    red[(((wave * 3 + slot) * 16) + j * 4 + r) * 64 + lane] = acc[j][ow * 4 + r];
+        }
+        __syncthreads();
+        float mine[4][4];   // [r][j]
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) mine[r][j] += red[(((sw * 3 + slot) * 16) + j * 4 + r) * 64 + lane];
-    }
+            for (int r = 0; r < 4; ++r) mine[r][j] = acc[j][wave * 4 + r];
+#pragma unroll
+        for (int sw = 0; sw < WAVES; ++sw) {
+            if (sw == wave) continue;
+            const int slot = wave < sw ? wave : wave - 1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mine[r][j] += red[(((sw * 3 + slot) * 16) + j * 4 + r) * 64 + lane];
+        }
 
-    if (t_of_lane >= (int)n_valid) return;
-    const uint32_t n_col = (nt0 + t_of_lane) * 32 + fc * 16 + q * 4;   // first of this lane's 4 columns
+        // ---- outputs shared with other workgroups ----------------------------------------------------------
+        bool store_now = true;
+        if (k_begin != 0 || k_end != p.kt) {
+            // contributors: workgroups first..last, the ones whose ranges meet [og*kt, (og+1)*kt)
+            const uint64_t lo = og * p.kt, hi = lo + p.kt - 1;
+            uint32_t first = (uint32_t)(lo * p.workgroups / p.units), last = (uint32_t)(hi * p.workgroups / p.units);
+            while (first + 1 < p.workgroups && range_start(p.units, p.workgroups, first + 1) <= lo) ++first;
+            while (range_start(p.units, p.workgroups, first) > lo) --first;
+            while (last + 1 < p.workgroups && range_start(p.units, p.workgroups, last + 1) <= hi) ++last;
+            while (range_start(p.units, p.workgroups, last) > hi) --last;
+            float4 *slot = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(2 * me + (og == my_first_og ? 0 : 1)) * 16 + wave * 4) * 64 + lane;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const uint32_t row_in_band = wave * 8 + g * 4 + r;
-        const uint32_t row = mt * 32 + row_in_band;
-        if (row >= p.m) continue;
-        if (p.ksplit > 1) {
-            float *to = p.partial + ((uint64_t)ks * p.batch * p.m + (uint64_t)bb * p.m + row) * p.n + n_col;
-            *reinterpret_cast<float4 *>(to) = make_float4(mine[r][0], mine[r][1], mine[r][2], mine[r][3]);
-            continue;
-        }
-        float v[4];
+            for (int r = 0; r < 4; ++r) slot_store(slot + r * 64, make_float4(mine[r][0], mine[r][1], mine[r][2], mine[r][3]));
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // our slot stores have completed ...
+            __syncthreads();
+            if (threadIdx.x == 0)                                    // ... before the arrival is announced
+                arrival = __hip_atomic_fetch_add(&p.counters[og], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            store_now = arrival == last - first;
+            if (store_now) {
+                float sum[4][4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float x = mine[r][j];
-            if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
-            v[j] = apply_activation(x, p.activation);
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) sum[r][j] = 0.f;
+                for (uint32_t w = first; w <= last; ++w) {         // fixed order: the result does not depend on who is last
+                    if (w == me) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) sum[r][j] += mine[r][j];
+                        continue;
+                    }
+                    const bool is_first_og = range_start(p.units, p.workgroups, w) / p.kt == og;
+                    const float4 *other = reinterpret_cast<const float4 *>(p.slots) + ((uint64_t)(2 * w + (is_first_og ? 0 : 1)) * 16 + wave * 4) * 64 + lane;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float4 v = slot_load(other + r * 64);
+                        sum[r][0] += v.x; sum[r][1] += v.y; sum[r][2] += v.z; sum[r][3] += v.w;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) mine[r][j] = sum[r][j];
+                if (threadIdx.x == 0) __hip_atomic_store(&p.counters[og], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+            }
         }
-        uint64_t elem;   // element offset of the 4-column run in C
-        if (p.c_tiled) {
-            const uint64_t tile = ((uint64_t)bb * p.mt + mt) * p.nt + nt0 + t_of_lane;
-            elem = tile * 1024 + ((row_in_band >> 4) * 2 + fc) * 256 + (row_in_band & 15) * 16 + q * 4;
-        } else {
-            elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
-        }
-        if (p.c_f32) {
-            *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
-        } else {
-            const uint32_t lo = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
-            const uint32_t hi = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
-            *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo, hi);
-        }
-    }
-}
 
-// Sums the k-range partials, applies bias / activation, converts and stores in the output layout.
-__global__ __launch_bounds__(256) void matmul_finish_kernel(const MatmulDev p) {
-    const uint64_t quads = (uint64_t)p.batch * p.m * (p.n / 4);
-    const uint64_t at = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (at >= quads) return;
-    const uint32_t n_col = (uint32_t)(at % (p.n / 4)) * 4;
-    const uint64_t brow = at / (p.n / 4);        // b*m + row
-    const uint32_t row = (uint32_t)(brow % p.m);
-    const uint32_t bb = (uint32_t)(brow / p.m);
-    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t ks = 0; ks < p.ksplit; ++ks) {
-        const float4 v = *reinterpret_cast<const float4 *>(p.partial + ((uint64_t)ks * p.batch * p.m + brow) * p.n + n_col);
-        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
-    }
-    float v[4] = {sum.x, sum.y, sum.z, sum.w};
+#if defined(TTMI_PROBE) && TTMI_PROBE == 7
+        if (p.units) { if (mine[0][0] == 1.2345f) p.c[0] = 1; return; }
+#endif
+        if (store_now && t_of_lane < (int)n_valid) {
+            const uint32_t n_col = (nt0 + t_of_lane) * 32 + fc * 16 + q * 4;   // first of this lane's 4 columns
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if (p.bias) v[j] += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
-        v[j] = apply_activation(v[j], p.activation);
-    }
-    uint64_t elem;
-    if (p.c_tiled) {
-        const uint32_t mt = row >> 5, rin = row & 31, nt = n_col >> 5, cin = n_col & 31;
-        const uint64_t tile = ((uint64_t)bb * p.mt + mt) * p.nt + nt;
-        elem = tile * 1024 + ((rin >> 4) * 2 + (cin >> 4)) * 256 + (rin & 15) * 16 + (cin & 15);
-    } else {
-        elem = brow * p.n + n_col;
-    }
-    if (p.c_f32) {
-        *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
-    } else {
-        const uint32_t lo = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
-        const uint32_t hi = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
-        *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo, hi);
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t row_in_band = wave * 8 + g * 4 + r;
+                const uint32_t row = mt * 32 + row_in_band;
+                if (row >= p.m) continue;
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float x = mine[r][j];
+                    if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
+                    v[j] = apply_activation(x, p.activation);
+                }
+                uint64_t elem;   // element offset of the 4-column run in C
+                if (p.c_tiled) {
+                    const uint64_t tile = ((uint64_t)bb * p.mt + mt) * p.nt + nt0 + t_of_lane;
+                    elem = tile * 1024 + ((row_in_band >> 4) * 2 + fc) * 256 + (row_in_band & 15) * 16 + q * 4;
+                } else {
+                    elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
+                }
+                if (p.c_f32) {
+                    *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                    const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
+                    const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
+                    *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
+                }
+            }
+        }
+        __syncthreads();   // LDS is reused by the next segment
     }
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// host side: split selection, workspace, launch
+// host side: decomposition, workspace, launch
 // ---------------------------------------------------------------------------------------------------------
 static uint32_t env_u32(const char *name, uint32_t fallback) {
     const char *v = getenv(name);
@@ -307,79 +426,88 @@ static uint32_t env_u32(const char *name, uint32_t fallback) {
     return x > 0 ? (uint32_t)x : fallback;
 }
 
-static uint32_t choose_ksplit(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
-    const uint32_t mt = (m + 31) / 32, kt = k / 32, nt = n / 32;
-    const uint32_t base = batch * mt * ((nt + GROUP_TILES - 1) / GROUP_TILES);
-    const uint32_t forced = env_u32("TTMI_MATMUL_KSPLIT", 0);
-    uint32_t split = forced ? forced : (env_u32("TTMI_MATMUL_TARGET_WGS", 768) + base - 1) / base;
-    const uint32_t max_split = kt / WAVES ? kt / WAVES : 1;   // every wavefront gets at least one k-tile
-    if (split > max_split) split = max_split;
-    if (split < 1) split = 1;
-    const uint32_t per = (kt + split - 1) / split;
-    return (kt + per - 1) / per;                              // drop empty ranges
+constexpr size_t SLOT_BYTES = 32 * GROUP_TILES * 32 * sizeof(float);   // one 32 x 128 fp32 partial
+
+struct Decomposition { uint32_t mt, kt, nt, ngroups, workgroups; uint64_t groups, units; };
+
+static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
+    Decomposition d{};
+    d.mt = (m + 31) / 32; d.kt = k / 32; d.nt = n / 32;
+    d.ngroups = (d.nt + GROUP_TILES - 1) / GROUP_TILES;
+    d.groups = (uint64_t)batch * d.mt * d.ngroups;
+    d.units = d.groups * d.kt;
+    // what one MI355X keeps resident: 256 CUs x 2 workgroups of 4 wavefronts
+    const uint64_t want = env_u32("TTMI_MATMUL_WGS", 512);
+    d.workgroups = (uint32_t)(d.units < want ? d.units : want);
+    return d;
 }
+
+static size_t counters_bytes(const Decomposition &d) { return (d.groups * sizeof(uint32_t) + 255) / 256 * 256; }
 
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int) {
     if (!batch || !m || !k || !n) return 0;
-    const uint32_t split = choose_ksplit(batch, m, k, n);
-    return split > 1 ? (size_t)split * batch * m * n * sizeof(float) : 0;
+    const Decomposition d = decompose(batch, m, k, n);
+    return counters_bytes(d) + (size_t)2 * d.workgroups * SLOT_BYTES;
 }
 
-// The library's own scratch, one per device, grown on demand and kept until the process ends.
-static void *g_scratch[64] = {nullptr};
-static size_t g_scratch_bytes[64] = {0};
+// The library's own scratch, per device, grown on demand and kept until the process ends: arrival counters
+// (zeroed when allocated; every launch leaves them at zero again) and partial-sum slots.  They are separate
+// allocations so that slot data of one problem size can never be read as counters of another.
+struct Scratch { void *ptr = nullptr; size_t bytes = 0; };
+static Scratch g_counters[64], g_slots[64];
 
-static int own_scratch(size_t bytes, void **out) {
+static int grow(Scratch &s, size_t bytes, bool zero) {
+    if (s.bytes >= bytes) return TTMI_OK;
+    if (s.ptr) {
+        if (int rc = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize")) return rc;
+        if (int rc = check_hip(hipFree(s.ptr), "hipFree")) return rc;
+        s.ptr = nullptr; s.bytes = 0;
+    }
+    if (int rc = check_hip(hipMalloc(&s.ptr, bytes), "hipMalloc(matmul scratch)")) return rc;
+    if (zero) if (int rc = check_hip(hipMemset(s.ptr, 0, bytes), "hipMemset(matmul scratch)")) return rc;
+    s.bytes = bytes;
+    return TTMI_OK;
+}
+
+static int own_scratch(size_t counter_bytes, size_t slot_bytes, void **counters, void **slots) {
     int dev = 0;
     if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
     if (dev < 0 || dev >= 64) return fail(TTMI_ERR_UNSUPPORTED, "device index %d out of range", dev);
-    if (g_scratch_bytes[dev] < bytes) {
-        if (g_scratch[dev]) {
-            if (int rc = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize")) return rc;
-            if (int rc = check_hip(hipFree(g_scratch[dev]), "hipFree")) return rc;
-            g_scratch[dev] = nullptr; g_scratch_bytes[dev] = 0;
-        }
-        if (int rc = check_hip(hipMalloc(&g_scratch[dev], bytes), "hipMalloc(matmul scratch)")) return rc;
-        g_scratch_bytes[dev] = bytes;
-    }
-    *out = g_scratch[dev];
+    if (int rc = grow(g_counters[dev], counter_bytes, true)) return rc;
+    if (int rc = grow(g_slots[dev], slot_bytes, false)) return rc;
+    *counters = g_counters[dev].ptr;
+    *slots = g_slots[dev].ptr;
     return TTMI_OK;
 }
 
 int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
+    const Decomposition d = decompose(x.batch, x.m, x.k, x.n);
     MatmulDev p{};
     p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
-    p.mt = (x.m + 31) / 32; p.kt = x.k / 32; p.nt = x.n / 32;
-    p.ngroups = (p.nt + GROUP_TILES - 1) / GROUP_TILES;
-    p.ksplit = choose_ksplit(x.batch, x.m, x.k, x.n);
-    p.kt_per_split = (p.kt + p.ksplit - 1) / p.ksplit;
+    p.mt = d.mt; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.workgroups = d.workgroups; p.units = d.units;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE;
     p.c_f32 = x.c_dtype == TTMI_FLOAT32; p.activation = x.activation;
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
-    const uint64_t blocks = (uint64_t)p.batch * p.mt * p.ngroups * p.ksplit;
-    if (blocks > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
-    if (p.ksplit > 1) {
-        const size_t need = (size_t)p.ksplit * p.batch * p.m * p.n * sizeof(float);
-        void *ws = x.workspace;
-        if (ws) {
-            if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
-            if (reinterpret_cast<uintptr_t>(ws) & 15u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 16-byte aligned");
-        } else if (int rc = own_scratch(need, &ws)) {
-            return rc;
-        }
-        p.partial = (float *)ws;
+    if (d.groups > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
+    const size_t slot_bytes = (size_t)2 * d.workgroups * SLOT_BYTES, need = counters_bytes(d) + slot_bytes;
+    void *counters = nullptr, *slots = nullptr;
+    if (x.workspace) {
+        if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
+        if (reinterpret_cast<uintptr_t>(x.workspace) & 255u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 256-byte aligned");
+        // a caller's buffer may hold anything: clear the arrival counters for this launch
+        if (int rc = check_hip(hipMemsetAsync(x.workspace, 0, counters_bytes(d), st), "hipMemsetAsync(counters)")) return rc;
+        counters = x.workspace;
+        slots = (uint8_t *)x.workspace + counters_bytes(d);
+    } else if (int rc = own_scratch(counters_bytes(d), slot_bytes, &counters, &slots)) {
+        return rc;
     }
-    if (x.b_fmt == TTMI_BFLOAT8_B) hipLaunchKernelGGL(matmul_stream_kernel<7>, dim3((uint32_t)blocks), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(matmul_stream_kernel<3>, dim3((uint32_t)blocks), dim3(256), 0, st, p);
-    if (int rc = check_launch("matmul_stream_kernel")) return rc;
-    if (p.ksplit > 1) {
-        const uint64_t quads = (uint64_t)p.batch * p.m * (p.n / 4);
-        hipLaunchKernelGGL(matmul_finish_kernel, dim3((uint32_t)((quads + 255) / 256)), dim3(256), 0, st, p);
-        if (int rc = check_launch("matmul_finish_kernel")) return rc;
-    }
-    return TTMI_OK;
+    p.counters = (uint32_t *)counters;
+    p.slots = (float *)slots;
+    if (x.b_fmt == TTMI_BFLOAT8_B) hipLaunchKernelGGL(matmul_stream_kernel<7>, dim3(d.workgroups), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(matmul_stream_kernel<3>, dim3(d.workgroups), dim3(256), 0, st, p);
+    return check_launch("matmul_stream_kernel");
 }
 
 }  // namespace ttmi
