@@ -45,6 +45,7 @@ struct MatmulDev {
     uint32_t workgroups;     // P
     uint32_t units;          // U = batch * mt * ngroups * kt
     uint32_t share, extra;   // U = P * share + extra: the first `extra` workgroups take share + 1 units
+    uint32_t split;          // k ranges per output group, or 0 for stream-K
     int a_tiled, c_tiled, c_f32;
 };
 
@@ -143,9 +144,20 @@ __device__ __forceinline__ float4 slot_load(const float4 *from) {
                        __uint_as_float((uint32_t)(hi >> 32)));
 }
 
-// U units dealt out contiguously to P workgroups: the first `extra` workgroups take share + 1 units, the rest share.
-__device__ __forceinline__ uint32_t range_start(const MatmulDev &p, uint32_t i) { return i * p.share + min(i, p.extra); }
+// Which units a workgroup takes.
+//   split > 0   every output group is cut into `split` nearly equal k ranges, one per workgroup (P = groups * split):
+//               one output per workgroup, at most `split` partial sums to add
+//   split == 0  "stream-K": the U units are dealt out contiguously, the first `extra` workgroups take share + 1 units,
+//               the rest `share`; a range may end one output and begin the next
+__device__ __forceinline__ uint32_t range_start(const MatmulDev &p, uint32_t i) {
+    if (p.split) return (i / p.split) * p.kt + ((i % p.split) * p.kt) / p.split;
+    return i * p.share + min(i, p.extra);
+}
 __device__ __forceinline__ uint32_t workgroup_of(const MatmulDev &p, uint32_t unit) {
+    if (p.split) {
+        const uint32_t og = unit / p.kt, within = unit - og * p.kt;
+        return og * p.split + ((within + 1) * p.split - 1) / p.kt;     // largest part j with (j * kt) / split <= within
+    }
     const uint32_t fat = p.extra * (p.share + 1);
     return unit < fat ? unit / (p.share + 1) : p.extra + (unit - fat) / p.share;
 }
@@ -451,7 +463,7 @@ static uint32_t env_u32(const char *name, uint32_t fallback) {
     return x > 0 ? (uint32_t)x : fallback;
 }
 
-struct Decomposition { uint32_t mt, kt, nt, ngroups, workgroups; uint64_t groups, units; };
+struct Decomposition { uint32_t mt, kt, nt, ngroups, workgroups, split; uint64_t groups, units; };
 
 static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
     Decomposition d{};
@@ -459,9 +471,19 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     d.ngroups = (d.nt + GROUP_TILES - 1) / GROUP_TILES;
     d.groups = (uint64_t)batch * d.mt * d.ngroups;
     d.units = d.groups * d.kt;
-    // what one MI355X keeps resident: 256 CUs x 3 workgroups of 4 wavefronts
-    const uint64_t want = env_u32("TTMI_MATMUL_WGS", 768);
-    d.workgroups = (uint32_t)(d.units < want ? d.units : want);
+    // workgroups in flight at once: 256 CUs x 3 workgroups of 4 wavefronts measured best (4 fit)
+    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", 768);
+    if (env_u32("TTMI_MATMUL_STREAMK", 0)) {
+        d.split = 0;
+        d.workgroups = (uint32_t)(d.units < resident ? d.units : resident);
+    } else {
+        // cut every output's k range into as many parts as keeps the chip full, every wavefront keeping >= 2 k-tiles
+        uint64_t parts = d.groups >= resident ? 1 : resident / d.groups;
+        const uint64_t most = d.kt / (2 * WAVES) ? d.kt / (2 * WAVES) : 1;
+        if (parts > most) parts = most;
+        d.split = (uint32_t)parts;
+        d.workgroups = (uint32_t)(d.groups * parts);
+    }
     return d;
 }
 
@@ -509,12 +531,12 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
     p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
     p.mt = d.mt; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
-    p.share = p.units / p.workgroups; p.extra = p.units % p.workgroups;
+    p.share = p.units / p.workgroups; p.extra = p.units % p.workgroups; p.split = d.split;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE;
     p.c_f32 = x.c_dtype == TTMI_FLOAT32;
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
-    if (d.units > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
+    if (d.units > 0x7fffffffull || d.groups * (d.split ? d.split : 1) > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
     const size_t slot_bytes = (size_t)2 * d.workgroups * SLOT_BYTES, need = counters_bytes(d) + slot_bytes;
     void *counters = nullptr, *slots = nullptr;
     if (x.workspace) {
