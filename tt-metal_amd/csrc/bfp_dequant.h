@@ -1,0 +1,154 @@
+// Device-side pieces shared by the block-float GEMM kernels: operand types, the LDS layout of staged packed tiles,
+// and the exact expansion of block-float codes into bf16 MFMA operands.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ttmi.h"
+
+namespace ttmi {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // first-class 16-byte value: stays in registers
+
+// LDS stage of one wavefront = the 2 adjacent packed tiles of one unit, placed by direct global->LDS loads
+// (global_load_lds_dwordx4: lane l of load i writes its 16 bytes at stage + i*1024 + l*16, from any global
+// address it likes).  Slots are laid out so that what one ds_read touches sits in different banks:
+//   face (tile t, face f = 2h + fc) has index h*4 + t*2 + fc and starts at index * face_stride, i.e. every face is
+//   followed by one 16-byte pad slot; the 8 exponent chunks follow the faces; the remaining slots are dummies.
+template <int W> struct Wfmt;
+template <> struct Wfmt<7> {
+    static constexpr int tile_bytes = 1088, chunks = 68, row_bytes = 16;
+    static constexpr int face_slots = 17, face_stride = face_slots * 16;   // 16 rows + 1 pad
+    static constexpr int exp_base = 8 * face_stride;                        // 2176
+    static constexpr int loads = 3, stage_bytes = loads * 1024;
+    static constexpr int bias_exp = 133;                                    // value = mantissa * 2^(E - 133)
+};
+template <> struct Wfmt<3> {
+    static constexpr int tile_bytes = 576, chunks = 36, row_bytes = 8;
+    static constexpr int face_slots = 9, face_stride = face_slots * 16;    // 8 chunks of 2 rows + 1 pad
+    static constexpr int exp_base = 8 * face_stride;                        // 1152
+    static constexpr int loads = 2, stage_bytes = loads * 1024;
+    static constexpr int bias_exp = 129;                                    // value = mantissa * 2^(E - 129)
+};
+
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 0xf) | (0x7 << 4) | (0xf << 8) | ((N >> 4) << 14));
+    asm volatile("" ::: "memory");
+}
+
+template <int ACT> __device__ __forceinline__ float apply_activation(float x) {
+    if (ACT == TTMI_ACT_RELU) return x > 0.f ? x : 0.f;
+    if (ACT == TTMI_ACT_GELU) return 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
+    if (ACT == TTMI_ACT_SILU) return x / (1.f + __expf(-x));
+    return x;
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+// v_cvt_f32_ubyteN: byte N of a word as float, one instruction (the compiler otherwise extracts the field first)
+template <int SEL> __device__ __forceinline__ float byte_to_float(uint32_t word) {
+    float r;
+    if (SEL == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(word));
+    else if (SEL == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(word));
+    else if (SEL == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(word));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(word));
+    return r;
+}
+
+// Eight weights of one output column, k rows 8g..8g+7, as the bf16 B operand of an MFMA.
+//   words[jj]  mantissa word of k row 8g+jj that contains this column's code, sign bit at bit 7 of its byte
+//   mags[jj]   the same word with only the mantissas left, one per byte
+//   scale[jj]  2^(E - bias_exp) of that row
+//   SEL        which byte of the word
+// Per pair of rows: 2 x v_cvt_f32_ubyteN, 2 x v_mul_f32, v_perm_b32 (keep the upper halves = exact bf16),
+// v_perm_b32 (fetch the two sign bytes) and v_and_or_b32.
+template <int SEL>
+__device__ __forceinline__ bf16x8 weights_operand8(const uint32_t (&words)[8], const uint32_t (&mags)[8], const float (&scale)[8]) {
+    uint32_t packed[4];
+    constexpr uint32_t sign_sel = ((4u + SEL) << 24) | (0x0cu << 16) | ((uint32_t)SEL << 8) | 0x0cu;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t v0 = __float_as_uint(byte_to_float<SEL>(mags[2 * p]) * scale[2 * p]);
+        const uint32_t v1 = __float_as_uint(byte_to_float<SEL>(mags[2 * p + 1]) * scale[2 * p + 1]);
+        const uint32_t both = __builtin_amdgcn_perm(v1, v0, 0x07060302u);
+        const uint32_t signs = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], sign_sel);
+        packed[p] = (signs & 0x80008000u) | both;
+    }
+    return __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+}
+
+// Fills `chunk_of[l]` with the global chunk (16 bytes, counted from the start of a 2-tile run) that lands in this
+// lane's slot of direct-to-LDS load l, for the stage layout described at Wfmt.
+template <int W> __device__ __forceinline__ void stage_chunks(int lane, uint32_t (&chunk_of)[Wfmt<W>::loads]) {
+    using F = Wfmt<W>;
+#pragma unroll
+    for (int l = 0; l < F::loads; ++l) {
+        const uint32_t slot = l * 64 + lane;
+        const uint32_t face_idx = slot / F::face_slots, within = slot % F::face_slots;
+        uint32_t chunk = 0;                                               // pads and dummies refetch chunk 0
+        if (face_idx < 8) {
+            if (within < (uint32_t)F::face_slots - 1) {
+                const uint32_t h = face_idx >> 2, t = (face_idx >> 1) & 1, f = 2 * h + (face_idx & 1);
+                chunk = t * F::chunks + 4 + f * (F::face_slots - 1) + within;
+            }
+        } else if (slot - 8 * F::face_slots < 8) {
+            const uint32_t e = slot - 8 * F::face_slots;                  // exponent chunk e%4 of tile e/4
+            chunk = (e >> 2) * F::chunks + (e & 3);
+        }
+        chunk_of[l] = chunk;
+    }
+}
+
+// The four bf16 B operands (columns 4c+0..3 of a 64-column group, k rows 8g..8g+7) of lane (c = lane % 16,
+// g = lane / 16) from a staged pair of packed tiles.  exp_at / mant_at: this lane's byte offsets into LDS
+// (see Wfmt); q = c % 4.  `after_lds_reads` runs once every LDS read has returned (the stage may be refilled).
+template <int W, typename AfterReads>
+__device__ __forceinline__ void staged_operands(const uint8_t *lds, uint32_t exp_at, uint32_t mant_at, int q,
+                                                AfterReads after_lds_reads, bf16x8 (&bop)[4]) {
+    using F = Wfmt<W>;
+    uint32_t e[8], words[8], mags[8];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) e[jj] = lds[exp_at + jj];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) words[jj] = *reinterpret_cast<const uint32_t *>(lds + mant_at + jj * F::row_bytes);
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0), vmcnt and expcnt untouched
+    asm volatile("" ::: "memory");
+    after_lds_reads();
+    // scale of row jj = 2^(E - bias_exp).  Writing the exponent field directly needs E - bias_exp + 127 >= 1;
+    // a wavefront that meets a smaller exponent (magnitudes below ~2^-120) takes v_ldexp_f32 instead.
+    const uint32_t e_min = min(min(min(e[0], e[1]), min(e[2], e[3])), min(min(e[4], e[5]), min(e[6], e[7])));
+    float scale[8];
+    if (__builtin_expect(__ballot(e_min < (uint32_t)(F::bias_exp - 126)) != 0, 0)) {
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) scale[jj] = __builtin_amdgcn_ldexpf(1.0f, (int)e[jj] - F::bias_exp);
+    } else {
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float((e[jj] << 23) - ((uint32_t)(F::bias_exp - 127) << 23));
+    }
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+        if (W == 7) {
+            mags[jj] = words[jj] & 0x7f7f7f7fu;
+        } else {
+            // four 4-bit codes -> one code per byte; sign bit moved from bit 3 to bit 7 of its byte
+            uint32_t v = (words[jj] >> (16 * (q & 1))) & 0xffffu;
+            v = (v | (v << 8)) & 0x00ff00ffu;
+            v = (v | (v << 4)) & 0x0f0f0f0fu;
+            words[jj] = v << 4;
+            mags[jj] = v & 0x07070707u;
+        }
+    }
+    bop[0] = weights_operand8<0>(words, mags, scale);
+    bop[1] = weights_operand8<1>(words, mags, scale);
+    bop[2] = weights_operand8<2>(words, mags, scale);
+    bop[3] = weights_operand8<3>(words, mags, scale);
+}
+
+}  // namespace ttmi

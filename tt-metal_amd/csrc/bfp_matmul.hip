@@ -25,13 +25,10 @@
 
 #include <type_traits>
 
+#include "bfp_dequant.h"
 #include "ttmi_internal.h"
 
 namespace ttmi {
-
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // first-class 16-byte value: stays in registers
 
 struct MatmulDev {
     const uint8_t *a;        // bf16
@@ -49,84 +46,12 @@ struct MatmulDev {
     int a_tiled, c_tiled, c_f32;
 };
 
-// LDS stage of one wavefront = the 2 adjacent packed tiles of one unit, placed by direct global->LDS loads
-// (global_load_lds_dwordx4: lane l of load i writes its 16 bytes at stage + i*1024 + l*16, from any global
-// address it likes).  Slots are laid out so that what one ds_read touches sits in different banks:
-//   face (tile t, face f = 2h + fc) has index h*4 + t*2 + fc and starts at index * face_stride, i.e. every face is
-//   followed by one 16-byte pad slot; the 8 exponent chunks follow the faces; the remaining slots are dummies.
-template <int W> struct Wfmt;
-template <> struct Wfmt<7> {
-    static constexpr int tile_bytes = 1088, chunks = 68, row_bytes = 16;
-    static constexpr int face_slots = 17, face_stride = face_slots * 16;   // 16 rows + 1 pad
-    static constexpr int exp_base = 8 * face_stride;                        // 2176
-    static constexpr int loads = 3, stage_bytes = loads * 1024;
-    static constexpr int bias_exp = 133;                                    // value = mantissa * 2^(E - 133)
-};
-template <> struct Wfmt<3> {
-    static constexpr int tile_bytes = 576, chunks = 36, row_bytes = 8;
-    static constexpr int face_slots = 9, face_stride = face_slots * 16;    // 8 chunks of 2 rows + 1 pad
-    static constexpr int exp_base = 8 * face_stride;                        // 1152
-    static constexpr int loads = 2, stage_bytes = loads * 1024;
-    static constexpr int bias_exp = 129;                                    // value = mantissa * 2^(E - 129)
-};
-
 constexpr int GROUP_TILES = 2;                       // n tiles per output group
 constexpr int GROUP_COLS = GROUP_TILES * 32;
 constexpr int WAVES = 4;
 constexpr int STAGES = 3;                            // LDS ring per wavefront: two units in flight, one in use
 constexpr int REDUCE_BYTES = WAVES * 32 * 64 * 4;    // every wavefront lays out its 32 accumulator registers
 constexpr size_t SLOT_BYTES = 32 * GROUP_COLS * sizeof(float);
-
-// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
-template <int N> __device__ __forceinline__ void wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt((N & 0xf) | (0x7 << 4) | (0xf << 8) | ((N >> 4) << 14));
-    asm volatile("" ::: "memory");
-}
-
-template <int ACT> __device__ __forceinline__ float apply_activation(float x) {
-    if (ACT == TTMI_ACT_RELU) return x > 0.f ? x : 0.f;
-    if (ACT == TTMI_ACT_GELU) return 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
-    if (ACT == TTMI_ACT_SILU) return x / (1.f + __expf(-x));
-    return x;
-}
-
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
-    uint32_t u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-}
-
-// v_cvt_f32_ubyteN: byte N of a word as float, one instruction (the compiler otherwise extracts the field first)
-template <int SEL> __device__ __forceinline__ float byte_to_float(uint32_t word) {
-    float r;
-    if (SEL == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(word));
-    else if (SEL == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(word));
-    else if (SEL == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(word));
-    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(word));
-    return r;
-}
-
-// Eight weights of one output column, k rows 8g..8g+7, as the bf16 B operand of an MFMA.
-//   words[jj]  mantissa word of k row 8g+jj that contains this column's code, sign bit at bit 7 of its byte
-//   mags[jj]   the same word with only the mantissas left, one per byte
-//   scale[jj]  2^(E - bias_exp) of that row
-//   SEL        which byte of the word
-// Per pair of rows: 2 x v_cvt_f32_ubyteN, 2 x v_mul_f32, v_perm_b32 (keep the upper halves = exact bf16),
-// v_perm_b32 (fetch the two sign bytes) and v_and_or_b32.
-template <int SEL>
-__device__ __forceinline__ bf16x8 weights_operand8(const uint32_t (&words)[8], const uint32_t (&mags)[8], const float (&scale)[8]) {
-    uint32_t packed[4];
-    constexpr uint32_t sign_sel = ((4u + SEL) << 24) | (0x0cu << 16) | ((uint32_t)SEL << 8) | 0x0cu;
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const uint32_t v0 = __float_as_uint(byte_to_float<SEL>(mags[2 * p]) * scale[2 * p]);
-        const uint32_t v1 = __float_as_uint(byte_to_float<SEL>(mags[2 * p + 1]) * scale[2 * p + 1]);
-        const uint32_t both = __builtin_amdgcn_perm(v1, v0, 0x07060302u);
-        const uint32_t signs = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], sign_sel);
-        packed[p] = (signs & 0x80008000u) | both;
-    }
-    return __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
-}
 
 // Partial sums that other workgroups read travel through device-coherent accesses: relaxed atomic stores and loads
 // at agent scope go past the per-XCD L2 (which is not coherent across XCDs), so no cache write-back or invalidate
@@ -182,24 +107,8 @@ __global__ __launch_bounds__(256, 3) void matmul_stream_kernel(const MatmulDev p
     const int h_of_lane = g >> 1, g_low = g & 1;                 // k rows 8g..8g+7 = rows 8*g_low.. of face 2*h + fc
 
     // ---- addressing that does not depend on the segment ---------------------------------------------------
-    // which global chunk (16 bytes, counted from the start of the 2-tile run) lands in this lane's slot of load l
     uint32_t chunk_of[NLOAD];
-#pragma unroll
-    for (int l = 0; l < NLOAD; ++l) {
-        const uint32_t slot = l * 64 + lane;
-        const uint32_t face_idx = slot / F::face_slots, within = slot % F::face_slots;
-        uint32_t chunk = 0;                                               // pads and dummies refetch chunk 0
-        if (face_idx < 8) {
-            if (within < (uint32_t)F::face_slots - 1) {
-                const uint32_t h = face_idx >> 2, t = (face_idx >> 1) & 1, f = 2 * h + (face_idx & 1);
-                chunk = t * F::chunks + 4 + f * (F::face_slots - 1) + within;
-            }
-        } else if (slot - 8 * F::face_slots < 8) {
-            const uint32_t e = slot - 8 * F::face_slots;                  // exponent chunk e%4 of tile e/4
-            chunk = (e >> 2) * F::chunks + (e & 3);
-        }
-        chunk_of[l] = chunk;
-    }
+    stage_chunks<W>(lane, chunk_of);
     // per-lane LDS offsets inside a stage (offsets, not pointers: the accesses stay LDS instructions)
     const uint32_t exp_off = wave * WAVE_LDS + F::exp_base + t_of_lane * 64 + (2 * h_of_lane + fc) * 16 + g_low * 8;
     const uint32_t mant_off = wave * WAVE_LDS + (h_of_lane * 4 + t_of_lane * 2 + fc) * F::face_stride + (g_low * 8) * F::row_bytes +
@@ -227,58 +136,15 @@ __global__ __launch_bounds__(256, 3) void matmul_stream_kernel(const MatmulDev p
         a_next[1] = *reinterpret_cast<const u32x4 *>(aptr + a_half);
         aptr += a_step;
     };
-    // Works on the unit in stage `stage` with activations (a_lo, a_hi).
+    // Works on the unit in the stage at `stage_off` with activations (a_lo, a_hi).
     auto compute = [&](uint32_t stage_off, const bf16x8 a_lo, const bf16x8 a_hi, auto after_lds_reads) {
-        // scale of row jj = 2^(E - bias_exp).  Writing the exponent field directly needs E - bias_exp + 127 >= 1;
-        // a wavefront that meets a smaller exponent (magnitudes below ~2^-120) takes v_ldexp_f32 instead.
-        uint32_t e[8];
+        bf16x8 bop[4];
+        staged_operands<W>(lds, stage_off + exp_off, stage_off + mant_off, q, after_lds_reads, bop);
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) e[jj] = lds[stage_off + exp_off + jj];
-        uint32_t words[8], mags[8];
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-            if (W == 7) words[jj] = *reinterpret_cast<const uint32_t *>(lds + stage_off + mant_off + jj * 16);
-            else words[jj] = *reinterpret_cast<const uint32_t *>(lds + stage_off + mant_off + jj * 8);
+        for (int j = 0; j < 4; ++j) {
+            acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bop[j], acc[0][j], 0, 0, 0);
+            acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bop[j], acc[1][j], 0, 0, 0);
         }
-        // every LDS read of the stage has returned before the stage is handed back to the loader
-        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0), vmcnt and expcnt untouched
-        asm volatile("" ::: "memory");
-        after_lds_reads();
-        const uint32_t e_min = min(min(min(e[0], e[1]), min(e[2], e[3])), min(min(e[4], e[5]), min(e[6], e[7])));
-        float scale[8];
-        if (__builtin_expect(__ballot(e_min < (uint32_t)(F::bias_exp - 126)) != 0, 0)) {
-#pragma unroll
-            for (int jj = 0; jj < 8; ++jj) scale[jj] = __builtin_amdgcn_ldexpf(1.0f, (int)e[jj] - F::bias_exp);
-        } else {
-#pragma unroll
-            for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float((e[jj] << 23) - ((uint32_t)(F::bias_exp - 127) << 23));
-        }
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-            if (W == 7) {
-                mags[jj] = words[jj] & 0x7f7f7f7fu;
-            } else {
-                // four 4-bit codes -> one code per byte; sign bit moved from bit 3 to bit 7 of its byte
-                uint32_t v = (words[jj] >> (16 * (q & 1))) & 0xffffu;
-                v = (v | (v << 8)) & 0x00ff00ffu;
-                v = (v | (v << 4)) & 0x0f0f0f0fu;
-                words[jj] = v << 4;
-                mags[jj] = v & 0x07070707u;
-            }
-        }
-        bf16x8 bop;
-        bop = weights_operand8<0>(words, mags, scale);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bop, acc[0][0], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bop, acc[1][0], 0, 0, 0);
-        bop = weights_operand8<1>(words, mags, scale);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bop, acc[0][1], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bop, acc[1][1], 0, 0, 0);
-        bop = weights_operand8<2>(words, mags, scale);
-        acc[0][2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bop, acc[0][2], 0, 0, 0);
-        acc[1][2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bop, acc[1][2], 0, 0, 0);
-        bop = weights_operand8<3>(words, mags, scale);
-        acc[0][3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bop, acc[0][3], 0, 0, 0);
-        acc[1][3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bop, acc[1][3], 0, 0, 0);
     };
 
     const uint32_t me = blockIdx.x;
@@ -525,7 +391,7 @@ static int own_scratch(size_t counter_bytes, size_t slot_bytes, void **counters,
     return TTMI_OK;
 }
 
-int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
+int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) {
     const Decomposition d = decompose(x.batch, x.m, x.k, x.n);
     MatmulDev p{};
     p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
@@ -563,6 +429,15 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
 #undef TTMI_LAUNCH_ACT
 #undef TTMI_LAUNCH
     return check_launch("matmul_stream_kernel");
+}
+
+// Tall activations are MFMA-bound and go to the tiled kernel; up to 127 rows the weights are streamed once per
+// 32-row band.  TTMI_MATMUL_KERNEL=stream|tile overrides the choice (for tests and measurements).
+int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
+    const char *force = getenv("TTMI_MATMUL_KERNEL");
+    if (force && force[0] == 's') return matmul_bfp_stream(x, st);
+    if (force && force[0] == 't') return matmul_bfp_tiled(x, st);
+    return x.m >= 128 ? matmul_bfp_tiled(x, st) : matmul_bfp_stream(x, st);
 }
 
 }  // namespace ttmi

@@ -32,6 +32,8 @@ struct MatmulArgs {
     void *workspace; size_t workspace_bytes;
 };
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
-int matmul_bfp(const MatmulArgs &args, hipStream_t st);
+int matmul_bfp(const MatmulArgs &args, hipStream_t st);         // streaming kernel (decode shapes) or the tiled one
+int matmul_bfp_stream(const MatmulArgs &args, hipStream_t st);
+int matmul_bfp_tiled(const MatmulArgs &args, hipStream_t st);
 
 }  // namespace ttmi
