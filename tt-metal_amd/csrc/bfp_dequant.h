@@ -106,6 +106,43 @@ template <int W> __device__ __forceinline__ void stage_chunks(int lane, uint32_t
     }
 }
 
+// The same expansion in separate steps, for kernels that overlap it with MFMAs of the previous k step:
+// read_staged issues the LDS reads, prepare_staged (once they have returned) derives the row scales and the
+// mantissa-only words, after which weights_operand8<j>(words, mags, scale) builds operand j.
+struct StagedWords { uint32_t e[8], words[8]; };
+
+template <int W> __device__ __forceinline__ void read_staged(const uint8_t *lds, uint32_t exp_at, uint32_t mant_at, StagedWords &s) {
+    using F = Wfmt<W>;
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) s.e[jj] = lds[exp_at + jj];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) s.words[jj] = *reinterpret_cast<const uint32_t *>(lds + mant_at + jj * F::row_bytes);
+}
+
+template <int W> __device__ __forceinline__ void prepare_staged(StagedWords &s, int q, float (&scale)[8], uint32_t (&mags)[8]) {
+    using F = Wfmt<W>;
+    const uint32_t e_min = min(min(min(s.e[0], s.e[1]), min(s.e[2], s.e[3])), min(min(s.e[4], s.e[5]), min(s.e[6], s.e[7])));
+    if (__builtin_expect(__ballot(e_min < (uint32_t)(F::bias_exp - 126)) != 0, 0)) {
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) scale[jj] = __builtin_amdgcn_ldexpf(1.0f, (int)s.e[jj] - F::bias_exp);
+    } else {
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float((s.e[jj] << 23) - ((uint32_t)(F::bias_exp - 127) << 23));
+    }
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+        if (W == 7) {
+            mags[jj] = s.words[jj] & 0x7f7f7f7fu;
+        } else {
+            uint32_t v = (s.words[jj] >> (16 * (q & 1))) & 0xffffu;
+            v = (v | (v << 8)) & 0x00ff00ffu;
+            v = (v | (v << 4)) & 0x0f0f0f0fu;
+            s.words[jj] = v << 4;
+            mags[jj] = v & 0x07070707u;
+        }
+    }
+}
+
 // The four bf16 B operands (columns 4c+0..3 of a 64-column group, k rows 8g..8g+7) of lane (c = lane % 16,
 // g = lane / 16) from a staged pair of packed tiles.  exp_at / mant_at: this lane's byte offsets into LDS
 // (see Wfmt); q = c % 4.  `after_lds_reads` runs once every LDS read has returned (the stage may be refilled).

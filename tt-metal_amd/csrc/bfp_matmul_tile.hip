@@ -12,6 +12,7 @@
 // Semantics as in bfp_matmul.hip (tt::operations::primary::matmul, tt_eager/tt_dnn/op_library/bmm/bmm_op.hpp:318-346).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include <type_traits>
 
@@ -77,7 +78,9 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
     for (int i = 0; i < A_LOADS; ++i) {
         const uint32_t row_in_block = wave * (BM / 4) + i * 16 + (lane >> 2);
         const uint32_t row = min(m0 + row_in_block, p.m - 1);            // rows past M repeat the last row, never stored
-        const uint32_t kq = lane & 3;
+        // the four 16-byte k chunks of a row are stored XOR-swizzled by (row / 4) % 4, so that the 16 lanes of one
+        // ds_read_b128 pass (16 rows, same k chunk) hit 16 different 16-byte bank groups
+        const uint32_t kq = (lane & 3) ^ ((lane >> 4) & 3);
         if (p.a_tiled) a_off[i] = (row >> 5) * p.kt * 2048 + (((row >> 4) & 1) * 2 + (kq >> 1)) * 512 + (row & 15) * 32 + (kq & 1) * 16;
         else a_off[i] = (row * p.k + kq * 8) * 2;
     }
@@ -87,7 +90,7 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
     const uint32_t exp_off = A_BYTES + wave * F::stage_bytes + F::exp_base + t_of_lane * 64 + (2 * h_of_lane + fc) * 16 + g_low * 8;
     const uint32_t mant_off = A_BYTES + wave * F::stage_bytes + (h_of_lane * 4 + t_of_lane * 2 + fc) * F::face_stride +
                               (g_low * 8) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);
-    const uint32_t a_read_off = c * 64 + g * 16;           // + mb * 1024: this lane's 16 bytes of the 16-row A operand
+    const uint32_t a_read_off = c * 64 + ((g ^ ((c >> 2) & 3)) * 16);   // + mb * 1024: this lane's 16 bytes of the A operand
 
     auto fetch = [&](uint32_t stage) {
         uint8_t *base = lds + stage * STAGE_BYTES;
@@ -111,32 +114,86 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[mb][j][r] = 0.f;
 
-    // ring: k step i lives in stage i % TILE_STAGES and is requested TILE_STAGES - 1 steps ahead
+    // Ring: k step i lives in stage i % TILE_STAGES and is requested TILE_STAGES - 1 steps ahead.  The loop is
+    // software-pipelined inside the wavefront: while the MFMAs of step i run, the weights of step i+1 are expanded
+    // into the other set of B operand registers.  Per iteration i:
+    //   wait until this wavefront's share of step i+1 has landed; barrier (now every share of step i+1 has landed and
+    //   every wavefront has finished reading step i-1, whose stage is refilled); read the packed words of step i+1;
+    //   then for each 16-row block: read its A operand of step i from LDS (a window of A_WINDOW is kept in flight),
+    //   issue its 4 MFMAs, and after every fourth of the blocks build one B operand of step i+1.
     const uint32_t total = p.kt;
     uint32_t requested = 0;
     for (; requested < total && requested < TILE_STAGES - 1; ++requested) fetch(requested);
-    uint32_t stage = 0;
-#pragma unroll 1
-    for (uint32_t i = 0; i < total; ++i) {
-        const uint32_t ahead = requested - i - 1;
+
+    constexpr int A_WINDOW = 8;
+    bf16x8 bop[2][4];
+    StagedWords sw;
+    uint32_t stage = 0, step = 0;      // the k step being multiplied and its stage
+    auto wait_for_step = [&](uint32_t which) {       // vector-memory operations complete in order
+        const uint32_t ahead = requested - which - 1;
         if (ahead >= 2) wait_vmcnt<2 * VM_PER_STEP>();
         else if (ahead == 1) wait_vmcnt<VM_PER_STEP>();
         else wait_vmcnt<0>();
-        __syncthreads();      // everybody's share of step i has landed, and everybody is done reading step i - 1
-        if (requested < total) { fetch(stage == 0 ? TILE_STAGES - 1 : stage - 1); ++requested; }
-        const uint32_t stage_off = stage * STAGE_BYTES;
-        bf16x8 aop[MB];
+    };
+    // prologue: operands of step 0
+    wait_for_step(0);
+    __syncthreads();
+    read_staged<W>(lds, exp_off, mant_off, sw);
+    {
+        float scale[8]; uint32_t mags[8];
+        prepare_staged<W>(sw, q, scale, mags);
+        bop[0][0] = weights_operand8<0>(sw.words, mags, scale);
+        bop[0][1] = weights_operand8<1>(sw.words, mags, scale);
+        bop[0][2] = weights_operand8<2>(sw.words, mags, scale);
+        bop[0][3] = weights_operand8<3>(sw.words, mags, scale);
+    }
+    auto iteration = [&](auto cur_buf, auto has_next) {
+        constexpr int C = decltype(cur_buf)::value, N = 1 - C;
+        constexpr bool more = decltype(has_next)::value;
+        const uint32_t next_stage = stage + 1 == TILE_STAGES ? 0 : stage + 1;
+        const uint32_t a_at = stage * STAGE_BYTES + a_read_off;
+        if (more) {
+            wait_for_step(step + 1);
+            __builtin_amdgcn_s_waitcnt(0xC07F);   // our LDS reads of the previous step have returned
+            __syncthreads();
+            if (requested < total) { fetch(stage == 0 ? TILE_STAGES - 1 : stage - 1); ++requested; }
+        }
+        bf16x8 aop[A_WINDOW];
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-            aop[mb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + stage_off + a_read_off + mb * 1024));
-        bf16x8 bop[4];
-        staged_operands<W>(lds, stage_off + exp_off, stage_off + mant_off, q, [] {}, bop);
+        for (int mb = 0; mb < A_WINDOW; ++mb) aop[mb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + a_at + mb * 1024));
+        if (more) read_staged<W>(lds, next_stage * STAGE_BYTES + exp_off, next_stage * STAGE_BYTES + mant_off, sw);
+        float scale[8]; uint32_t mags[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-                acc[mb][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[mb], bop[j], acc[mb][j], 0, 0, 0);
-        stage = stage + 1 == TILE_STAGES ? 0 : stage + 1;
+            for (int j = 0; j < 4; ++j) acc[mb][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[mb % A_WINDOW], bop[C][j], acc[mb][j], 0, 0, 0);
+            if (mb + A_WINDOW < MB) aop[mb % A_WINDOW] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + a_at + (mb + A_WINDOW) * 1024));
+            if (more) {
+                constexpr int every = MB / 4;          // one operand of the next step per MB/4 row blocks
+                if (mb == 0) prepare_staged<W>(sw, q, scale, mags);
+                if (mb == every - 1) bop[N][0] = weights_operand8<0>(sw.words, mags, scale);
+                if (mb == 2 * every - 1) bop[N][1] = weights_operand8<1>(sw.words, mags, scale);
+                if (mb == 3 * every - 1) bop[N][2] = weights_operand8<2>(sw.words, mags, scale);
+                if (mb == 4 * every - 1) bop[N][3] = weights_operand8<3>(sw.words, mags, scale);
+            }
+        }
+        stage = next_stage;
+        ++step;
+    };
+    using Buf0 = std::integral_constant<int, 0>;
+    using Buf1 = std::integral_constant<int, 1>;
+    // pairs of steps that both have a successor, then the last one or two steps; no branch inside a step touches
+    // the accumulators
+#pragma unroll 1
+    while (step + 2 < total) {
+        iteration(Buf0{}, std::true_type{});
+        iteration(Buf1{}, std::true_type{});
+    }
+    if (total - step == 2) {
+        iteration(Buf0{}, std::true_type{});
+        iteration(Buf1{}, std::false_type{});
+    } else {
+        iteration(Buf0{}, std::false_type{});
     }
 
     // ---- epilogue: lane holds rows mb*16 + 4g + r, columns 4c .. 4c+3 of its wavefront's 64 ------------------
@@ -198,7 +255,8 @@ int matmul_bfp_tiled(const MatmulArgs &x, hipStream_t st) {
     // 256-row blocks when they fill the chip, 128-row blocks otherwise (fewer idle CUs, half the accumulators)
     const uint32_t tiles_n = (x.n + TILE_COLS - 1) / TILE_COLS;
     const uint64_t big = (uint64_t)x.batch * ((x.m + 255) / 256) * tiles_n;
-    const bool use_256 = x.m > 128 && big >= 256 && x.m % 256 == 0;
+    const char *force_bm = getenv("TTMI_MATMUL_BM");
+    const bool use_256 = force_bm ? force_bm[0] == '2' : (x.m > 128 && big >= 256 && x.m % 256 == 0);
     const uint32_t bm = use_256 ? 256 : 128;
     p.tiles_m = (x.m + bm - 1) / bm; p.tiles_n = tiles_n;
     const uint64_t blocks = (uint64_t)x.batch * p.tiles_m * p.tiles_n;
