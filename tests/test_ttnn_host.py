@@ -1,0 +1,82 @@
+"""Host-side behaviour of the TT-NN / tt_lib mirror that needs no GPU: shapes, names, argument validation.
+
+The cases follow tests/ttnn/unit_tests/test_shape.py and the error paths of ttnn/ttnn/operations/core.py:245-311
+and ttnn/ttnn/operations/matmul.py:200-220 of the reference.
+"""
+import pytest
+import torch
+
+import ttnn
+import tt_lib
+
+
+def test_shape_equality_operator():
+    a = ttnn.Shape((1, 2, 3, 4))
+    assert a == (1, 2, 3, 4) and (1, 2, 3, 4) == a
+    assert a.with_tile_padding() == (1, 2, 3, 4) and (1, 2, 3, 4) == a.with_tile_padding()
+    b = ttnn.Shape((1, 2, 3, 4))
+    assert a == b
+    c = ttnn.Shape((1, 2, 3, 4), (1, 2, 32, 32))
+    assert a != c and b != c
+    assert c == (1, 2, 3, 4) and (1, 2, 3, 4) == c
+    assert c.with_tile_padding() == (1, 2, 32, 32) and (1, 2, 32, 32) == c.with_tile_padding()
+    d = ttnn.Shape((1, 2, 32, 32))
+    assert a != d and c != d and d == (1, 2, 32, 32) and d.with_tile_padding() == (1, 2, 32, 32)
+    e = ttnn.Shape((1, 2, 3, 4), (1, 2, 32, 32))
+    assert c == e and a != e and d != e
+    f = ttnn.Shape((1, 2, 4, 4), (1, 2, 32, 32))
+    assert all(x != f for x in (a, b, c, d, e)) and f == (1, 2, 4, 4)
+    g = ttnn.Shape((2, 4, 4), (2, 32, 32))
+    assert all(x != g for x in (a, b, c, d, e, f))
+    assert g == (2, 4, 4) and g.with_tile_padding() == (2, 32, 32)
+
+
+def test_shape_indexing_and_rank():
+    s = ttnn.Shape((1, 2, 3, 4), (1, 2, 32, 32))
+    assert len(s) == 4 and s.rank == 4 and s[-1] == 4 and s[-2] == 3 and tuple(s) == (1, 2, 3, 4)
+    assert s[-2:] == (3, 4) and s[-2:].with_tile_padding() == (32, 32)
+    assert "3[32]" in repr(s)
+    with pytest.raises(RuntimeError):
+        ttnn.Shape((1, 2), (1, 2, 3))
+
+
+def test_names_match_the_reference_enums():
+    # tt_eager/tensor/types.hpp:24-34: the integer values travel through the C ABI
+    assert int(ttnn.bfloat16) == 0 and int(ttnn.float32) == 1 and int(ttnn.bfloat8_b) == 3 and int(ttnn.bfloat4_b) == 4
+    assert int(ttnn.ROW_MAJOR_LAYOUT) == 0 and int(ttnn.TILE_LAYOUT) == 1 and ttnn.TILE_SIZE == 32
+    assert tt_lib.tensor.DataType.BFLOAT8_B is ttnn.bfloat8_b and tt_lib.tensor.Layout.TILE is ttnn.TILE_LAYOUT
+    assert ttnn.DRAM_MEMORY_CONFIG == tt_lib.tensor.MemoryConfig()
+
+
+@pytest.mark.parametrize("dtype", [ttnn.bfloat8_b, ttnn.bfloat4_b])
+def test_from_torch_block_float_argument_errors(dtype):
+    with pytest.raises(RuntimeError, match="requires TILE_LAYOUT"):
+        ttnn.from_torch(torch.zeros(32, 32), dtype=dtype, layout=ttnn.ROW_MAJOR_LAYOUT)
+    with pytest.raises(RuntimeError, match="at least 2 dimensions"):
+        ttnn.from_torch(torch.zeros(32), dtype=dtype, layout=ttnn.TILE_LAYOUT)
+    with pytest.raises(RuntimeError, match="Rank 5 is not supported"):
+        ttnn.from_torch(torch.zeros(1, 1, 1, 32, 32), dtype=dtype, layout=ttnn.TILE_LAYOUT)
+    with pytest.raises(RuntimeError, match="must be of type"):
+        ttnn.from_torch(torch.zeros(32, 32, dtype=torch.uint8), dtype=dtype, layout=ttnn.TILE_LAYOUT)
+    with pytest.raises(RuntimeError, match="device must be specified"):
+        ttnn.from_torch(torch.zeros(32, 32), dtype=dtype, layout=ttnn.TILE_LAYOUT, memory_config=ttnn.DRAM_MEMORY_CONFIG)
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU error path")
+def test_block_float_conversion_without_gpu_fails_loudly():
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ttnn.from_torch(torch.zeros(32, 32), dtype=ttnn.bfloat8_b, layout=ttnn.TILE_LAYOUT)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ttnn.open_device(0)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        tt_lib.tensor.Tensor(torch.zeros(1, 1, 32, 32), tt_lib.tensor.DataType.BFLOAT8_B)
+
+
+def test_matmul_validation_on_host_tensors():
+    a = ttnn.from_torch(torch.zeros(32, 32, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="layout TILE"):
+        ttnn.matmul(a, a)
+    with pytest.raises(RuntimeError, match="rank"):
+        ttnn.matmul(ttnn.from_torch(torch.zeros(32, dtype=torch.bfloat16)), a)
+    with pytest.raises(RuntimeError, match="must be of type"):
+        ttnn.matmul(ttnn.from_torch(torch.zeros(32, 32, dtype=torch.float32)), a)

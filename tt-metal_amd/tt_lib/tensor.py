@@ -314,20 +314,26 @@ def _matmul(a: Tensor, b: Tensor, *, bcast_batch: bool, bias: Optional[Tensor] =
         if bias._padded[-1] != n:
             raise RuntimeError("TT_FATAL: bias width must match the output width")
         bb = bias
-        if bb.dtype in _BFP:
-            raise RuntimeError("bias must be BFLOAT16")
+        bh = bb._padded[-2] if len(bb._padded) > 1 else 1
         # bias is a [.., 32, N] tile row in the reference; row 0 carries the values (matmul.hpp:117-140)
-        row = capi.untilize(bb._buf, (1, bb._padded[-2] if len(bb._padded) > 1 else 1, n)) if bb.layout == Layout.TILE else bb._buf.view(-1, n)
+        if bb.dtype in _BFP:
+            row = capi.unpack_tensor(int(bb.dtype), bb._buf, (1, bh, n), dtype=torch.bfloat16)
+        elif bb.layout == Layout.TILE:
+            row = capi.untilize(bb._buf, (1, bh, n))
+        else:
+            row = bb._buf.view(-1, n)
         bias_buf = row.reshape(-1, n)[0].contiguous().to(torch.bfloat16)
-    out_dtype = DataType(output_dtype) if output_dtype is not None else (a.dtype if a.dtype == DataType.BFLOAT16 else DataType.BFLOAT16)
-    if out_dtype != DataType.BFLOAT16:
-        raise RuntimeError(f"{op}: output dtype {out_dtype.name} is not supported yet (BFLOAT16 only)")
+    out_dtype = DataType(output_dtype) if output_dtype is not None else a.dtype  # bmm_op.hpp:388: output takes input a's dtype
+    if out_dtype not in (DataType.BFLOAT16,) + _BFP:
+        raise RuntimeError(f"{op}: output dtype {out_dtype.name} is not supported (BFLOAT16, BFLOAT8_B, BFLOAT4_B)")
     with torch.cuda.device(a._device.torch_device):
         c = capi.matmul_bfp(a_buf, capi.TILE, b._buf, int(b.dtype), batch_a, batch_b, m, k, n, bias=bias_buf,
                             activation=activation, c_layout=capi.TILE, out_dtype=torch.bfloat16)
+        if out_dtype in _BFP:  # the packer of the reference's compute kernel, applied to the bf16 result tiles
+            c = capi.pack_chunks(int(out_dtype), c.float(), False)
     logical = tuple(a._shape[:-1]) + (b._shape[-1],)
     padded = pa[:-1] + (n,)
-    return Tensor(None, _raw=(c, logical, padded, DataType.BFLOAT16, Layout.TILE, a._device))
+    return Tensor(None, _raw=(c, logical, padded, out_dtype, Layout.TILE, a._device))
 
 
 def matmul(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None, kernel_config=None,

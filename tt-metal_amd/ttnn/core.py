@@ -1,0 +1,137 @@
+"""ttnn.from_torch / to_torch / to_layout / to_device / from_device / reshape (ttnn/ttnn/operations/core.py)."""
+from __future__ import annotations
+
+from typing import Optional, Tuple, Union
+
+import torch
+
+import ttnn
+from tt_lib.tensor import DataType, Layout, Tensor, Device, _BFP, _TORCH, _pad32, _run_on_gpu
+from ttmi import capi
+
+
+def _check_rank(operation_name, shape, ranks=(1, 2, 3, 4, 5, 6, 7, 8)):
+    if len(shape) not in ranks:
+        raise RuntimeError(f"{operation_name}: ttnn.Tensor must be of rank {ranks}, but got {len(shape)}")
+
+
+def from_torch(tensor: "torch.Tensor", dtype: Optional[DataType] = None, *, layout: Optional[Layout] = ttnn.ROW_MAJOR_LAYOUT,
+               device: Optional[Device] = None, memory_config=None, mesh_mapper=None) -> Tensor:
+    """core.py:245-311.  For bfloat8_b / bfloat4_b the reference pads to tile multiples, packs, unpacks, tilizes and
+    packs again on the host; here that whole sequence is ONE fused kernel (pad + tilize + pack), bit-identical to it."""
+    _check_rank("ttnn.from_torch", tensor.shape)
+    if tensor.dtype not in (torch.bfloat16, torch.float32, torch.int16, torch.int32, torch.int64, torch.float16):
+        raise RuntimeError(f"ttnn.from_torch: ttnn.Tensor must be of type bfloat16/float32/int16/int32/int64/float16, but got {tensor.dtype}")
+    if mesh_mapper is not None:
+        raise RuntimeError("ttnn.from_torch: mesh_mapper needs several devices; this build drives one GPU")
+    if memory_config is not None and device is None:
+        raise RuntimeError("device must be specified when memory_config is specified")
+    if dtype in _BFP:
+        if len(tensor.shape) < 2:
+            raise RuntimeError("ttnn.from_torch: bfloat8_b/bfloat4_b requires at least 2 dimensions!")
+        if layout != ttnn.TILE_LAYOUT:
+            raise RuntimeError("ttnn.from_torch: bfloat8_b/bfloat4_b requires TILE_LAYOUT!")
+        if len(tensor.shape) > 4:
+            raise RuntimeError(f"Rank {len(tensor.shape)} is not supported!")  # tensor_impl.hpp:143-155
+        src = tensor
+        if src.dtype == torch.float16:
+            src = src.to(torch.bfloat16)          # the reference's dtype-less pre-pass rounds fp16 to bf16 (core.py:282)
+        if src.dtype not in (torch.float32, torch.bfloat16):
+            src = src.to(torch.float32)
+        src = src.contiguous()
+        logical = tuple(src.shape)
+        padded = logical[:-2] + (_pad32(logical[-2]), _pad32(logical[-1]))
+        fmt = int(dtype)
+        target = device.torch_device if device is not None else None
+        words = _run_on_gpu(src, lambda d: capi.pack_tensor(fmt, d), target)
+        if device is not None:
+            words = words.to(device.torch_device)
+        return Tensor(None, _raw=(words, logical, padded, DataType(dtype), Layout.TILE, device))
+
+    t = Tensor(tensor, dtype)
+    if layout is not None:
+        t = to_layout(t, layout)
+    if device is not None:
+        t = to_device(t, device, memory_config=memory_config or ttnn.DRAM_MEMORY_CONFIG)
+    return t
+
+
+def to_torch(tensor: Tensor, *, torch_rank: Optional[int] = None, mesh_composer=None) -> "torch.Tensor":
+    """core.py:336-394: block-float tensors come back as float32, sliced to the logical shape."""
+    if mesh_composer is not None:
+        raise RuntimeError("ttnn.to_torch: mesh_composer needs several devices; this build drives one GPU")
+    _check_rank("ttnn.to_torch", tensor._shape)
+    logical, padded = tuple(tensor._shape), tuple(tensor._padded)
+    if tensor.dtype in _BFP and tensor.layout == Layout.TILE:
+        fmt = int(tensor.dtype)
+        batch, h, w = Tensor._bhw(padded)
+        # one fused kernel: unpack + untilize, cropping the tile padding of the last two dimensions
+        crop = padded[:-2] + (logical[-2], logical[-1])
+        out = _run_on_gpu(tensor._buf, lambda d: capi.unpack_tensor(fmt, d, (batch, logical[-2], logical[-1])))
+        out = out.cpu().view(crop)
+    else:
+        host = tensor.cpu() if tensor.storage_type() == ttnn.DEVICE_STORAGE_TYPE else tensor
+        if host.layout != Layout.ROW_MAJOR:
+            host = host.to(Layout.ROW_MAJOR)
+        out = host.to_torch()
+    out = out[tuple(slice(None, x) for x in logical)]
+    if torch_rank is None:
+        return out
+    while len(out.shape) != torch_rank:
+        if out.shape[0] != 1:
+            raise RuntimeError("ttnn: Unable to squeeze to desired rank!")
+        out = out.squeeze(0)
+    return out
+
+
+def to_layout(tensor: Tensor, layout: Layout, dtype: Optional[DataType] = None, memory_config=None, use_multicore: bool = False) -> Tensor:
+    """core.py:609-803: TILE pads the last two dimensions to multiples of 32 with zeros and keeps the logical shape."""
+    if layout not in (ttnn.ROW_MAJOR_LAYOUT, ttnn.TILE_LAYOUT):
+        raise RuntimeError(f"Unsupported layout: {layout}")
+    if dtype is not None and dtype != tensor.dtype:
+        raise RuntimeError("ttnn.to_layout: changing dtype with the layout is not supported by this build")
+    if tensor.layout == layout:
+        return tensor
+    logical, padded = tuple(tensor._shape), tuple(tensor._padded)
+    if layout == ttnn.TILE_LAYOUT:
+        if tensor.dtype in _BFP:
+            return tensor.to(Layout.TILE)
+        rank = len(logical)
+        if rank < 2 or rank > 4:
+            raise RuntimeError(f"Rank {rank} is not supported!")
+        batch = 1
+        for s in logical[:-2]:
+            batch *= s
+        dense = tensor._buf.reshape(padded)[tuple(slice(None, x) for x in logical)].reshape(batch, logical[-2], logical[-1])
+        dev = tensor._device.torch_device if tensor._device else None
+        buf = _run_on_gpu(dense.contiguous(), lambda d: capi.tilize(d), dev)  # pads with zeros and tilizes in one kernel
+        new_padded = logical[:-2] + (_pad32(logical[-2]), _pad32(logical[-1]))
+        return Tensor(None, _raw=(buf, logical, new_padded, tensor.dtype, Layout.TILE, tensor._device))
+    # to ROW_MAJOR: the tile padding stays part of the (padded) shape, as in the reference
+    return tensor.to(Layout.ROW_MAJOR)
+
+
+def to_device(tensor: Tensor, device: Device, *, memory_config=None) -> Tensor:
+    return tensor.to(device)
+
+
+def from_device(tensor: Tensor) -> Tensor:
+    return tensor.cpu()
+
+
+def deallocate(tensor: Tensor) -> None:
+    tensor.deallocate(force=True)
+
+
+def reshape(input_tensor: Tensor, shape: Union["ttnn.Shape", Tuple[int, ...]]) -> Tensor:
+    return input_tensor.reshape(shape)
+
+
+def unsqueeze_to_4D(tensor: Tensor) -> Tensor:
+    rank = len(tensor._shape)
+    if rank == 4:
+        return tensor
+    if rank > 4:
+        raise RuntimeError("Tensor cannot have more than 4 dimensions!")
+    lead = (1,) * (4 - rank)
+    return tensor.reshape(ttnn.Shape(lead + tuple(tensor._shape), lead + tuple(tensor._padded)))
