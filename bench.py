@@ -27,6 +27,13 @@ for _p in (ROOT, os.path.join(ROOT, "tt-metal_amd")):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 ROTATE_BYTES = 512 << 20
+WORKLOAD_NAMES = {
+    "decode_falcon": "decode_falcon: bf16 [32,4544] x BFP8_B [4544,18176], then [32,18176] x BFP8_B [18176,4544] (Falcon-7B decode MLP)",
+    "decode_mistral": "decode_mistral: M=32 bf16 x fused QKV / O (BFP8_B) and gate / up / down (BFP4_B) of a Mistral-7B layer",
+    "prefill": "prefill: bf16 [2048,4096] x BFP8_B [4096,14336], and bmm [12,384,1024] x [12,1024,1024] BFP8_B",
+    "pack_bfp4_4k": "pack_bfp4_4k: fused tilize+pack and unpack+untilize of fp32 [1,1,4096,4096] (stress mixture) to BFP4_B",
+    "pack_bfp8_1k": "pack_bfp8_1k: fused tilize+pack and unpack+untilize of fp32 [1,1,1024,1024] ~ N(0,1) to BFP8_B",
+}
 
 
 def parse_args():
@@ -38,6 +45,9 @@ def parse_args():
                     choices=["decode_falcon", "decode_mistral", "prefill", "pack_bfp4_4k", "pack_bfp8_1k"])
     ap.add_argument("--legs", default="all", choices=["all", "primary", "none"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--counter-calibration", action="store_true",
+                    help="first launch a plain elementwise copy of 256 MiB three times, so that a hardware-counter run "
+                         "(FETCH_SIZE / WRITE_SIZE) can be scaled by what the same counter reads for a known transfer")
     return ap.parse_args()
 
 
@@ -123,7 +133,7 @@ def main():
         leg = {"workload": name, "shape": [b, m, k, n], "weights": fmt, "ms": round(ms, 5),
                "tflops": round(flops / (ms * 1e-3) / 1e12, 2), "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1),
                "algorithmic_bytes": nbytes, "flops": flops, "weight_copies_rotated": ncopies, "roofline": roof}
-        return leg, (wcopies, acopies, FMT[fmt], b, m, k, n)
+        return leg, (run, wcopies, acopies, c)
 
     def codec_leg(name, x_np, fmt, steps, warmup):
         x = dev(x_np)
@@ -146,13 +156,25 @@ def main():
         # same loop on one buffer: the working set sits in the Infinity Cache ("hot")
         ms_p_hot = time_loop(lambda i: capi.check(L.ttmi_pack_rowmajor_as_bfp_tiles(*pack_calls[0])), steps, warmup)
         legs = []
+        runs = (lambda i: capi.check(L.ttmi_pack_rowmajor_as_bfp_tiles(*pack_calls[i % ncopies])),
+                lambda i: capi.check(L.ttmi_unpack_bfp_tiles_as_rowmajor(*unpack_calls[i % ncopies])))
+        keep = (xs, ws, out_words, out_x)
         for op, ms, hot in (("pack", ms_p, ms_p_hot), ("unpack", ms_u, None)):
             leg = {"workload": f"{name}_{op}", "shape": list(x.shape), "ms": round(ms, 5), "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1),
                    "algorithmic_bytes": nbytes, "buffers_rotated": ncopies, "roofline": hbm_roofline(nbytes, ms)}
             if hot is not None:
                 leg["gbs_cache_resident"] = round(nbytes / (hot * 1e-3) / 1e9, 1)
             legs.append(leg)
-        return legs
+        return legs, (runs, keep)
+
+    if args.counter_calibration:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)   # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     t0 = time.time()
     legs = []
@@ -167,39 +189,54 @@ def main():
     order = [args.workload] + ([w for w in ("decode_falcon", "decode_mistral", "prefill", "pack_bfp4_4k", "pack_bfp8_1k")
                                if w != args.workload] if args.legs == "all" else [])
     results = {}
+    primary_runs, primary_keep = [], []
     for wl in order:
         note(f"workload {wl}")
-        sub_steps = steps if wl == args.workload else max(10, min(steps, 30))
+        is_primary = wl == args.workload
+        sub_steps = steps if is_primary else max(10, min(steps, 30))
         if wl in gemm_sets:
             sub = []
             for idx, spec in enumerate(gemm_sets[wl]):
                 big = spec[1] > 64
-                leg, state = gemm_leg(spec, max(5, sub_steps // 5) if big else sub_steps, 2 if big else warmup, 1234 + 10 * idx)
+                leg, state = gemm_leg(spec, max(5, sub_steps // 5) if big and not is_primary else sub_steps, 2 if big else warmup, 1234 + 10 * idx)
                 sub.append(leg)
-                if wl == args.workload and idx == 0:
-                    primary_state = state
-                else:
-                    del state
+                if is_primary:
+                    primary_runs.append(state[0])
+                    primary_keep.append(state)
+                del state
                 torch.cuda.empty_cache()
             results[wl] = sub
         else:
             fmt = capi.BFLOAT4_B if wl == "pack_bfp4_4k" else capi.BFLOAT8_B
             x = workloads.stress_mixture() if wl == "pack_bfp4_4k" else workloads.roundtrip_1k()
-            results[wl] = codec_leg(wl, x, fmt, sub_steps, warmup)
+            results[wl], state = codec_leg(wl, x, fmt, sub_steps, warmup)
+            if is_primary:
+                primary_runs.extend(state[0])
+                primary_keep.append(state)
+            del state
+            torch.cuda.empty_cache()
+        if is_primary:
+            # THE timed region of the bench contract: W warm-up steps, then exactly K steps, one step = every part of
+            # the workload once, back to back on one stream, device synchronised on both sides
+            def step(i):
+                for run in primary_runs:
+                    run(i)
+
+            total_ms = time_loop(step, steps, warmup)
+            primary_keep.clear()
+            primary_runs = []
             torch.cuda.empty_cache()
 
     prim = results[args.workload]
-    total_ms = sum(l["ms"] for l in prim)
     if args.workload in gemm_sets:
         total_flops = sum(l["flops"] for l in prim)
         value, unit = total_flops / (total_ms * 1e-3) / 1e12, "TFLOP/s"
-        metric = "bfp_weight_matmul_tflops"
         dtype = "bf16"
     else:
         total_bytes = sum(l["algorithmic_bytes"] for l in prim)
         value, unit = total_bytes / (total_ms * 1e-3) / 1e9, "GB/s"
-        metric = "bfp_pack_unpack_gbs"
         dtype = "u32"
+    metric = "bfp8_b-weight matmul TFLOP/s + % roofline (M=32, M=2048); pack/unpack GB/s"
     dominant = max(prim, key=lambda l: l["ms"])
 
     # ------------------------------------------------------------------------------------------------
@@ -260,7 +297,7 @@ def main():
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(total_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic",
-        "config": {"workload": args.workload, "parts": [l["workload"] for l in prim],
+        "config": {"workload": WORKLOAD_NAMES[args.workload], "parts": [l["workload"] for l in prim],
                    "note": "weights rotate over distinct copies (>512 MiB) so the Infinity Cache cannot serve them"},
         "roofline": dict(dominant["roofline"], kernel=dominant["workload"]),
         "cpu_baseline": cpu,
