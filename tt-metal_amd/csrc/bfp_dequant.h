@@ -144,19 +144,31 @@ template <int W> __device__ __forceinline__ void prepare_staged(StagedWords &s, 
 }
 
 // The four bf16 B operands (columns 4c+0..3 of a 64-column group, k rows 8g..8g+7) of lane (c = lane % 16,
-// g = lane / 16) from a staged pair of packed tiles.  exp_at / mant_at: this lane's byte offsets into LDS
-// (see Wfmt); q = c % 4.  `after_lds_reads` runs once every LDS read has returned (the stage may be refilled).
-template <int W, typename AfterReads>
-__device__ __forceinline__ void staged_operands(const uint8_t *lds, uint32_t exp_at, uint32_t mant_at, int q,
-                                                AfterReads after_lds_reads, bf16x8 (&bop)[4]) {
+// g = lane / 16) from a staged pair of packed tiles.  exp_at / mant_at: this lane's LDS byte addresses of the
+// exponents and mantissa words in stage 0 (see Wfmt); q = c % 4.  `after_lds_reads` runs once every LDS read has
+// returned (the stage may be refilled).
+// LDS reads are written as inline assembly: the compiler orders every LDS read it knows of behind ALL outstanding
+// direct-to-LDS loads (it cannot tell that they write other stages), which would drain the prefetch pipeline at
+// every unit.  STAGE_OFF is a compile-time byte offset added to both addresses; the s_waitcnt carries the results
+// as operands so that nothing that uses them can be scheduled in front of it.
+template <int W, int STAGE_OFF, typename AfterReads>
+__device__ __forceinline__ void staged_operands(uint32_t exp_at, uint32_t mant_at, int q, AfterReads after_lds_reads, bf16x8 (&bop)[4]) {
     using F = Wfmt<W>;
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
     uint32_t e[8], words[8], mags[8];
+    u32x2 e01, w01, w23, w45, w67;
+    const uint32_t mant_stage = mant_at + STAGE_OFF;
+    constexpr int R = F::row_bytes / 4;      // dwords between consecutive k rows
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(e01) : "v"(exp_at), "n"(STAGE_OFF));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(w01) : "v"(mant_stage), "n"(0 * R), "n"(1 * R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(w23) : "v"(mant_stage), "n"(2 * R), "n"(3 * R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(w45) : "v"(mant_stage), "n"(4 * R), "n"(5 * R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(w67) : "v"(mant_stage), "n"(6 * R), "n"(7 * R));
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e01), "+v"(w01), "+v"(w23), "+v"(w45), "+v"(w67)::"memory");
 #pragma unroll
-    for (int jj = 0; jj < 8; ++jj) e[jj] = lds[exp_at + jj];
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) words[jj] = *reinterpret_cast<const uint32_t *>(lds + mant_at + jj * F::row_bytes);
-    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0), vmcnt and expcnt untouched
-    asm volatile("" ::: "memory");
+    for (int jj = 0; jj < 8; ++jj) e[jj] = (e01[jj >> 2] >> (8 * (jj & 3))) & 0xffu;
+    words[0] = w01[0]; words[1] = w01[1]; words[2] = w23[0]; words[3] = w23[1];
+    words[4] = w45[0]; words[5] = w45[1]; words[6] = w67[0]; words[7] = w67[1];
     after_lds_reads();
     // scale of row jj = 2^(E - bias_exp).  Writing the exponent field directly needs E - bias_exp + 127 >= 1;
     // a wavefront that meets a smaller exponent (magnitudes below ~2^-120) takes v_ldexp_f32 instead.

@@ -35,8 +35,7 @@ struct MatmulDev {
     const uint8_t *b;        // packed tiles
     const uint16_t *bias;    // bf16 [n] or null
     uint8_t *c;              // output (bf16 or fp32)
-    float *slots;            // 2 slots of 32x64 fp32 per workgroup, for outputs shared between workgroups
-    uint32_t *counters;      // one arrival counter per output group (all zero between launches)
+    float *slots;            // 2 slots of 32x64 fp32 per workgroup, for outputs shared between workgroups (see SLOT_EMPTY)
     uint32_t batch, b_batch, m, k, n;
     uint32_t mt, kt, nt, ngroups;
     uint32_t workgroups;     // P
@@ -49,25 +48,31 @@ struct MatmulDev {
 constexpr int GROUP_TILES = 2;                       // n tiles per output group
 constexpr int GROUP_COLS = GROUP_TILES * 32;
 constexpr int WAVES = 4;
-constexpr int STAGES = 3;                            // LDS ring per wavefront: two units in flight, one in use
+constexpr int WGS_PER_CU = 3;                        // workgroups of 4 wavefronts per CU (registers and LDS allow 3)
+constexpr int STAGES = 3;                            // LDS ring per wavefront = units requested ahead of the arithmetic
+constexpr int A_LOADS = 2;                           // activation loads per unit (rows c and c + 16 of the band)
 constexpr int REDUCE_BYTES = WAVES * 32 * 64 * 4;    // every wavefront lays out its 32 accumulator registers
 constexpr size_t SLOT_BYTES = 32 * GROUP_COLS * sizeof(float);
 
-// Partial sums that other workgroups read travel through device-coherent accesses: relaxed atomic stores and loads
-// at agent scope go past the per-XCD L2 (which is not coherent across XCDs), so no cache write-back or invalidate
-// is needed — a full agent-scope fence here costs more than the whole GEMM.
-__device__ __forceinline__ void slot_store(float4 *to, const float4 v) {
-    uint64_t *q = reinterpret_cast<uint64_t *>(to);
-    __hip_atomic_store(q, ((uint64_t)__float_as_uint(v.y) << 32) | __float_as_uint(v.x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(q + 1, ((uint64_t)__float_as_uint(v.w) << 32) | __float_as_uint(v.z), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Partial sums that other workgroups read travel through device-coherent accesses (the sc1 bit: past the per-XCD L2,
+// which is not coherent across XCDs), 16 bytes per lane, so neither a cache write-back nor an invalidate is needed —
+// a full agent-scope fence here costs more than the whole GEMM.  There are no flags and no counters: every slot
+// word holds SLOT_EMPTY between launches, the producer overwrites it with data (which it keeps from ever having
+// that bit pattern), and the consumer simply re-reads until no word is SLOT_EMPTY, then puts SLOT_EMPTY back.
+constexpr uint32_t SLOT_EMPTY = 0xffffffffu;         // a NaN that arithmetic on bf16-derived inputs does not produce
+constexpr uint32_t SLOT_SPIN_LIMIT = 1u << 20;       // bounded wait: a lost producer must not hang the GPU
+
+__device__ __forceinline__ void slot_store(float4 *to, const u32x4 v) {
+    // A store of more than 8 bytes reads its data registers for two more cycles after it has issued; the compiler
+    // inserts the wait states for stores of its own, here the s_nop does it.
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(to), "v"(v) : "memory");
 }
-__device__ __forceinline__ float4 slot_load(const float4 *from) {
-    uint64_t *q = reinterpret_cast<uint64_t *>(const_cast<float4 *>(from));
-    const uint64_t lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint64_t hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return make_float4(__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)), __uint_as_float((uint32_t)hi),
-                       __uint_as_float((uint32_t)(hi >> 32)));
+__device__ __forceinline__ u32x4 slot_load_issue(const float4 *from) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(from) : "memory");
+    return v;
 }
+__device__ __forceinline__ uint32_t not_empty(uint32_t bits) { return bits == SLOT_EMPTY ? 0xfffffffeu : bits; }
 
 // Which units a workgroup takes.
 //   split > 0   every output group is cut into `split` nearly equal k ranges, one per workgroup (P = groups * split):
@@ -93,14 +98,14 @@ __device__ __forceinline__ uint32_t workgroup_of(const MatmulDev &p, uint32_t un
 // bumps the group's arrival counter; the workgroup that arrives last adds the slots in workgroup order (so the
 // result does not depend on who was last), applies the epilogue, stores, and resets the counter.
 template <int W, int ACT>
-__global__ __launch_bounds__(256, 3) void matmul_stream_kernel(const MatmulDev p) {
+__global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const MatmulDev p) {
     using F = Wfmt<W>;
     constexpr int WAVE_LDS = STAGES * F::stage_bytes;
     constexpr int LDS_BYTES = REDUCE_BYTES > WAVES * WAVE_LDS ? REDUCE_BYTES : WAVES * WAVE_LDS;
     constexpr int NLOAD = F::loads;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
-    __shared__ uint32_t arrival;
 
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 15, g = lane >> 4;                      // column quad and k-row group of this lane
     const int t_of_lane = c >> 3, fc = (c >> 2) & 1, q = c & 3;  // tile, face column and word inside the face row
@@ -117,29 +122,48 @@ __global__ __launch_bounds__(256, 3) void matmul_stream_kernel(const MatmulDev p
     const uint32_t a_step = p.a_tiled ? WAVES * 2048 : WAVES * 64;
 
     f32x4 acc[2][4];                                  // [16-row half of the band][operand j]
-    u32x4 a_next[2];                                  // activations of the unit after the one being worked on
+    u32x4 a_ring[STAGES][2] = {};                     // activations of the units in flight, one entry per LDS stage
     uint32_t src_off[NLOAD];
     uint32_t a_half = 0;                              // bytes from row c to row c + 16 of the band (set per segment)
     const uint8_t *wptr = nullptr, *aptr = nullptr;
 
-    // Requests the 2 packed tiles of one unit straight into LDS stage `stage` (wavefront-uniform).
-    auto fetch_weights = [&](uint32_t stage) {
+    // Requests one unit: its 2 packed tiles straight into LDS stage S, its activations into a_ring[S].
+    auto fetch = [&](auto stage_tag) __attribute__((always_inline)) {
+        constexpr int S = decltype(stage_tag)::value;
 #pragma unroll
         for (int l = 0; l < NLOAD; ++l)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[l]),
-                                             (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + stage * F::stage_bytes + l * 1024),
+                                             (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * F::stage_bytes + l * 1024),
                                              16, 0, 0);
         wptr += w_step;
-    };
-    auto fetch_activations = [&]() {
-        a_next[0] = *reinterpret_cast<const u32x4 *>(aptr);
-        a_next[1] = *reinterpret_cast<const u32x4 *>(aptr + a_half);
+        // The activation loads and the waits for them are inline assembly as well: with direct-to-LDS loads pending
+        // the compiler waits for ALL vector-memory operations before the first use of any loaded register.  The
+        // ring registers are read-write operands, so each entry stays in one physical register from request to use.
+        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][0]) : "v"(aptr) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][1]) : "v"(aptr + a_half) : "memory");
         aptr += a_step;
     };
-    // Works on the unit in the stage at `stage_off` with activations (a_lo, a_hi).
-    auto compute = [&](uint32_t stage_off, const bf16x8 a_lo, const bf16x8 a_hi, auto after_lds_reads) {
+    // Works on the unit in stage S; once its LDS reads have returned the stage is handed to unit i + STAGES.
+    // `younger` = units requested after this one and still allowed to be in flight.
+    auto work = [&](auto stage_tag, auto younger_tag, bool refill) __attribute__((always_inline)) {
+        constexpr int S = decltype(stage_tag)::value;
+        constexpr int YOUNGER = decltype(younger_tag)::value;
+        if (YOUNGER >= 0) wait_vmcnt<(YOUNGER < 0 ? 0 : YOUNGER) * (NLOAD + A_LOADS)>();   // < 0: the caller has waited
+        asm volatile("" : "+v"(a_ring[S][0]), "+v"(a_ring[S][1]) :: "memory");          // uses stay behind the wait
+        // The activations leave the ring through explicit moves: the ring registers are then free for the next
+        // request, which lands in them directly (a copy of a register still being loaded would wait for the load).
+        u32x4 a_now[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                uint32_t moved;
+                asm volatile("v_mov_b32 %0, %1" : "=v"(moved) : "v"(a_ring[S][h][e]));
+                a_now[h][e] = moved;
+            }
+        const bf16x8 a_lo = __builtin_bit_cast(bf16x8, a_now[0]), a_hi = __builtin_bit_cast(bf16x8, a_now[1]);
         bf16x8 bop[4];
-        staged_operands<W>(lds, stage_off + exp_off, stage_off + mant_off, q, after_lds_reads, bop);
+        staged_operands<W, S * F::stage_bytes>(lds_base + exp_off, lds_base + mant_off, q, [&]() __attribute__((always_inline)) { if (refill) fetch(stage_tag); }, bop);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bop[j], acc[0][j], 0, 0, 0);
@@ -186,26 +210,38 @@ __global__ __launch_bounds__(256, 3) void matmul_stream_kernel(const MatmulDev p
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc[mh][j][r] = 0.f;
 
-        // This wavefront's units: k_begin + wave, + WAVES, ... (`total` of them).  Unit i lives in stage i % STAGES.
-        // Vector-memory operations complete in order, so they are issued in this order:
-        //   weights(0), weights(1), activations(0) | per unit i: activations(i+1), [LDS reads of i], weights(i+2), math
-        // At the top of unit i everything but the youngest weights request must have landed: vmcnt(NLOAD) while a
-        // request is still young, vmcnt(0) at the tail.
+        // This wavefront's units: k_begin + wave, + WAVES, ... (`total` of them).  Unit i lives in stage i % STAGES and
+        // is requested STAGES units ahead: when unit i has been read out of its stage, unit i + STAGES is requested
+        // into it.  Vector-memory operations complete in order, so at the top of unit i exactly the requests of the
+        // units after it may still be in flight: min(STAGES - 1, total - 1 - i) of them.
         const uint32_t span = k_end - k_begin;
         const uint32_t total = span > (uint32_t)wave ? (span - wave + WAVES - 1) / WAVES : 0;
-        if (total > 0) fetch_weights(0);
-        if (total > 1) fetch_weights(1);
-        if (total > 0) fetch_activations();
-        uint32_t stage = 0;
+        static_assert(STAGES == 3, "the unrolled pipeline below is written for three stages");
+        using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>; using S2 = std::integral_constant<int, 2>;
+        uint32_t i = 0;
+        if (total >= 2 * STAGES) {
+            // steady state: every unit worked on here has a successor to request, so the number of requests in
+            // flight at each wait is a constant the compiler can see (no conditional request on the way in)
+            fetch(S0{}); fetch(S1{}); fetch(S2{});
 #pragma unroll 1
-        for (uint32_t i = 0; i < total; ++i) {
-            if (i >= 1 && i + 1 < total) wait_vmcnt<NLOAD>(); else if (i == 0 && total > 1) wait_vmcnt<NLOAD>(); else wait_vmcnt<0>();
-            const bf16x8 a_lo = __builtin_bit_cast(bf16x8, a_next[0]), a_hi = __builtin_bit_cast(bf16x8, a_next[1]);
-            if (i + 1 < total) fetch_activations();
-            const uint32_t refill_stage = stage == 0 ? STAGES - 1 : stage - 1;     // (i + 2) % STAGES
-            compute(stage * F::stage_bytes, a_lo, a_hi, [&]() { if (i + 2 < total) fetch_weights(refill_stage); });
-            stage = stage + 1 == STAGES ? 0 : stage + 1;
+            for (; i + 2 * STAGES <= total; i += STAGES) {
+                work(S0{}, S2{}, true);
+                work(S1{}, S2{}, true);
+                work(S2{}, S2{}, true);
+            }
+        } else {
+            if (total > 0) fetch(S0{});
+            if (total > 1) fetch(S1{});
+            if (total > 2) fetch(S2{});
         }
+        // at most 2 * STAGES - 1 units are left, starting in stage 0
+        auto tail = [&](auto stage_tag, uint32_t at) __attribute__((always_inline)) {
+            if (at >= total) return;
+            const uint32_t after = total - 1 - at;
+            if (after >= 2) wait_vmcnt<2 * (NLOAD + A_LOADS)>(); else if (after == 1) wait_vmcnt<NLOAD + A_LOADS>(); else wait_vmcnt<0>();
+            work(stage_tag, std::integral_constant<int, -1>{}, at + STAGES < total);
+        };
+        tail(S0{}, i); tail(S1{}, i + 1); tail(S2{}, i + 2); tail(S0{}, i + 3); tail(S1{}, i + 4);
 
         // ---- add the four wavefronts' partial sums through LDS --------------------------------------------------
         // Every wavefront writes all 32 of its accumulator registers (register indices are compile-time constants;
@@ -235,53 +271,75 @@ __global__ __launch_bounds__(256, 3) void matmul_stream_kernel(const MatmulDev p
         }
 
         // ---- outputs shared with other workgroups ----------------------------------------------------------
+        // Contributors are the workgroups first..last whose ranges meet this output's k range.  The last one (the
+        // highest index: every other contributor was dispatched before it and waits for nobody, so it will finish)
+        // collects the others' partial sums and adds them in workgroup order, its own last: the result does not
+        // depend on timing.  Wavefront w of every contributor holds the same rows, so the hand-over is wavefront to
+        // wavefront and needs no workgroup barrier.
         bool store_now = true;
         if (k_begin != 0 || k_end != p.kt) {
-            // contributors: workgroups first..last, the ones whose ranges meet [og*kt, (og+1)*kt)
             const uint32_t lo = og * p.kt;
             const uint32_t first = workgroup_of(p, lo), last = workgroup_of(p, lo + p.kt - 1);
-            float4 *slot = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(2 * me + (og == my_first_og ? 0 : 1)) * 8 + wave * 2) * 64 + lane;
+            if (me != last) {
+                float4 *slot = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(2 * me + (og == my_first_og ? 0 : 1)) * 8 + wave * 2) * 64 + lane;
 #pragma unroll
-            for (int r = 0; r < 2; ++r) slot_store(slot + r * 64, make_float4(mine[r][0], mine[r][1], mine[r][2], mine[r][3]));
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // our slot stores have completed ...
-            __syncthreads();
-            if (threadIdx.x == 0)                                    // ... before the arrival is announced
-                arrival = __hip_atomic_fetch_add(&p.counters[og], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __syncthreads();
-            store_now = arrival == last - first;
-            if (store_now) {
+                for (int r = 0; r < 2; ++r) {
+                    u32x4 v;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[r][j]));
+                    slot_store(slot + r * 64, v);
+                }
+                store_now = false;
+            } else {
                 float sum[2][4];
 #pragma unroll
                 for (int r = 0; r < 2; ++r)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) sum[r][j] = 0.f;
-                // fixed order (the result does not depend on who is last), four contributors' loads in flight at a time
-                for (uint32_t w0 = first; w0 <= last; w0 += 4) {
-                    float4 part[4][2];
+                const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
+                for (uint32_t w0 = first; w0 < last; w0 += 4) {          // four contributors' loads in flight at a time
+                    u32x4 part[4][2];
+                    float4 *other[4];
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
-                        const uint32_t w = min(w0 + u, last);
+                        const uint32_t w = min(w0 + u, last - 1);
                         const uint32_t which = range_start(p, w) >= lo ? 0u : 1u;      // first or second output of w
-                        const float4 *other = reinterpret_cast<const float4 *>(p.slots) + ((uint64_t)(2 * w + which) * 8 + wave * 2) * 64 + lane;
-#pragma unroll
-                        for (int r = 0; r < 2; ++r) part[u][r] = slot_load(other + r * 64);
+                        other[u] = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(2 * w + which) * 8 + wave * 2) * 64 + lane;
                     }
+                    uint32_t spins = 0;
+                    bool waiting;
+                    do {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int r = 0; r < 2; ++r) part[u][r] = slot_load_issue(other[u] + r * 64);
+                        asm volatile("s_waitcnt vmcnt(0)" : "+v"(part[0][0]), "+v"(part[0][1]), "+v"(part[1][0]), "+v"(part[1][1]),
+                                     "+v"(part[2][0]), "+v"(part[2][1]), "+v"(part[3][0]), "+v"(part[3][1])::"memory");
+                        bool missing = false;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) missing |= part[u][r][j] == SLOT_EMPTY;
+                        waiting = __ballot(missing) != 0 && ++spins < SLOT_SPIN_LIMIT;
+                        if (waiting) __builtin_amdgcn_s_sleep(4);
+                    } while (waiting);
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
-                        const uint32_t w = w0 + u;
-                        if (w > last) break;
+                        if (w0 + u >= last) break;
 #pragma unroll
                         for (int r = 0; r < 2; ++r) {
-                            const float4 v = w == me ? make_float4(mine[r][0], mine[r][1], mine[r][2], mine[r][3]) : part[u][r];
-                            sum[r][0] += v.x; sum[r][1] += v.y; sum[r][2] += v.z; sum[r][3] += v.w;
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) sum[r][j] += __uint_as_float(part[u][r][j]);
+                            slot_store(other[u] + r * 64, empty);                       // ready for the next launch
                         }
                     }
                 }
 #pragma unroll
                 for (int r = 0; r < 2; ++r)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) mine[r][j] = sum[r][j];
-                if (threadIdx.x == 0) __hip_atomic_store(&p.counters[og], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+                    for (int j = 0; j < 4; ++j) mine[r][j] = sum[r][j] + mine[r][j];
             }
         }
 
@@ -353,41 +411,33 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     return d;
 }
 
-static size_t counters_bytes(const Decomposition &d) { return (d.groups * sizeof(uint32_t) + 255) / 256 * 256; }
-
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int) {
     if (!batch || !m || !k || !n) return 0;
     const Decomposition d = decompose(batch, m, k, n);
-    return counters_bytes(d) + (size_t)2 * d.workgroups * SLOT_BYTES;
+    return (size_t)2 * d.workgroups * SLOT_BYTES;
 }
 
-// The library's own scratch, per device, grown on demand and kept until the process ends: arrival counters
-// (zeroed when allocated; every launch leaves them at zero again) and partial-sum slots.  They are separate
-// allocations so that slot data of one problem size can never be read as counters of another.
+// The library's own partial-sum slots, per device, grown on demand and kept until the process ends.  Every word is
+// SLOT_EMPTY when allocated, and every launch leaves it that way.
 struct Scratch { void *ptr = nullptr; size_t bytes = 0; };
-static Scratch g_counters[64], g_slots[64];
+static Scratch g_slots[64];
 
-static int grow(Scratch &s, size_t bytes, bool zero) {
-    if (s.bytes >= bytes) return TTMI_OK;
-    if (s.ptr) {
-        if (int rc = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize")) return rc;
-        if (int rc = check_hip(hipFree(s.ptr), "hipFree")) return rc;
-        s.ptr = nullptr; s.bytes = 0;
-    }
-    if (int rc = check_hip(hipMalloc(&s.ptr, bytes), "hipMalloc(matmul scratch)")) return rc;
-    if (zero) if (int rc = check_hip(hipMemset(s.ptr, 0, bytes), "hipMemset(matmul scratch)")) return rc;
-    s.bytes = bytes;
-    return TTMI_OK;
-}
-
-static int own_scratch(size_t counter_bytes, size_t slot_bytes, void **counters, void **slots) {
+static int own_slots(size_t bytes, void **slots) {
     int dev = 0;
     if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
     if (dev < 0 || dev >= 64) return fail(TTMI_ERR_UNSUPPORTED, "device index %d out of range", dev);
-    if (int rc = grow(g_counters[dev], counter_bytes, true)) return rc;
-    if (int rc = grow(g_slots[dev], slot_bytes, false)) return rc;
-    *counters = g_counters[dev].ptr;
-    *slots = g_slots[dev].ptr;
+    Scratch &s = g_slots[dev];
+    if (s.bytes < bytes) {
+        if (s.ptr) {
+            if (int rc = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize")) return rc;
+            if (int rc = check_hip(hipFree(s.ptr), "hipFree")) return rc;
+            s.ptr = nullptr; s.bytes = 0;
+        }
+        if (int rc = check_hip(hipMalloc(&s.ptr, bytes), "hipMalloc(matmul slots)")) return rc;
+        if (int rc = check_hip(hipMemset(s.ptr, 0xff, bytes), "hipMemset(matmul slots)")) return rc;
+        s.bytes = bytes;
+    }
+    *slots = s.ptr;
     return TTMI_OK;
 }
 
@@ -403,19 +453,19 @@ int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) {
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
     if (d.units > 0x7fffffffull || d.groups * (d.split ? d.split : 1) > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
-    const size_t slot_bytes = (size_t)2 * d.workgroups * SLOT_BYTES, need = counters_bytes(d) + slot_bytes;
-    void *counters = nullptr, *slots = nullptr;
-    if (x.workspace) {
+    const size_t need = (size_t)2 * d.workgroups * SLOT_BYTES;
+    void *slots = nullptr;
+    if (d.split == 1) {
+        // every output belongs to one workgroup: no slot is touched
+    } else if (x.workspace) {
         if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
         if (reinterpret_cast<uintptr_t>(x.workspace) & 255u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 256-byte aligned");
-        // a caller's buffer may hold anything: clear the arrival counters for this launch
-        if (int rc = check_hip(hipMemsetAsync(x.workspace, 0, counters_bytes(d), st), "hipMemsetAsync(counters)")) return rc;
-        counters = x.workspace;
-        slots = (uint8_t *)x.workspace + counters_bytes(d);
-    } else if (int rc = own_scratch(counters_bytes(d), slot_bytes, &counters, &slots)) {
+        // a caller's buffer may hold anything: mark every slot of this launch empty
+        if (int rc = check_hip(hipMemsetAsync(x.workspace, 0xff, need, st), "hipMemsetAsync(slots)")) return rc;
+        slots = x.workspace;
+    } else if (int rc = own_slots(need, &slots)) {
         return rc;
     }
-    p.counters = (uint32_t *)counters;
     p.slots = (float *)slots;
 #define TTMI_LAUNCH(W, ACT) hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
 #define TTMI_LAUNCH_ACT(W)                                              \
