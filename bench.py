@@ -45,6 +45,7 @@ def parse_args():
                     choices=["decode_falcon", "decode_mistral", "prefill", "pack_bfp4_4k", "pack_bfp8_1k"])
     ap.add_argument("--legs", default="all", choices=["all", "primary", "none"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--row-major", action="store_true", help="GEMM activations and output dense row-major instead of TILE layout")
     ap.add_argument("--counter-calibration", action="store_true",
                     help="first launch a plain elementwise copy of 256 MiB three times, so that a hardware-counter run "
                          "(FETCH_SIZE / WRITE_SIZE) can be scaled by what the same counter reads for a known transfer")
@@ -122,8 +123,13 @@ def main():
         L = capi.lib()
         stream = torch.cuda.current_stream().cuda_stream
         c = torch.empty((b, m, n), dtype=torch.bfloat16, device="cuda")
-        calls = [(acopies[j].data_ptr(), capi.ROW_MAJOR, wcopies[j].data_ptr(), FMT[fmt], b, b, m, k, n, None, capi.ACT_NONE,
-                  c.data_ptr(), capi.ROW_MAJOR, capi.BFLOAT16, None, 0, stream) for j in range(ncopies)]
+        # operands in TILE layout, as ttnn.matmul requires of its inputs and returns its output
+        # (ttnn/cpp/ttnn/operations/matmul.hpp:39-42); --row-major times dense row-major activations and output instead
+        layout = capi.ROW_MAJOR if args.row_major else capi.TILE
+        if layout == capi.TILE:
+            acopies = [capi.tilize(t) for t in acopies]
+        calls = [(acopies[j].data_ptr(), layout, wcopies[j].data_ptr(), FMT[fmt], b, b, m, k, n, None, capi.ACT_NONE,
+                  c.data_ptr(), layout, capi.BFLOAT16, None, 0, stream) for j in range(ncopies)]
 
         def run(i):
             capi.check(L.ttmi_matmul_bfp(*calls[i % ncopies]))
@@ -132,7 +138,8 @@ def main():
         roof = hbm_roofline(nbytes, ms) if hbm_bound else mfma_roofline(flops, ms)
         leg = {"workload": name, "shape": [b, m, k, n], "weights": fmt, "ms": round(ms, 5),
                "tflops": round(flops / (ms * 1e-3) / 1e12, 2), "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1),
-               "algorithmic_bytes": nbytes, "flops": flops, "weight_copies_rotated": ncopies, "roofline": roof}
+               "algorithmic_bytes": nbytes, "flops": flops, "weight_copies_rotated": ncopies,
+               "layout": "row_major" if args.row_major else "tile", "roofline": roof}
         return leg, (run, wcopies, acopies, c)
 
     def codec_leg(name, x_np, fmt, steps, warmup):

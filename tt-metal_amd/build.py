@@ -9,12 +9,15 @@ import os
 import subprocess
 import sys
 
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libttmi.so")
 SOURCES = ["ttmi_capi.hip", "bfp_codec.hip", "bfp_matmul.hip", "bfp_matmul_tile.hip"]
+ISA_CHECKED = ("bfp_matmul.hip",)
 HEADERS = [os.path.join(CSRC, "ttmi_internal.h"), os.path.join(CSRC, "bfp_dequant.h"), os.path.join(ROOT, "include", "ttmi.h")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -41,6 +44,19 @@ def build(force: bool = False, verbose: bool = False) -> str:
         path = os.path.join(CSRC, src)
         obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
         if force or _stale(obj, [path] + HEADERS):
+            if src in ISA_CHECKED:
+                # the device assembly of this file is inspected before the object is built (see check_isa.py)
+                asm = os.path.join(LIB_DIR, src.replace(".hip", ".s"))
+                cmd = [HIPCC] + FLAGS + ["-S", "--cuda-device-only", path, "-o", asm]
+                if verbose:
+                    print(" ".join(cmd), flush=True)
+                subprocess.run(cmd, check=True)
+                import check_isa
+                if check_isa.check(asm):
+                    if os.path.exists(obj):
+                        os.remove(obj)
+                    raise RuntimeError(f"{src}: the compiler moved registers of hand-scheduled loads; see check_isa.py")
+                os.remove(asm)
             cmd = [HIPCC] + FLAGS + ["-c", path, "-o", obj]
             if verbose:
                 print(" ".join(cmd), flush=True)
