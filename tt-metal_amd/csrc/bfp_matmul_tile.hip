@@ -1,14 +1,22 @@
 // Tiled GEMM with block-float weights for gfx950, for tall activations (prefill, batched bmm): MFMA-bound.
 //
-//   workgroup  4 wavefronts compute a (16*MB)-row x 256-column block of C (MB = 16 or 8); the k loop advances one
-//              packed tile (32 rows of W) at a time through a ring of LDS stages filled by direct global->LDS loads
-//   A          the block's rows x 32 k values of bf16 go to LDS as they lie in memory (64 bytes per row) and are
-//              shared by the 4 wavefronts; a 16-row A operand of v_mfma_f32_16x16x32_bf16 is one ds_read_b128 per lane
-//   W          every wavefront owns 64 columns = 2 packed tiles per k step, staged in the layout of Wfmt and expanded
-//              straight into B operands (byte j of the 8 mantissa words a lane reads = column 4c+j), so the weights
-//              are dequantised exactly once per workgroup and never written back to LDS as bf16
-//   math       per k step a wavefront issues MB x 4 MFMAs (16x16x32) on 4 B operands; the VALU work of building
-//              operand j+1 overlaps the MFMAs of operand j
+// Two kernels share the staging and the weight expansion:
+//   matmul_tile_kernel   4 wavefronts, (32*MB)-row x 256-column block of C; used with MB = 4 (128 rows) when 256-row
+//                        blocks would leave CUs idle or M is not a multiple of 256
+//   matmul_tile8_kernel  8 wavefronts, 256 x 256 block; the two wavefronts of a column group split the weight
+//                        expansion and exchange operands through LDS (described at the kernel)
+//   staging    the k loop advances one packed tile row (32 rows of W) at a time through a ring of LDS stages filled by
+//              direct global->LDS loads
+//   math       v_mfma_f32_32x32x16_bf16, fp32 accumulation
+//   A          the block's rows x 32 k values of bf16 go to LDS as they lie in memory (64 bytes per row, the four
+//              16-byte chunks of a row XOR-swizzled) and are shared by the wavefronts; the A operand of one MFMA
+//              (32 rows x 16 k) is one ds_read_b128 per lane
+//   W          a wavefront's 64 columns = 2 packed tiles per k step, staged in the layout of Wfmt and expanded straight
+//              into B operands, never written back to LDS as packed data.  Lane (c = lane % 32, kh = lane / 32) reads,
+//              for a 16-row slab s of the step, the 8 mantissa words of k rows 16s + 8kh .. + 7 that hold columns
+//              4(c % 16) .. + 3; of each word it uses the two bytes 2(c / 16) and 2(c / 16) + 1: byte cb is its column
+//              in 32-column operand cb.  Which 32 of the 64 columns an operand holds is therefore a permutation that
+//              only the epilogue has to know.
 // Semantics as in bfp_matmul.hip (tt::operations::primary::matmul, tt_eager/tt_dnn/op_library/bmm/bmm_op.hpp:318-346).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -20,6 +28,8 @@
 #include "ttmi_internal.h"
 
 namespace ttmi {
+
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 
 struct TileDev {
     const uint8_t *a;        // bf16
@@ -34,22 +44,57 @@ struct TileDev {
 constexpr int TILE_STAGES = 4;
 constexpr int TILE_COLS = 256;
 
+// One 16-row slab of a staged pair of packed tiles, as read from LDS by one lane, and its expansion.
+struct Slab { uint32_t e[8], words[8]; };
+
+template <int W> __device__ __forceinline__ void read_slab(const uint8_t *lds, uint32_t exp_at, uint32_t mant_at, Slab &s) {
+    using F = Wfmt<W>;
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) s.e[jj] = lds[exp_at + jj];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) s.words[jj] = *reinterpret_cast<const uint32_t *>(lds + mant_at + jj * F::row_bytes);
+}
+
+// Row scales and mantissa-only words of a slab; `half_shift` = 16 * (c / 16) brings this lane's two columns to bytes 0, 1.
+// The scale of a row is its exponent byte moved into the exponent field of a float: 2^(E - 127), i.e. 2^(bias_exp - 127)
+// times too large for every row alike; the epilogue takes that power of two out of the sums again (exactly).  Rows with
+// E = 0 (all zeros or fp32 subnormals, magnitudes below 2^-126) get scale 0.
+template <int W> __device__ __forceinline__ void prepare_slab(Slab &s, int q, uint32_t half_shift, float (&scale)[8], uint32_t (&mags)[8]) {
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(s.e[jj] << 23);
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+        if (W == 7) {
+            s.words[jj] >>= half_shift;
+            mags[jj] = s.words[jj] & 0x7f7fu;
+        } else {
+            // four 4-bit codes -> one code per byte, sign bit moved from bit 3 to bit 7 of its byte
+            uint32_t v = (s.words[jj] >> (16 * (q & 1))) & 0xffffu;
+            v = (v | (v << 8)) & 0x00ff00ffu;
+            v = ((v | (v << 4)) & 0x0f0f0f0fu) >> half_shift;
+            s.words[jj] = v << 4;
+            mags[jj] = v & 0x0707u;
+        }
+    }
+}
+
 template <int W, int ACT, int MB>
 __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
     using F = Wfmt<W>;
-    constexpr int BM = 16 * MB;
+    constexpr int BM = 32 * MB;
     constexpr int A_BYTES = BM * 64;                       // rows x 32 bf16
     constexpr int STAGE_BYTES = A_BYTES + 4 * F::stage_bytes;
     constexpr int NLOAD = F::loads;
-    constexpr int A_LOADS = MB / 4;                        // direct-to-LDS loads of 16 rows each, per wavefront
+    constexpr int A_LOADS = MB / 2;                        // direct-to-LDS loads of 16 rows each, per wavefront
     constexpr int VM_PER_STEP = NLOAD + A_LOADS;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[TILE_STAGES * STAGE_BYTES];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int c = lane & 15, g = lane >> 4;
-    const int t_of_lane = c >> 3, fc = (c >> 2) & 1, q = c & 3;
-    const int h_of_lane = g >> 1, g_low = g & 1;
+    const int c = lane & 31, kh = lane >> 5;                      // MFMA row / column index and k half of this lane
+    const int c16 = c & 15, half = c >> 4;
+    const int t_of_lane = c16 >> 3, fc = (c16 >> 2) & 1, q = c16 & 3;
+    const uint32_t half_shift = 16 * half;
 
     // block coordinates: consecutive workgroups (which land on different XCDs) take different m blocks of the same
     // n block, so each XCD's L2 keeps re-serving one band of A while all of them stream the same weights
@@ -78,8 +123,8 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
     for (int i = 0; i < A_LOADS; ++i) {
         const uint32_t row_in_block = wave * (BM / 4) + i * 16 + (lane >> 2);
         const uint32_t row = min(m0 + row_in_block, p.m - 1);            // rows past M repeat the last row, never stored
-        // the four 16-byte k chunks of a row are stored XOR-swizzled by (row / 4) % 4, so that the 16 lanes of one
-        // ds_read_b128 pass (16 rows, same k chunk) hit 16 different 16-byte bank groups
+        // the four 16-byte k chunks of a row are stored XOR-swizzled by (row / 4) % 4, so that lanes reading the same
+        // k chunk of consecutive rows hit different 16-byte bank groups
         const uint32_t kq = (lane & 3) ^ ((lane >> 4) & 3);
         if (p.a_tiled) a_off[i] = (row >> 5) * p.kt * 2048 + (((row >> 4) & 1) * 2 + (kq >> 1)) * 512 + (row & 15) * 32 + (kq & 1) * 16;
         else a_off[i] = (row * p.k + kq * 8) * 2;
@@ -87,12 +132,15 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
     if (p.a_tiled) { a_base = p.a + (uint64_t)bb * ((p.m + 31) / 32) * p.kt * 2048; a_step = 2048; }
     else { a_base = p.a + (uint64_t)bb * p.m * p.k * 2; a_step = 64; }
 
-    const uint32_t exp_off = A_BYTES + wave * F::stage_bytes + F::exp_base + t_of_lane * 64 + (2 * h_of_lane + fc) * 16 + g_low * 8;
-    const uint32_t mant_off = A_BYTES + wave * F::stage_bytes + (h_of_lane * 4 + t_of_lane * 2 + fc) * F::face_stride +
-                              (g_low * 8) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);
-    const uint32_t a_read_off = c * 64 + ((g ^ ((c >> 2) & 3)) * 16);   // + mb * 1024: this lane's 16 bytes of the A operand
+    // slab s of the step: k rows 16s + 8kh .. + 7 = rows 8kh .. of faces (h = s)
+    const uint32_t exp_off = A_BYTES + wave * F::stage_bytes + F::exp_base + t_of_lane * 64 + fc * 16 + kh * 8;        // + s * 32
+    const uint32_t mant_off = A_BYTES + wave * F::stage_bytes + (t_of_lane * 2 + fc) * F::face_stride +
+                              (kh * 8) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);                                   // + s * 4 * face_stride
+    // A operand of MFMA (row block rb, slab s): row rb*32 + c, 16-byte chunk 2s + kh of that row
+    const uint32_t a_read_off0 = c * 64 + (((0 + kh) ^ ((c >> 2) & 3)) * 16);   // + rb * 2048
+    const uint32_t a_read_off1 = c * 64 + (((2 + kh) ^ ((c >> 2) & 3)) * 16);
 
-    auto fetch = [&](uint32_t stage) {
+    auto fetch = [&](uint32_t stage) __attribute__((always_inline)) {
         uint8_t *base = lds + stage * STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
@@ -106,128 +154,357 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
         wptr += w_step;
     };
 
-    f32x4 acc[MB][4];
+    f32x16 acc[MB][2];                                 // [32-row block][32-column operand]
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int rb = 0; rb < MB; ++rb)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[mb][j][r] = 0.f;
+            for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.f;
 
     // Ring: k step i lives in stage i % TILE_STAGES and is requested TILE_STAGES - 1 steps ahead.  The loop is
     // software-pipelined inside the wavefront: while the MFMAs of step i run, the weights of step i+1 are expanded
     // into the other set of B operand registers.  Per iteration i:
     //   wait until this wavefront's share of step i+1 has landed; barrier (now every share of step i+1 has landed and
     //   every wavefront has finished reading step i-1, whose stage is refilled); read the packed words of step i+1;
-    //   then for each 16-row block: read its A operand of step i from LDS (a window of A_WINDOW is kept in flight),
-    //   issue its 4 MFMAs, and after every fourth of the blocks build one B operand of step i+1.
+    //   then for each slab and 32-row block: read its A operand of step i from LDS (a window of them is kept in
+    //   flight), issue its 2 MFMAs, and in between build the B operands of step i+1.
     const uint32_t total = p.kt;
     uint32_t requested = 0;
     for (; requested < total && requested < TILE_STAGES - 1; ++requested) fetch(requested);
 
-    constexpr int A_WINDOW = 8;
-    bf16x8 bop[2][4];
-    StagedWords sw;
+    bf16x8 bop[2][2][2];               // [buffer][slab][operand]
+    Slab slab[2];
     uint32_t stage = 0, step = 0;      // the k step being multiplied and its stage
-    auto wait_for_step = [&](uint32_t which) {       // vector-memory operations complete in order
+    auto wait_for_step = [&](uint32_t which) __attribute__((always_inline)) {       // vector-memory operations complete in order
         const uint32_t ahead = requested - which - 1;
         if (ahead >= 2) wait_vmcnt<2 * VM_PER_STEP>();
         else if (ahead == 1) wait_vmcnt<VM_PER_STEP>();
         else wait_vmcnt<0>();
     };
+    auto expand = [&](auto buf, auto which_slab) __attribute__((always_inline)) {
+        constexpr int B = decltype(buf)::value, S = decltype(which_slab)::value;
+        float scale[8]; uint32_t mags[8];
+        prepare_slab<W>(slab[S], q, half_shift, scale, mags);
+        bop[B][S][0] = weights_operand8<0>(slab[S].words, mags, scale);
+        bop[B][S][1] = weights_operand8<1>(slab[S].words, mags, scale);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
     // prologue: operands of step 0
     wait_for_step(0);
     __syncthreads();
-    read_staged<W>(lds, exp_off, mant_off, sw);
-    {
-        float scale[8]; uint32_t mags[8];
-        prepare_staged<W>(sw, q, scale, mags);
-        bop[0][0] = weights_operand8<0>(sw.words, mags, scale);
-        bop[0][1] = weights_operand8<1>(sw.words, mags, scale);
-        bop[0][2] = weights_operand8<2>(sw.words, mags, scale);
-        bop[0][3] = weights_operand8<3>(sw.words, mags, scale);
-    }
-    auto iteration = [&](auto cur_buf, auto has_next) {
+    read_slab<W>(lds, exp_off, mant_off, slab[0]);
+    read_slab<W>(lds, exp_off + 32, mant_off + 4 * F::face_stride, slab[1]);
+    expand(I0{}, I0{});
+    expand(I0{}, I1{});
+
+    auto iteration = [&](auto cur_buf, auto has_next) __attribute__((always_inline)) {
         constexpr int C = decltype(cur_buf)::value, N = 1 - C;
         constexpr bool more = decltype(has_next)::value;
         const uint32_t next_stage = stage + 1 == TILE_STAGES ? 0 : stage + 1;
-        const uint32_t a_at = stage * STAGE_BYTES + a_read_off;
+        const uint32_t a_at0 = stage * STAGE_BYTES + a_read_off0, a_at1 = stage * STAGE_BYTES + a_read_off1;
         if (more) {
             wait_for_step(step + 1);
+            // a bare barrier: __syncthreads() would also wait for every direct-to-LDS load still in flight (its
+            // fence counts them as memory operations of this workgroup), and the ring lives on keeping them in flight
             __builtin_amdgcn_s_waitcnt(0xC07F);   // our LDS reads of the previous step have returned
-            __syncthreads();
+            __builtin_amdgcn_s_barrier();
             if (requested < total) { fetch(stage == 0 ? TILE_STAGES - 1 : stage - 1); ++requested; }
         }
-        bf16x8 aop[A_WINDOW];
+        // A operands in order of use: (slab 0, rb 0..MB-1), (slab 1, rb 0..MB-1); AW of them in flight
+        constexpr int AW = 4, NA = 2 * MB;
+        bf16x8 aop[AW];
+        auto a_addr = [&](int i) { return (i < MB ? a_at0 : a_at1) + (uint32_t)(i % MB) * 2048u; };
 #pragma unroll
-        for (int mb = 0; mb < A_WINDOW; ++mb) aop[mb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + a_at + mb * 1024));
-        if (more) read_staged<W>(lds, next_stage * STAGE_BYTES + exp_off, next_stage * STAGE_BYTES + mant_off, sw);
-        float scale[8]; uint32_t mags[8];
+        for (int i = 0; i < AW; ++i) aop[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + a_addr(i)));
+        if (more) {
+            read_slab<W>(lds, next_stage * STAGE_BYTES + exp_off, next_stage * STAGE_BYTES + mant_off, slab[0]);
+            read_slab<W>(lds, next_stage * STAGE_BYTES + exp_off + 32, next_stage * STAGE_BYTES + mant_off + 4 * F::face_stride, slab[1]);
+        }
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[mb][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[mb % A_WINDOW], bop[C][j], acc[mb][j], 0, 0, 0);
-            if (mb + A_WINDOW < MB) aop[mb % A_WINDOW] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + a_at + (mb + A_WINDOW) * 1024));
+        for (int i = 0; i < NA; ++i) {
+            const int s = i / MB, rb = i % MB;
+            acc[rb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aop[i % AW], bop[C][s][0], acc[rb][0], 0, 0, 0);
+            acc[rb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aop[i % AW], bop[C][s][1], acc[rb][1], 0, 0, 0);
+            if (i + AW < NA) aop[i % AW] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + a_addr(i + AW)));
             if (more) {
-                constexpr int every = MB / 4;          // one operand of the next step per MB/4 row blocks
-                if (mb == 0) prepare_staged<W>(sw, q, scale, mags);
-                if (mb == every - 1) bop[N][0] = weights_operand8<0>(sw.words, mags, scale);
-                if (mb == 2 * every - 1) bop[N][1] = weights_operand8<1>(sw.words, mags, scale);
-                if (mb == 3 * every - 1) bop[N][2] = weights_operand8<2>(sw.words, mags, scale);
-                if (mb == 4 * every - 1) bop[N][3] = weights_operand8<3>(sw.words, mags, scale);
+                if (i == NA / 4) expand(std::integral_constant<int, N>{}, I0{});
+                if (i == (3 * NA) / 4) expand(std::integral_constant<int, N>{}, I1{});
             }
         }
         stage = next_stage;
         ++step;
     };
-    using Buf0 = std::integral_constant<int, 0>;
-    using Buf1 = std::integral_constant<int, 1>;
     // pairs of steps that both have a successor, then the last one or two steps; no branch inside a step touches
     // the accumulators
 #pragma unroll 1
     while (step + 2 < total) {
-        iteration(Buf0{}, std::true_type{});
-        iteration(Buf1{}, std::true_type{});
+        iteration(I0{}, std::true_type{});
+        iteration(I1{}, std::true_type{});
     }
     if (total - step == 2) {
-        iteration(Buf0{}, std::true_type{});
-        iteration(Buf1{}, std::false_type{});
+        iteration(I0{}, std::true_type{});
+        iteration(I1{}, std::false_type{});
     } else {
-        iteration(Buf0{}, std::false_type{});
+        iteration(I0{}, std::false_type{});
     }
 
-    // ---- epilogue: lane holds rows mb*16 + 4g + r, columns 4c .. 4c+3 of its wavefront's 64 ------------------
+    // ---- epilogue: acc[rb][cb][i] is row rb*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the wavefront's 64
     if (t_of_lane >= (int)n_valid) return;
-    const uint32_t n_col = (nt0 + t_of_lane) * 32 + fc * 16 + q * 4;
-    float bias_v[4] = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t col_in_tile = fc * 16 + q * 4 + half * 2;
+    const uint32_t n_col = (nt0 + t_of_lane) * 32 + col_in_tile;
+    float bias_v[2] = {0.f, 0.f};
     if (p.bias) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bias_v[j] = __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
+        for (int cb = 0; cb < 2; ++cb) bias_v[cb] = __uint_as_float((uint32_t)p.bias[n_col + cb] << 16);
     }
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
+    for (int rb = 0; rb < MB; ++rb) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t row = m0 + mb * 16 + g * 4 + r;
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t row = m0 + rb * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
             if (row >= p.m) continue;
-            float v[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = apply_activation<ACT>(acc[mb][j][r] + bias_v[j]);
+            constexpr float unscale = 1.0f / (float)(1u << (F::bias_exp - 127));      // see prepare_slab
+            const float v0 = apply_activation<ACT>(acc[rb][0][i] * unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * unscale + bias_v[1]);
             uint64_t elem;
             if (p.c_tiled) {
                 const uint64_t tile = ((uint64_t)bb * ((p.m + 31) / 32) + (row >> 5)) * p.nt + nt0 + t_of_lane;
-                elem = tile * 1024 + (((row >> 4) & 1) * 2 + fc) * 256 + (row & 15) * 16 + q * 4;
+                elem = tile * 1024 + (((row >> 4) & 1) * 2 + fc) * 256 + (row & 15) * 16 + q * 4 + half * 2;
             } else {
                 elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
             }
             if (p.c_f32) {
-                *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<float2 *>(p.c + elem * 4) = make_float2(v0, v1);
             } else {
-                const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
-                const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
-                *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
+                *reinterpret_cast<uint32_t *>(p.c + elem * 2) = f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
             }
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// 256 x 256 block with EIGHT wavefronts (two per SIMD).  A single wavefront per SIMD cannot issue the weight
+// expansion and the MFMAs of a 256-row block fast enough; two can, if the expansion is not done twice.  Wavefront
+// (wc = w % 4, wr = w / 4) owns rows 128*wr .. +127 and columns 64*wc .. +63 of the block.  The two wavefronts of a
+// column group share the work of expanding its weights: wr expands slab wr (k rows 16*wr .. +15) of the NEXT k step
+// into bf16 B operands and leaves them in LDS, exactly as its lanes would hold them in registers; after the step's
+// barrier both read all four operands of the group (2 slabs x 2 operands, one ds_read_b128 each).
+//   LDS   ring of TILE_STAGES stages [A: 256 rows x 64 B][packed W: 4 column groups], then two operand buffers
+//         [column group][slab][operand][lane] x 16 B (step parity)
+//   step  wait for the own direct-to-LDS loads of step i+1, barrier, request step i+3, then interleaved:
+//         (a) operands of step i and A from LDS -> 16 MFMAs (32x32x16), (b) expand slab wr of step i+1 -> LDS
+template <int W, int ACT>
+__global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
+    using F = Wfmt<W>;
+    constexpr int MB = 4;                                  // 32-row blocks per wavefront
+    constexpr int A_BYTES = 256 * 64;
+    constexpr int STAGE_BYTES = A_BYTES + 4 * F::stage_bytes;
+    constexpr int OPS_BYTES = 4 * 2 * 2 * 64 * 16;         // one operand buffer
+    constexpr int OPS_BASE = TILE_STAGES * STAGE_BYTES;
+    constexpr int NLOAD = F::loads;
+    constexpr int W_LOADS0 = (NLOAD + 1) / 2, W_LOADS1 = NLOAD - W_LOADS0;   // packed-weight loads issued by wr = 0 / wr = 1
+    constexpr int A_LOADS = 2;                             // 16 loads of 16 rows each over 8 wavefronts
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[OPS_BASE + 2 * OPS_BYTES];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wc = wave & 3, wr = wave >> 2;
+    const int c = lane & 31, kh = lane >> 5;
+    const int c16 = c & 15, half = c >> 4;
+    const int t_of_lane = c16 >> 3, fc = (c16 >> 2) & 1, q = c16 & 3;
+    const uint32_t half_shift = 16 * half;
+
+    uint32_t idx = blockIdx.x;
+    const uint32_t tm = idx % p.tiles_m; idx /= p.tiles_m;
+    const uint32_t tn = idx % p.tiles_n;
+    const uint32_t bb = idx / p.tiles_n;
+    const uint32_t m0 = tm * 256;
+    const uint32_t nt0 = tn * (TILE_COLS / 32) + wc * 2;               // first packed tile column of this column group
+    const uint32_t n_valid = nt0 >= p.nt ? 0u : min(2u, p.nt - nt0);
+
+    // ---- direct-to-LDS loads of this wavefront ---------------------------------------------------------------
+    uint32_t chunk_of[NLOAD], src_off[NLOAD];
+    stage_chunks<W>(lane, chunk_of);
+    const uint32_t chunks_valid = (n_valid ? n_valid : 1u) * F::chunks;
+#pragma unroll
+    for (int l = 0; l < NLOAD; ++l) src_off[l] = min(chunk_of[l], chunks_valid - 1) * 16;
+    const uint32_t nt_src = n_valid ? nt0 : 0u;
+    const uint8_t *wptr = p.b + ((uint64_t)(p.b_batch == 1 ? 0 : bb) * p.kt * p.nt + nt_src) * F::tile_bytes;
+    const uint64_t w_step = (uint64_t)p.nt * F::tile_bytes;
+    uint32_t a_off[A_LOADS];
+    const uint8_t *a_base;
+    uint32_t a_step;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const uint32_t row_in_block = wave * 32 + i * 16 + (lane >> 2);
+        const uint32_t row = min(m0 + row_in_block, p.m - 1);
+        const uint32_t kq = (lane & 3) ^ ((lane >> 4) & 3);              // XOR swizzle of the row's four 16-byte chunks
+        if (p.a_tiled) a_off[i] = (row >> 5) * p.kt * 2048 + (((row >> 4) & 1) * 2 + (kq >> 1)) * 512 + (row & 15) * 32 + (kq & 1) * 16;
+        else a_off[i] = (row * p.k + kq * 8) * 2;
+    }
+    if (p.a_tiled) { a_base = p.a + (uint64_t)bb * ((p.m + 31) / 32) * p.kt * 2048; a_step = 2048; }
+    else { a_base = p.a + (uint64_t)bb * p.m * p.k * 2; a_step = 64; }
+
+    auto fetch = [&](uint32_t stage) __attribute__((always_inline)) {
+        uint8_t *base = lds + stage * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(a_base + a_off[i]),
+                                             (__attribute__((address_space(3))) void *)(base + (wave * 32 + i * 16) * 64), 16, 0, 0);
+        if (wr == 0) {
+#pragma unroll
+            for (int l = 0; l < W_LOADS0; ++l)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[l]),
+                                                 (__attribute__((address_space(3))) void *)(base + A_BYTES + wc * F::stage_bytes + l * 1024), 16, 0, 0);
+        } else {
+#pragma unroll
+            for (int l = W_LOADS0; l < NLOAD; ++l)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[l]),
+                                                 (__attribute__((address_space(3))) void *)(base + A_BYTES + wc * F::stage_bytes + l * 1024), 16, 0, 0);
+        }
+        a_base += a_step;
+        wptr += w_step;
+    };
+
+    // the slab this wavefront expands: slab wr = faces (h = wr), k rows 8kh .. of them
+    const uint32_t exp_off = A_BYTES + wc * F::stage_bytes + F::exp_base + t_of_lane * 64 + fc * 16 + kh * 8 + wr * 32;
+    const uint32_t mant_off = A_BYTES + wc * F::stage_bytes + (wr * 4 + t_of_lane * 2 + fc) * F::face_stride +
+                              (kh * 8) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);
+    const uint32_t ops_write_off = OPS_BASE + ((wc * 2 + wr) * 2) * 1024 + lane * 16;         // + parity * OPS_BYTES, + operand * 1024
+    const uint32_t ops_partner_off = OPS_BASE + ((wc * 2 + (1 - wr)) * 2) * 1024 + lane * 16;  // the other slab's operands
+    // A operand of MFMA (row block rb, slab s): row wr*128 + rb*32 + c, 16-byte chunk 2s + kh of that row (+ rb * 2048)
+    const uint32_t a_own_off = (wr * 128 + c) * 64 + (((2 * wr + kh) ^ ((c >> 2) & 3)) * 16);
+    const uint32_t a_partner_off = (wr * 128 + c) * 64 + (((2 * (1 - wr) + kh) ^ ((c >> 2) & 3)) * 16);
+
+    f32x16 acc[MB][2];
+#pragma unroll
+    for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.f;
+
+    const uint32_t total = p.kt;
+    uint32_t requested = 0;
+    for (; requested < total && requested < TILE_STAGES - 1; ++requested) fetch(requested);
+
+    uint32_t stage = 0, step = 0;
+    auto wait_for_step = [&](uint32_t which) __attribute__((always_inline)) {       // vector-memory operations complete in order
+        const uint32_t ahead = which < requested ? requested - which - 1 : 0;
+        if (wr == 0) {
+            constexpr int VM = A_LOADS + W_LOADS0;
+            if (ahead >= 2) wait_vmcnt<2 * VM>(); else if (ahead == 1) wait_vmcnt<VM>(); else wait_vmcnt<0>();
+        } else {
+            constexpr int VM = A_LOADS + W_LOADS1;
+            if (ahead >= 2) wait_vmcnt<2 * VM>(); else if (ahead == 1) wait_vmcnt<VM>(); else wait_vmcnt<0>();
+        }
+    };
+    // Expands slab wr of the step in `from_stage`: the operands stay in registers for this wavefront and go to operand
+    // buffer `parity` for the other wavefront of the column group.
+    auto expand = [&](uint32_t from_stage, uint32_t parity, bf16x8 (&ops)[2]) __attribute__((always_inline)) {
+        Slab slab;
+        read_slab<W>(lds, from_stage * STAGE_BYTES + exp_off, from_stage * STAGE_BYTES + mant_off, slab);
+        float scale[8]; uint32_t mags[8];
+        prepare_slab<W>(slab, q, half_shift, scale, mags);
+        ops[0] = weights_operand8<0>(slab.words, mags, scale);
+        ops[1] = weights_operand8<1>(slab.words, mags, scale);
+        *reinterpret_cast<u32x4 *>(lds + parity * OPS_BYTES + ops_write_off) = __builtin_bit_cast(u32x4, ops[0]);
+        *reinterpret_cast<u32x4 *>(lds + parity * OPS_BYTES + ops_write_off + 1024) = __builtin_bit_cast(u32x4, ops[1]);
+    };
+    auto read_a = [&](uint32_t from_stage, uint32_t off, bf16x8 (&a)[MB]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int rb = 0; rb < MB; ++rb)
+            a[rb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + from_stage * STAGE_BYTES + off + (uint32_t)rb * 2048u));
+    };
+
+    // prologue: own operands and own-slab A of step 0
+    bf16x8 own[2], a_own[MB];
+    wait_for_step(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    expand(0, 0, own);
+    read_a(0, a_own_off, a_own);
+
+    // One k step.  Everything the first eight MFMAs need (own-slab operands, own-slab A) is already in registers when
+    // the barrier opens; the other slab's operands and A arrive from LDS while those MFMAs run.  Then this
+    // wavefront's slab of the next step is expanded, the second eight MFMAs follow, and the own-slab A of the next
+    // step (in LDS since the barrier) is read ahead.
+    auto iteration = [&](auto has_next) __attribute__((always_inline)) {
+        constexpr bool more = decltype(has_next)::value;
+        const uint32_t next_stage = stage + 1 == TILE_STAGES ? 0 : stage + 1;
+        const uint32_t parity = step & 1;
+        if (more) wait_for_step(step + 1);
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // our LDS reads and operand writes of the previous step are done
+        __builtin_amdgcn_s_barrier();
+        if (more && requested < total) { fetch(stage == 0 ? TILE_STAGES - 1 : stage - 1); ++requested; }
+        bf16x8 part[2], a_part[MB];
+        part[0] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + parity * OPS_BYTES + ops_partner_off));
+        part[1] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + parity * OPS_BYTES + ops_partner_off + 1024));
+        read_a(stage, a_partner_off, a_part);
+#pragma unroll
+        for (int rb = 0; rb < MB; ++rb) {
+            acc[rb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_own[rb], own[0], acc[rb][0], 0, 0, 0);
+            acc[rb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_own[rb], own[1], acc[rb][1], 0, 0, 0);
+        }
+        bf16x8 next_own[2];
+        if (more) expand(next_stage, parity ^ 1, next_own);
+#pragma unroll
+        for (int rb = 0; rb < MB; ++rb) {
+            acc[rb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_part[rb], part[0], acc[rb][0], 0, 0, 0);
+            acc[rb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_part[rb], part[1], acc[rb][1], 0, 0, 0);
+        }
+        if (more) {
+            read_a(next_stage, a_own_off, a_own);
+            own[0] = next_own[0]; own[1] = next_own[1];
+        }
+        stage = next_stage;
+        ++step;
+    };
+#pragma unroll 1
+    while (step + 1 < total) iteration(std::true_type{});
+    iteration(std::false_type{});
+
+    // ---- epilogue: acc[rb][cb][i] is row wr*128 + rb*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the group's 64
+    if (t_of_lane >= (int)n_valid) return;
+    const uint32_t col_in_tile = fc * 16 + q * 4 + half * 2;
+    const uint32_t n_col = (nt0 + t_of_lane) * 32 + col_in_tile;
+    float bias_v[2] = {0.f, 0.f};
+    if (p.bias) {
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) bias_v[cb] = __uint_as_float((uint32_t)p.bias[n_col + cb] << 16);
+    }
+#pragma unroll
+    for (int rb = 0; rb < MB; ++rb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t row = m0 + wr * 128 + rb * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
+            if (row >= p.m) continue;
+            constexpr float unscale = 1.0f / (float)(1u << (F::bias_exp - 127));      // see prepare_slab
+            const float v0 = apply_activation<ACT>(acc[rb][0][i] * unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * unscale + bias_v[1]);
+            uint64_t elem;
+            if (p.c_tiled) {
+                const uint64_t tile = ((uint64_t)bb * ((p.m + 31) / 32) + (row >> 5)) * p.nt + nt0 + t_of_lane;
+                elem = tile * 1024 + (((row >> 4) & 1) * 2 + fc) * 256 + (row & 15) * 16 + q * 4 + half * 2;
+            } else {
+                elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
+            }
+            if (p.c_f32) {
+                *reinterpret_cast<float2 *>(p.c + elem * 4) = make_float2(v0, v1);
+            } else {
+                *reinterpret_cast<uint32_t *>(p.c + elem * 2) = f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
+            }
+        }
+    }
+}
+
+template <int W>
+static void launch_tile8_act(const TileDev &p, int activation, uint32_t blocks, hipStream_t st) {
+    switch (activation) {
+        case TTMI_ACT_RELU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_RELU>), dim3(blocks), dim3(512), 0, st, p); break;
+        case TTMI_ACT_GELU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_GELU>), dim3(blocks), dim3(512), 0, st, p); break;
+        case TTMI_ACT_SILU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_SILU>), dim3(blocks), dim3(512), 0, st, p); break;
+        default: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_NONE>), dim3(blocks), dim3(512), 0, st, p); break;
     }
 }
 
@@ -266,11 +543,11 @@ int matmul_bfp_tiled(const MatmulArgs &x, hipStream_t st) {
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
     if (x.b_fmt == TTMI_BFLOAT8_B) {
-        if (use_256) launch_tile_act<7, 16>(p, x.activation, (uint32_t)blocks, st);
-        else launch_tile_act<7, 8>(p, x.activation, (uint32_t)blocks, st);
+        if (use_256) launch_tile8_act<7>(p, x.activation, (uint32_t)blocks, st);
+        else launch_tile_act<7, 4>(p, x.activation, (uint32_t)blocks, st);
     } else {
-        if (use_256) launch_tile_act<3, 16>(p, x.activation, (uint32_t)blocks, st);
-        else launch_tile_act<3, 8>(p, x.activation, (uint32_t)blocks, st);
+        if (use_256) launch_tile8_act<3>(p, x.activation, (uint32_t)blocks, st);
+        else launch_tile_act<3, 4>(p, x.activation, (uint32_t)blocks, st);
     }
     return check_launch("matmul_tile_kernel");
 }
