@@ -45,15 +45,18 @@ template <int LPR> __device__ __forceinline__ uint32_t row_max(uint32_t v) {
     return v;
 }
 
+// Code of one element (tt_metal/common/bfloat8.hpp:23-87, blockfloat_common.hpp:67-147): hidden one OR-ed in even
+// for a zero exponent field, truncating shift by the exponent gap, round half up, saturate, sign dropped when the
+// mantissa rounds to zero, +-0 -> 0.  The two shifts are folded into one:
+//     ((m >> gap) + h) >> s  ==  (m + (h << gap)) >> (gap + s)        (h = 2^(s-1), s = 24 - W)
+// and every gap above 31 - s gives 0 either way (m < 2^24), so the gap is clamped there and nothing overflows.
 template <int W> __device__ __forceinline__ uint32_t to_code(uint32_t bits, uint32_t shared) {
-    const uint32_t mag = bits & 0x7fffffffu;
-    const uint32_t gap = shared - (mag >> 23);
-    uint32_t m = (bits & 0x007fffffu) | 0x00800000u;   // hidden one, also for a zero exponent field
-    m = gap > 31u ? 0u : (m >> gap);                   // truncating pre-shift
-    m = (m + (1u << (23 - W))) >> (24 - W);            // round half up
-    m = m > ((1u << W) - 1u) ? ((1u << W) - 1u) : m;   // saturate, no carry into the exponent
-    const uint32_t code = m ? (((bits >> 31) << W) | m) : 0u;
-    return mag ? code : 0u;
+    constexpr uint32_t s = 24 - W, h = 1u << (s - 1), top = (1u << W) - 1u;
+    const uint32_t gap = min(shared - ((bits >> 23) & 0xffu), 31u - s);
+    const uint32_t m24 = (bits & 0x007fffffu) | 0x00800000u;
+    uint32_t m = min(((h << gap) + m24) >> (gap + s), top);
+    m = (bits & 0x7fffffffu) ? m : 0u;
+    return m ? (((bits >> 31) << W) | m) : 0u;
 }
 
 template <int W> __device__ __forceinline__ uint32_t from_code(uint32_t code, uint32_t shared) {
@@ -176,6 +179,7 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
 #pragma unroll
         for (int e = 0; e < EPL; ++e) { const uint32_t f = bits[e] & 0x7f800000u; top = f > top ? f : top; }
         const uint32_t shared = row_max<LPR>(top) >> 23;
+        const bool tiny_rows = MODE == SRC_TENSOR && __ballot(shared < (uint32_t)W) != 0;
         uint32_t lo = 0, hi = 0;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
@@ -183,7 +187,8 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
             // from_torch runs pack -> unpack -> tilize -> pack (tt_eager/tensor/tensor_impl.cpp:179-197).  A code
             // whose mantissa is the single bit 2^(W-1-E) unpacks to exponent field 0 with a zero fraction, i.e.
             // to +-0, and the second pack turns that into code 0; every other code survives the round trip.
-            if (MODE == SRC_TENSOR && shared < (uint32_t)W && (code & ((1u << W) - 1u)) == (1u << ((W - 1 - shared) & 31u))) code = 0;
+            // Only rows with E < W (magnitudes below 2^-120) can be hit: a wavefront-wide detour.
+            if (MODE == SRC_TENSOR && tiny_rows && shared < (uint32_t)W && (code & ((1u << W) - 1u)) == (1u << ((W - 1 - shared) & 31u))) code = 0;
             const int sh = (W + 1) * e;
             if (sh < 32) lo |= code << sh; else hi |= code << (sh - 32);
         }

@@ -24,6 +24,7 @@ template <> struct Wfmt<7> {
     static constexpr int exp_base = 8 * face_stride;                        // 2176
     static constexpr int loads = 3, stage_bytes = loads * 1024;
     static constexpr int bias_exp = 133;                                    // value = mantissa * 2^(E - 133)
+    static constexpr float unscale = 1.0f / 64.0f;                          // 2^(127 - bias_exp)
 };
 template <> struct Wfmt<3> {
     static constexpr int tile_bytes = 576, chunks = 36, row_bytes = 8;
@@ -31,6 +32,7 @@ template <> struct Wfmt<3> {
     static constexpr int exp_base = 8 * face_stride;                        // 1152
     static constexpr int loads = 2, stage_bytes = loads * 1024;
     static constexpr int bias_exp = 129;                                    // value = mantissa * 2^(E - 129)
+    static constexpr float unscale = 1.0f / 4.0f;                           // 2^(127 - bias_exp)
 };
 
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
@@ -106,43 +108,6 @@ template <int W> __device__ __forceinline__ void stage_chunks(int lane, uint32_t
     }
 }
 
-// The same expansion in separate steps, for kernels that overlap it with MFMAs of the previous k step:
-// read_staged issues the LDS reads, prepare_staged (once they have returned) derives the row scales and the
-// mantissa-only words, after which weights_operand8<j>(words, mags, scale) builds operand j.
-struct StagedWords { uint32_t e[8], words[8]; };
-
-template <int W> __device__ __forceinline__ void read_staged(const uint8_t *lds, uint32_t exp_at, uint32_t mant_at, StagedWords &s) {
-    using F = Wfmt<W>;
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) s.e[jj] = lds[exp_at + jj];
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) s.words[jj] = *reinterpret_cast<const uint32_t *>(lds + mant_at + jj * F::row_bytes);
-}
-
-template <int W> __device__ __forceinline__ void prepare_staged(StagedWords &s, int q, float (&scale)[8], uint32_t (&mags)[8]) {
-    using F = Wfmt<W>;
-    const uint32_t e_min = min(min(min(s.e[0], s.e[1]), min(s.e[2], s.e[3])), min(min(s.e[4], s.e[5]), min(s.e[6], s.e[7])));
-    if (__builtin_expect(__ballot(e_min < (uint32_t)(F::bias_exp - 126)) != 0, 0)) {
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) scale[jj] = __builtin_amdgcn_ldexpf(1.0f, (int)s.e[jj] - F::bias_exp);
-    } else {
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float((s.e[jj] << 23) - ((uint32_t)(F::bias_exp - 127) << 23));
-    }
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) {
-        if (W == 7) {
-            mags[jj] = s.words[jj] & 0x7f7f7f7fu;
-        } else {
-            uint32_t v = (s.words[jj] >> (16 * (q & 1))) & 0xffffu;
-            v = (v | (v << 8)) & 0x00ff00ffu;
-            v = (v | (v << 4)) & 0x0f0f0f0fu;
-            s.words[jj] = v << 4;
-            mags[jj] = v & 0x07070707u;
-        }
-    }
-}
-
 // The four bf16 B operands (columns 4c+0..3 of a 64-column group, k rows 8g..8g+7) of lane (c = lane % 16,
 // g = lane / 16) from a staged pair of packed tiles.  exp_at / mant_at: this lane's LDS byte addresses of the
 // exponents and mantissa words in stage 0 (see Wfmt); q = c % 4.  `after_lds_reads` runs once every LDS read has
@@ -170,17 +135,12 @@ __device__ __forceinline__ void staged_operands(uint32_t exp_at, uint32_t mant_a
     words[0] = w01[0]; words[1] = w01[1]; words[2] = w23[0]; words[3] = w23[1];
     words[4] = w45[0]; words[5] = w45[1]; words[6] = w67[0]; words[7] = w67[1];
     after_lds_reads();
-    // scale of row jj = 2^(E - bias_exp).  Writing the exponent field directly needs E - bias_exp + 127 >= 1;
-    // a wavefront that meets a smaller exponent (magnitudes below ~2^-120) takes v_ldexp_f32 instead.
-    const uint32_t e_min = min(min(min(e[0], e[1]), min(e[2], e[3])), min(min(e[4], e[5]), min(e[6], e[7])));
+    // The scale of row jj is its exponent byte moved into the exponent field of a float: 2^(E - 127), that is
+    // 2^(bias_exp - 127) times too large for every row alike; whoever stores the sums takes that power of two out
+    // again (exactly, see Wfmt::unscale).  Rows with E = 0 (all zeros, or fp32 subnormals below 2^-126) get scale 0.
     float scale[8];
-    if (__builtin_expect(__ballot(e_min < (uint32_t)(F::bias_exp - 126)) != 0, 0)) {
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) scale[jj] = __builtin_amdgcn_ldexpf(1.0f, (int)e[jj] - F::bias_exp);
-    } else {
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float((e[jj] << 23) - ((uint32_t)(F::bias_exp - 127) << 23));
-    }
+    for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(e[jj] << 23);
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) {
         if (W == 7) {

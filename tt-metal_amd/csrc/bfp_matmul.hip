@@ -353,7 +353,7 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
                 float v[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    float x = mine[r][j];
+                    float x = mine[r][j] * F::unscale;
                     if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
                     v[j] = apply_activation<ACT>(x);
                 }

@@ -265,8 +265,7 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
         for (int i = 0; i < 16; ++i) {
             const uint32_t row = m0 + rb * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
             if (row >= p.m) continue;
-            constexpr float unscale = 1.0f / (float)(1u << (F::bias_exp - 127));      // see prepare_slab
-            const float v0 = apply_activation<ACT>(acc[rb][0][i] * unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * unscale + bias_v[1]);
+            const float v0 = apply_activation<ACT>(acc[rb][0][i] * F::unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * F::unscale + bias_v[1]);
             uint64_t elem;
             if (p.c_tiled) {
                 const uint64_t tile = ((uint64_t)bb * ((p.m + 31) / 32) + (row >> 5)) * p.nt + nt0 + t_of_lane;
@@ -480,8 +479,7 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
         for (int i = 0; i < 16; ++i) {
             const uint32_t row = m0 + wr * 128 + rb * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
             if (row >= p.m) continue;
-            constexpr float unscale = 1.0f / (float)(1u << (F::bias_exp - 127));      // see prepare_slab
-            const float v0 = apply_activation<ACT>(acc[rb][0][i] * unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * unscale + bias_v[1]);
+            const float v0 = apply_activation<ACT>(acc[rb][0][i] * F::unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * F::unscale + bias_v[1]);
             uint64_t elem;
             if (p.c_tiled) {
                 const uint64_t tile = ((uint64_t)bb * ((p.m + 31) / 32) + (row >> 5)) * p.nt + nt0 + t_of_lane;
