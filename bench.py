@@ -27,6 +27,16 @@ for _p in (ROOT, os.path.join(ROOT, "tt-metal_amd")):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 ROTATE_BYTES = 512 << 20
+# HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, on this same command;
+# summary and scaling factors in profiles/bench_all_workloads_hbm_traffic.md).  Counters cannot be read from inside
+# this process, so the figures of that run are carried here; None where the run could not tell two launches apart.
+MEASURED_TRAFFIC_BYTES = {
+    "falcon_h_to_4h": 103_258_000, "falcon_4h_to_h": 115_897_000, "mistral_qkv": None, "mistral_o": None,
+    "mistral_gate": 48_660_000, "mistral_up": 48_660_000, "mistral_down": 53_066_000,
+    "prefill_ff1": 591_831_000, "bert_bmm": 87_922_000,
+    "pack_bfp4_4k_pack": 76_677_000, "pack_bfp4_4k_unpack": 76_642_000,
+    "pack_bfp8_1k_pack": 5_446_000 * 1024 // 1000, "pack_bfp8_1k_unpack": 5_276_000 * 1024 // 1000,
+}
 WORKLOAD_NAMES = {
     "decode_falcon": "decode_falcon: bf16 [32,4544] x BFP8_B [4544,18176], then [32,18176] x BFP8_B [18176,4544] (Falcon-7B decode MLP)",
     "decode_mistral": "decode_mistral: M=32 bf16 x fused QKV / O (BFP8_B) and gate / up / down (BFP4_B) of a Mistral-7B layer",
@@ -299,6 +309,9 @@ def main():
                    "sample": f"oracle from_torch + to_torch host sequences on fp32 {list(x.shape)}",
                    "from_torch_pack_melem_s_1thread": round(x.size / t_pack / 1e6, 1),
                    "to_torch_unpack_melem_s_1thread": round(x.size / t_unpack / 1e6, 1)}
+
+    for leg in (l for wl in order for l in results[wl]):
+        leg["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(leg["workload"])
 
     line = {
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,

@@ -395,8 +395,9 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     d.ngroups = (d.nt + GROUP_TILES - 1) / GROUP_TILES;
     d.groups = (uint64_t)batch * d.mt * d.ngroups;
     d.units = d.groups * d.kt;
-    // workgroups in flight at once: 256 CUs x 3 workgroups of 4 wavefronts measured best (4 fit)
-    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", 768);
+    // workgroups to aim for: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone nearly get there,
+    // x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot reset)
+    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", d.groups >= 256 ? 768 : 512);
     if (env_u32("TTMI_MATMUL_STREAMK", 0)) {
         d.split = 0;
         d.workgroups = (uint32_t)(d.units < resident ? d.units : resident);
