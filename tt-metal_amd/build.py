@@ -70,5 +70,25 @@ def build(force: bool = False, verbose: bool = False) -> str:
     return LIB
 
 
+def build_bindings(force: bool = False, verbose: bool = False) -> str:
+    """Builds the pybind11 module tt-metal_amd/lib/_ttmi*.so (host C++ only; links libttmi.so next to it)."""
+    import sysconfig
+
+    import pybind11
+
+    build(force=False, verbose=verbose)
+    src = os.path.join(CSRC, "ttmi_pybind.cpp")
+    out = os.path.join(LIB_DIR, "_ttmi" + sysconfig.get_config_var("EXT_SUFFIX"))
+    if force or _stale(out, [src, os.path.join(ROOT, "include", "ttmi.h"), LIB]):
+        cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
+               "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"], "-I", os.path.join(ROOT, "include"),
+               src, "-o", out, "-L", LIB_DIR, "-lttmi", "-Wl,-rpath,$ORIGIN"]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True)
+    return out
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv, verbose=True))
+    print(build_bindings(force="--force" in sys.argv, verbose=True))
