@@ -262,9 +262,22 @@ def main():
     cpu = None
     if not args.no_cpu_baseline:
         note("cpu baseline")
+        from concurrent.futures import ThreadPoolExecutor
+
         from oracle import bfp_oracle as oracle
 
         oracle.build()
+        host_threads = torch.get_num_threads()
+
+        def pack_all_cores(fmt_code, x2d):
+            """The oracle's from_torch sequence on bands of 32-row multiples, one band per host thread (ctypes drops the GIL)."""
+            rows = x2d.shape[0]
+            band = max(32, (rows // host_threads) // 32 * 32)
+            bands = [x2d[r:r + band] for r in range(0, rows, band)]
+            t = time.time()
+            with ThreadPoolExecutor(host_threads) as pool:
+                list(pool.map(lambda b: oracle.from_torch_bfp_tiles(fmt_code, np.ascontiguousarray(b)), bands))
+            return time.time() - t
         if args.workload in gemm_sets:
             name, m, k, n, fmt, batch = gemm_sets[args.workload][0]
             n_s = min(n, 2048)
@@ -294,6 +307,7 @@ def main():
                              f"oracle from_torch sequence on that slice, 1 thread",
                    "gold_bmm_1thread_tflops": round(2.0 * m * k * n_g / t_gold / 1e12, 5),
                    "from_torch_pack_melem_s_1thread": round(k * n_s / t_pack / 1e6, 1),
+                   "from_torch_pack_melem_s_all_threads": round(k * n_s / pack_all_cores(FMT[fmt], w) / 1e6, 1),
                    "to_torch_unpack_melem_s_1thread": round(k * n_s / t_unpack / 1e6, 1)}
         else:
             fmt = capi.BFLOAT4_B if args.workload == "pack_bfp4_4k" else capi.BFLOAT8_B
@@ -308,6 +322,8 @@ def main():
             cpu = {"value": round(2 * nb / (t_pack + t_unpack) / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                    "sample": f"oracle from_torch + to_torch host sequences on fp32 {list(x.shape)}",
                    "from_torch_pack_melem_s_1thread": round(x.size / t_pack / 1e6, 1),
+                   "from_torch_pack_melem_s_all_threads": round(x.size / pack_all_cores(fmt, x.reshape(-1, x.shape[-1])) / 1e6, 1),
+                   "host_threads": host_threads,
                    "to_torch_unpack_melem_s_1thread": round(x.size / t_unpack / 1e6, 1)}
 
     for leg in (l for wl in order for l in results[wl]):
