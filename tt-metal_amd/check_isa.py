@@ -2,14 +2,18 @@
 
 bfp_matmul.hip issues some global loads as inline assembly and waits for them with its own s_waitcnt, because the
 compiler's waits would drain the prefetch pipeline.  The compiler therefore believes that a loaded register holds its
-value as soon as the load has issued.  That is only safe if it never copies, moves or reuses such a register between
-the load and the wait.  This script reads the device assembly of the file and fails the build if that ever happens:
+value as soon as the load has issued.  That is only safe if it never copies, moves, reads or reuses such a register
+between the load and the point where the data is taken over.  This script reads the device assembly of the file,
+builds the control-flow graph of each streaming kernel and propagates the set of registers with a load in flight:
 
-  ring loads   (global_load_dwordx4 without sc1, activations in flight across loop iterations): from the first of
-               them to the last inline v_mov_b32 that hands a loaded register on (the pipelined loop and its tails),
-               their destination registers may be mentioned only inside inline-assembly blocks
-  slot loads   (global_load_dwordx4 ... sc1, partial sums of other workgroups): between the load and the inline
-               s_waitcnt vmcnt(0) that follows it, no compiler-generated instruction may mention the destination
+  ring loads   (inline global_load_dwordx4 without sc1: activations in flight across loop iterations) are in flight
+               until an inline `v_mov_b32 vX, vN` reads register N
+  slot loads   (inline global_load_dwordx4 ... sc1: partial sums of other workgroups) are in flight until the next
+               `s_waitcnt vmcnt(0)`
+  any `s_waitcnt vmcnt(0)` ends every flight (the kernel drains the ring that way when its k range is done)
+
+and fails the build if any compiler-generated instruction mentions a register while it is in flight, or if a register is
+still in flight when the kernel ends.
 
     python tt-metal_amd/check_isa.py file.s
 """
@@ -19,19 +23,21 @@ import re
 import sys
 
 _REG = re.compile(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]")
+_BRANCH = re.compile(r"^s_(cbranch_\w+|branch)\s+(\.LBB\w+)")
 
 
-def _regs(text: str) -> set:
+def _regs(text: str) -> frozenset:
     out = set()
     for m in _REG.finditer(text):
         if m.group(1) is not None:
             out.add(int(m.group(1)))
         else:
             out.update(range(int(m.group(2)), int(m.group(3)) + 1))
-    return out
+    return frozenset(out)
 
 
 def _kernels(lines):
+    """(name, lines) of every function: from its label to the .Lfunc_end label (blocks may follow an s_endpgm)."""
     name, body = None, []
     for line in lines:
         m = re.match(r"^(_Z\w+):", line)
@@ -39,10 +45,117 @@ def _kernels(lines):
             name, body = m.group(1), []
             continue
         if name is not None:
-            body.append(line)
-            if line.strip().startswith("s_endpgm"):
+            if line.startswith(".Lfunc_end"):
                 yield name, body
                 name = None
+            else:
+                body.append(line)
+
+
+def _blocks(body):
+    """Basic blocks: list of dicts {label, instrs: [(text, inline_asm)], succ: [labels or '+1' or 'end']}."""
+    blocks, cur, in_asm = [], {"label": None, "instrs": [], "succ": None}, False
+
+    def close(succ):
+        nonlocal cur
+        cur["succ"] = succ
+        blocks.append(cur)
+        cur = {"label": None, "instrs": [], "succ": None}
+
+    for line in body:
+        s = line.strip()
+        if s.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if s.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        m = re.match(r"^(\.LBB\w+):", s)
+        if m:
+            if cur["instrs"] or cur["label"] is not None:
+                close(["+1"])
+            cur["label"] = m.group(1)
+            continue
+        if not s or s.startswith(";") or s.startswith("."):
+            continue
+        text = s.split(";")[0].strip()
+        cur["instrs"].append((text, in_asm))
+        b = _BRANCH.match(text)
+        if b:
+            close([b.group(2)] if b.group(1) == "branch" else [b.group(2), "+1"])
+        elif text.startswith("s_endpgm"):
+            close(["end"])
+    if cur["instrs"]:
+        close(["end"])
+    return blocks
+
+
+def _check_kernel(name, body, problems):
+    blocks = _blocks(body)
+    index = {b["label"]: i for i, b in enumerate(blocks) if b["label"] is not None}
+    succs = []
+    for i, b in enumerate(blocks):
+        out = []
+        for t in b["succ"]:
+            if t == "+1":
+                if i + 1 < len(blocks):
+                    out.append(i + 1)
+            elif t != "end":
+                if t not in index:
+                    problems.append(f"{name}: branch to unknown label {t}")
+                else:
+                    out.append(index[t])
+        succs.append(out)
+    n_ring = sum(1 for b in blocks for t, a in b["instrs"] if a and t.startswith("global_load_dwordx4") and "sc1" not in t)
+    if not n_ring:
+        problems.append(f"{name}: no hand-written activation loads found (has the kernel changed?)")
+
+    def run(block, state, report):
+        ring, slot = set(state[0]), set(state[1])
+        for text, asm in block["instrs"]:
+            if asm:
+                if text.startswith("global_load_dwordx4"):
+                    dest = _regs(text.split(",")[0])
+                    (slot if "sc1" in text else ring).update(dest)
+                elif text.startswith("v_mov_b32"):
+                    ring -= _regs(text.split(",")[-1])
+                elif text.startswith("s_waitcnt vmcnt(0)"):
+                    ring.clear()
+                    slot.clear()
+                continue
+            if text.startswith("s_waitcnt") and "vmcnt(0)" in text:      # every vector-memory operation has landed
+                ring.clear()
+                slot.clear()
+                continue
+            if report is not None:
+                hit = _regs(text) & (ring | slot)
+                if hit:
+                    report.append(f"{name}: compiler instruction touches registers {sorted(hit)} while a hand-scheduled load into them is in flight: {text}")
+            if text.startswith("s_endpgm") and report is not None and (ring or slot):
+                report.append(f"{name}: registers {sorted(ring | slot)} still have a load in flight at s_endpgm")
+        return frozenset(ring), frozenset(slot)
+
+    empty = (frozenset(), frozenset())
+    state_in = [None] * len(blocks)
+    state_in[0] = empty
+    work = [0]
+    while work:
+        i = work.pop()
+        out = run(blocks[i], state_in[i], None)
+        for j in succs[i]:
+            merged = out if state_in[j] is None else (state_in[j][0] | out[0], state_in[j][1] | out[1])
+            if merged != state_in[j]:
+                state_in[j] = merged
+                work.append(j)
+    found = []
+    for i, b in enumerate(blocks):
+        if state_in[i] is not None:
+            run(b, state_in[i], found)
+    seen = set()
+    for f in found:
+        if f not in seen:
+            seen.add(f)
+            problems.append(f)
 
 
 def check(path: str, kernel_substring: str = "matmul_stream_kernel") -> int:
@@ -50,58 +163,15 @@ def check(path: str, kernel_substring: str = "matmul_stream_kernel") -> int:
     with open(path) as f:
         lines = f.read().split("\n")
     for name, body in _kernels(lines):
-        if kernel_substring not in name:
-            continue
-        checked += 1
-        # classify instructions: (index, text, inside inline assembly?)
-        instrs, in_asm = [], False
-        for line in body:
-            s = line.strip()
-            if s.startswith(";;#ASMSTART"):
-                in_asm = True
-                continue
-            if s.startswith(";;#ASMEND"):
-                in_asm = False
-                continue
-            if not s or s.startswith(";") or s.startswith("."):
-                if re.match(r"^\.LBB", s):
-                    instrs.append((s, in_asm, True))
-                continue
-            instrs.append((s.split(";")[0].strip(), in_asm, False))
-        ring = set()
-        for text, asm, _ in instrs:
-            if asm and text.startswith("global_load_dwordx4") and "sc1" not in text:
-                ring |= _regs(text.split(",")[0])
-        if not ring:
-            problems.append(f"{name}: no hand-written activation loads found (has the kernel changed?)")
-        # the stretch of code from the first request to the last hand-over (loop and tails as laid out in the file)
-        first = min((i for i, (t, a, _) in enumerate(instrs) if a and t.startswith("global_load_dwordx4") and "sc1" not in t), default=0)
-        last = max((i for i, (t, a, _) in enumerate(instrs) if a and t.startswith("v_mov_b32") and _regs(t.split(",")[-1]) & ring), default=0)
-        for text, asm, label in instrs[first:last + 1]:
-            if label or asm:
-                continue
-            hit = _regs(text) & ring
-            if hit:
-                problems.append(f"{name}: compiler instruction touches activation ring registers {sorted(hit)}: {text}")
-        for i, (text, asm, _) in enumerate(instrs):
-            if not (asm and text.startswith("global_load_dwordx4") and "sc1" in text):
-                continue
-            dest = _regs(text.split(",")[0])
-            for later, later_asm, later_label in instrs[i + 1:]:
-                if later_asm and later.startswith("s_waitcnt vmcnt(0)"):
-                    break
-                if later_label:
-                    problems.append(f"{name}: branch target between a slot load and its wait: {later}")
-                    break
-                if not later_asm and _regs(later) & dest:
-                    problems.append(f"{name}: compiler instruction touches a slot load's destination before the wait: {later}")
-                    break
-            else:
-                problems.append(f"{name}: slot load without a following inline wait: {text}")
+        if kernel_substring in name:
+            checked += 1
+            _check_kernel(name, body, problems)
     if not checked:
         problems.append(f"no kernel matching '{kernel_substring}' in {path}")
-    for p in problems:
+    for p in problems[:40]:
         print("check_isa:", p, file=sys.stderr)
+    if len(problems) > 40:
+        print(f"check_isa: ... and {len(problems) - 40} more", file=sys.stderr)
     return len(problems)
 
 

@@ -16,9 +16,9 @@
 //              4c+j of the group and k rows 8g..8g+7: byte j of the 8 mantissa words it reads from LDS.  The packed
 //              layout (16 consecutive columns of one k row share a word run) never has to be transposed.
 //   workgroup  4 wavefronts take the units of a contiguous range round-robin, add their partial sums through LDS
-//              and store; the range is this workgroup's equal share of ALL units ("stream-K"), so every workgroup
-//              streams the same number of bytes whatever K and N are.  Outputs whose k range is shared between
-//              workgroups are finished by the workgroup that arrives last (see the kernel).
+//              and store; the range is one of the nearly equal parts the host cuts every output's k range into, as
+//              many as fill the chip.  Outputs whose k range is shared between workgroups are finished by the
+//              workgroup that owns the last part (see the kernel).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -78,7 +78,7 @@ __device__ __forceinline__ uint32_t not_empty(uint32_t bits) { return bits == SL
 //   split > 0   every output group is cut into `split` nearly equal k ranges, one per workgroup (P = groups * split):
 //               one output per workgroup, at most `split` partial sums to add
 //   split == 0  "stream-K": the U units are dealt out contiguously, the first `extra` workgroups take share + 1 units,
-//               the rest `share`; a range may end one output and begin the next
+//               the rest `share`; a range may end one output and begin the next (the host does not choose this)
 __device__ __forceinline__ uint32_t range_start(const MatmulDev &p, uint32_t i) {
     if (p.split) return (i / p.split) * p.kt + ((i % p.split) * p.kt) / p.split;
     return i * p.share + min(i, p.extra);
@@ -92,11 +92,12 @@ __device__ __forceinline__ uint32_t workgroup_of(const MatmulDev &p, uint32_t un
     return unit < fat ? unit / (p.share + 1) : p.extra + (unit - fat) / p.share;
 }
 
-// Work decomposition ("stream-K"): units are numbered with the k-tile fastest and dealt out contiguously and
-// evenly to P workgroups (P = what the chip holds at once).  A workgroup whose range covers all k-tiles of an
-// output group stores that output directly.  Otherwise it writes its fp32 partial sums to a slot of its own and
-// bumps the group's arrival counter; the workgroup that arrives last adds the slots in workgroup order (so the
-// result does not depend on who was last), applies the epilogue, stores, and resets the counter.
+// Work decomposition: units are numbered with the k-tile fastest; a workgroup takes a contiguous range of them (see
+// range_start).  A workgroup whose range covers all k-tiles of an output group stores that output directly.
+// Otherwise the contributors to an output hand their fp32 partial sums over in slots: every contributor but the one
+// with the highest index writes its sums to its own slot; that last one waits for each slot to lose its SLOT_EMPTY
+// pattern, adds the slots in workgroup order to its own sums (so the result does not depend on timing), applies the
+// epilogue, stores, and puts the empty pattern back.
 template <int W, int ACT>
 __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const MatmulDev p) {
     using F = Wfmt<W>;
@@ -243,6 +244,7 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
         };
         tail(S0{}, i); tail(S1{}, i + 1); tail(S2{}, i + 2); tail(S0{}, i + 3); tail(S1{}, i + 4);
 
+        wait_vmcnt<0>();   // nothing in flight any more (already true; also what the build-time ISA check keys on)
         // ---- add the four wavefronts' partial sums through LDS --------------------------------------------------
         // Every wavefront writes all 32 of its accumulator registers (register indices are compile-time constants;
         // who reads what is decided by addresses), then wavefront w keeps half w/2 of the band, registers
@@ -398,17 +400,14 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     // workgroups to aim for: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone nearly get there,
     // x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot reset)
     const uint64_t resident = env_u32("TTMI_MATMUL_WGS", d.groups >= 256 ? 768 : 512);
-    if (env_u32("TTMI_MATMUL_STREAMK", 0)) {
-        d.split = 0;
-        d.workgroups = (uint32_t)(d.units < resident ? d.units : resident);
-    } else {
-        // cut every output's k range into as many parts as keeps the chip full, every wavefront keeping >= 2 k-tiles
-        uint64_t parts = d.groups >= resident ? 1 : resident / d.groups;
-        const uint64_t most = d.kt / (2 * WAVES) ? d.kt / (2 * WAVES) : 1;
-        if (parts > most) parts = most;
-        d.split = (uint32_t)parts;
-        d.workgroups = (uint32_t)(d.groups * parts);
-    }
+    // cut every output's k range into as many parts as keeps the chip full, every wavefront keeping >= 2 k-tiles
+    // (the kernel can also deal the units out evenly across output boundaries, split == 0, but a workgroup that is
+    // consumer of one output and producer of the next would then make its successor wait: not offered)
+    uint64_t parts = d.groups >= resident ? 1 : resident / d.groups;
+    const uint64_t most = d.kt / (2 * WAVES) ? d.kt / (2 * WAVES) : 1;
+    if (parts > most) parts = most;
+    d.split = (uint32_t)parts;
+    d.workgroups = (uint32_t)(d.groups * parts);
     return d;
 }
 
