@@ -159,6 +159,55 @@ def test_caller_workspace(oracle):
         capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP4, 1, 1, m, k, n, workspace=small)
 
 
+@pytest.mark.parametrize("kernel", ["stream", "tile", "tile256", "expanded"])
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("batch,b_batch,m,k,n", [(1, 1, 256, 128, 256), (1, 1, 300, 96, 288), (2, 1, 130, 160, 96), (1, 1, 288, 224, 96),
+                                                 (2, 2, 512, 64, 544), (1, 1, 40, 32, 2080)])
+def test_every_kernel_on_every_shape(oracle, kernel, fmt, batch, b_batch, m, k, n, monkeypatch):
+    """Each GEMM kernel forced onto shapes it would not be chosen for: ragged row blocks, odd tile counts, one k step,
+    more than eight 256-column blocks, shared and per-slice weights; TILE layout in and out, bias and activation."""
+    monkeypatch.setenv("TTMI_MATMUL_KERNEL", kernel[:4])
+    if kernel == "tile256":
+        monkeypatch.setenv("TTMI_MATMUL_BM", "256")
+    a_bits = workloads.activations_bf16(m, k, seed=75, batch=batch)
+    w = workloads.weights_f32(k, n, seed=76, batch=b_batch)
+    words, w_unpacked = pack_weights(oracle, w, fmt)
+    a = workloads.bf16_bits_to_f32(a_bits).reshape(batch, m, k)
+    w_unpacked = w_unpacked.reshape(b_batch, k, n)
+    a_dev = bf16_dev(a_bits).reshape(batch, m, k)
+    c = capi.matmul_bfp(a_dev, capi.ROW_MAJOR, words, fmt, batch, b_batch, m, k, n, out_dtype=torch.float32)
+    for b in range(batch):
+        check_against_reference(c[b].cpu().numpy(), a[b], w_unpacked[b if b_batch > 1 else 0], k, bf16_out=False)
+    # TILE layout on both sides gives the same bits as row-major
+    c_rm = capi.matmul_bfp(a_dev, capi.ROW_MAJOR, words, fmt, batch, b_batch, m, k, n)
+    if m % 32 == 0:                                          # the C ABI takes TILE operands only with whole tiles
+        c_tiles = capi.matmul_bfp(capi.tilize(a_dev), capi.TILE, words, fmt, batch, b_batch, m, k, n, c_layout=capi.TILE)
+        assert torch.equal(capi.untilize(c_tiles, (batch, m, n)).view(torch.int16), c_rm.view(torch.int16))
+    # bias and activation
+    bias_bits = workloads.f32_to_bf16_bits_rne(workloads.normal_tensor((n,), seed=77))
+    g = capi.matmul_bfp(a_dev, capi.ROW_MAJOR, words, fmt, batch, b_batch, m, k, n, bias=bf16_dev(bias_bits),
+                        activation=capi.ACT_RELU, out_dtype=torch.float32)
+    want = torch.relu(c + torch.from_numpy(workloads.bf16_bits_to_f32(bias_bits)).cuda())
+    assert torch.allclose(g, want, rtol=1e-5, atol=1e-5)
+
+
+def test_expanded_weights_in_a_caller_workspace(oracle, monkeypatch):
+    monkeypatch.setenv("TTMI_MATMUL_KERNEL", "expanded")
+    m, k, n = 512, 128, 160
+    a_bits = workloads.activations_bf16(m, k, seed=78)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=79), BFP8)
+    need = capi.lib().ttmi_matmul_bfp_workspace_bytes(1, m, k, n, BFP8)
+    assert need == (k // 32) * 3 * 4096                      # 2 bytes per weight, 64-column groups
+    ws = torch.full((need,), 0x5A, dtype=torch.uint8, device="cuda")
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n, workspace=ws)
+    check_against_reference(c.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+    own = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    assert torch.equal(own.view(torch.int16), c.view(torch.int16))
+    with pytest.raises(RuntimeError, match="workspace"):
+        capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n,
+                        workspace=torch.empty(need - 256, dtype=torch.uint8, device="cuda"))
+
+
 @pytest.mark.parametrize("name,m,k,n,fmt,batch", workloads.DECODE_FALCON + workloads.DECODE_MISTRAL)
 def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch):
     a_bits = workloads.activations_bf16(m, k, seed=80)

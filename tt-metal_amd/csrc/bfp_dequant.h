@@ -160,4 +160,83 @@ __device__ __forceinline__ void staged_operands(uint32_t exp_at, uint32_t mant_a
     bop[3] = weights_operand8<3>(words, mags, scale);
 }
 
+// Epilogue of the tiled GEMM kernels for one wavefront: a 128-row x 64-column part of C (one 64-column weight group) whose
+// accumulators lie as v_mfma_f32_32x32x16 leaves them, with the column order of the weight expansion:
+//   acc[rb][cb][i] = row 32 rb + 8 (i / 4) + 4 kh + i % 4, column 32 t + 16 fc + 4 q + 2 half + cb of the 64, for lane
+//   (c = lane % 32, kh = lane / 32), c16 = c % 16, half = c / 16, t = c16 / 8, fc = (c16 / 4) % 2, q = c16 % 4.
+// A lane therefore owns pairs of adjacent columns, 4 bytes of bf16: stored directly that is one 32- or 64-byte piece per
+// row and instruction.  Instead the wavefront lays the bf16 block out in 16 KB of LDS of its own exactly as it lies in
+// memory (TILE layout: per 32 rows the two tiles are 4 KB contiguous; row-major: 128 bytes per row) and copies it out
+// with 16 bytes per lane.  fp32 output is stored directly (8 bytes per lane).
+struct StoreTarget {
+    uint8_t *c;              // output
+    const uint16_t *bias;    // bf16 [n] or null
+    uint32_t m, n, nt;       // rows of a batch slice, columns, n / 32
+    uint64_t slice;          // batch slice
+    uint32_t row0;           // first row of the part
+    uint32_t nt0;            // first packed tile column of the group (the group has 1 or 2 tiles)
+    float unscale;
+    int c_tiled, c_f32;
+};
+
+template <int ACT, typename Acc>
+__device__ __forceinline__ void store_wave_part(const Acc (&acc)[4][2], const StoreTarget &o, uint8_t *lds_wave, int lane) {
+    const int c = lane & 31, kh = lane >> 5;
+    const int c16 = c & 15, half = c >> 4;
+    const int t = c16 >> 3, fc = (c16 >> 2) & 1, q = c16 & 3;
+    if (o.nt0 >= o.nt) return;
+    const uint32_t tiles = min(2u, o.nt - o.nt0);
+    const uint32_t col = t * 32 + fc * 16 + q * 4 + half * 2;             // of the group's 64
+    const bool lane_valid = (uint32_t)t < tiles;
+    float bias_v[2] = {0.f, 0.f};
+    if (o.bias && lane_valid) {
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) bias_v[cb] = __uint_as_float((uint32_t)o.bias[o.nt0 * 32 + col + cb] << 16);
+    }
+    const uint32_t mt = (o.m + 31) / 32;
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t r32 = (i >> 2) * 8 + kh * 4 + (i & 3);
+            const float v0 = apply_activation<ACT>(acc[rb][0][i] * o.unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * o.unscale + bias_v[1]);
+            if (o.c_f32) {
+                const uint32_t row = o.row0 + rb * 32 + r32;
+                if (row >= o.m || !lane_valid) continue;
+                uint64_t elem;
+                if (o.c_tiled) elem = ((o.slice * mt + (row >> 5)) * o.nt + o.nt0 + t) * 1024 + (((row >> 4) & 1) * 2 + fc) * 256 + (row & 15) * 16 + q * 4 + half * 2;
+                else elem = (o.slice * o.m + row) * o.n + o.nt0 * 32 + col;
+                *reinterpret_cast<float2 *>(o.c + elem * 4) = make_float2(v0, v1);
+            } else {
+                const uint32_t both = f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
+                const uint32_t at = o.c_tiled ? rb * 4096 + t * 2048 + (((r32 >> 4) & 1) * 2 + fc) * 512 + (r32 & 15) * 32 + q * 8 + half * 4
+                                              : (rb * 32 + r32) * 128 + col * 2;
+                *reinterpret_cast<uint32_t *>(lds_wave + at) = both;
+            }
+        }
+    }
+    if (o.c_f32) return;
+    if (o.c_tiled) {
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+            const uint32_t row = o.row0 + rb * 32;
+            if (row >= o.m) break;
+            uint8_t *dst = o.c + ((o.slice * mt + (row >> 5)) * o.nt + o.nt0) * 2048;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if ((uint32_t)j < tiles * 2)
+                    *reinterpret_cast<u32x4 *>(dst + j * 1024 + lane * 16) = *reinterpret_cast<const u32x4 *>(lds_wave + rb * 4096 + j * 1024 + lane * 16);
+        }
+    } else {
+        const uint32_t chunk = lane & 7;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const uint32_t r = j * 8 + (lane >> 3), row = o.row0 + r;
+            if (row < o.m && chunk < tiles * 4)
+                *reinterpret_cast<u32x4 *>(o.c + ((o.slice * o.m + row) * o.n + o.nt0 * 32) * 2 + chunk * 16) =
+                    *reinterpret_cast<const u32x4 *>(lds_wave + r * 128 + chunk * 16);
+        }
+    }
+}
+
 }  // namespace ttmi

@@ -411,12 +411,6 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     return d;
 }
 
-size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int) {
-    if (!batch || !m || !k || !n) return 0;
-    const Decomposition d = decompose(batch, m, k, n);
-    return (size_t)2 * d.workgroups * SLOT_BYTES;
-}
-
 // The library's own partial-sum slots, per device, grown on demand and kept until the process ends.  Every word is
 // SLOT_EMPTY when allocated, and every launch leaves it that way.
 struct Scratch { void *ptr = nullptr; size_t bytes = 0; };
@@ -481,13 +475,36 @@ int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) {
     return check_launch("matmul_stream_kernel");
 }
 
-// Tall activations are MFMA-bound and go to the tiled kernel; up to 127 rows the weights are streamed once per
-// 32-row band.  TTMI_MATMUL_KERNEL=stream|tile overrides the choice (for tests and measurements).
-int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
+// Which kernel a shape goes to.  Up to 127 rows the weights are streamed once per 32-row band (HBM-bound); taller
+// activations are MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows on (two or more 256-row blocks
+// share every weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
+// TTMI_MATMUL_KERNEL=stream|tile|expanded overrides the choice (for tests and measurements).
+enum class Kernel { Stream, Tile, Expanded };
+static Kernel choose_kernel(uint32_t m) {
     const char *force = getenv("TTMI_MATMUL_KERNEL");
-    if (force && force[0] == 's') return matmul_bfp_stream(x, st);
-    if (force && force[0] == 't') return matmul_bfp_tiled(x, st);
-    return x.m >= 128 ? matmul_bfp_tiled(x, st) : matmul_bfp_stream(x, st);
+    if (force && force[0] == 's') return Kernel::Stream;
+    if (force && force[0] == 't') return Kernel::Tile;
+    if (force && force[0] == 'e') return Kernel::Expanded;
+    return m >= 512 ? Kernel::Expanded : m >= 128 ? Kernel::Tile : Kernel::Stream;
+}
+
+size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int) {
+    if (!batch || !m || !k || !n) return 0;
+    switch (choose_kernel(m)) {
+        case Kernel::Expanded: return matmul_expanded_workspace_bytes(batch, k, n);   // as if every slice had weights of its own
+        case Kernel::Tile: return 0;
+        default: break;
+    }
+    const Decomposition d = decompose(batch, m, k, n);
+    return d.split == 1 ? 0 : (size_t)2 * d.workgroups * SLOT_BYTES;
+}
+
+int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
+    switch (choose_kernel(x.m)) {
+        case Kernel::Expanded: return matmul_bfp_expanded(x, st);
+        case Kernel::Tile: return matmul_bfp_tiled(x, st);
+        default: return matmul_bfp_stream(x, st);
+    }
 }
 
 }  // namespace ttmi
