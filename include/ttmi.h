@@ -108,7 +108,10 @@ TTMI_API size_t ttmi_matmul_bfp_workspace_bytes(uint32_t batch, uint32_t m, uint
  *   bias     NULL or bf16 [n] (row-broadcast add, matmul.hpp:117-214)
  *   c        c_dtype TTMI_BFLOAT16 (round to nearest even) or TTMI_FLOAT32; c_layout as for a
  *   workspace NULL (the library keeps a per-device buffer of its own, allocated on first use) or at least
- *            ttmi_matmul_bfp_workspace_bytes() bytes of device memory, 256-byte aligned
+ *            ttmi_matmul_bfp_workspace_bytes() bytes of device memory, 256-byte aligned.  Up to 127 rows it holds
+ *            partial sums of workgroups that share an output (a few MB); from 512 rows on the weights expanded to
+ *            bf16 (2 bytes per weight; the size query assumes every batch slice has weights of its own, a call with
+ *            b_batch == 1 needs only one slice's worth)
  * fp32 accumulation throughout. */
 TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch,
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,

@@ -184,7 +184,7 @@ __global__ __launch_bounds__(512, 1) void matmul_expanded_kernel(const ExpandedD
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.f;
 
-    bf16x8 a0[RB], b0[CB], a1[RB], b1[CB];
+    bf16x8 a0[RB], b0[CB], a1[RB], b1[CB], a2[RB], b2[CB];
     request(0); request(1); request(2);
     wait_vmcnt<VM_PER_STEP>();                 // steps 0 and 1 have landed (ours)
     __builtin_amdgcn_s_barrier();              // everybody's
@@ -192,29 +192,37 @@ __global__ __launch_bounds__(512, 1) void matmul_expanded_kernel(const ExpandedD
     for (int j = 0; j < 6; ++j) read_operand(0, 0, j, a0, b0);
 
     // Between two MFMAs a wavefront issues at most one LDS read or one request (order of the reads: what the next slab
-    // needs first), so that the matrix pipe never waits for a burst of them.
+    // needs first), so that the matrix pipe never waits for a burst of them.  The operands of the next step's first
+    // slab are read early in this step into a third set of registers: all wavefronts reach the barrier together, and
+    // whatever they wait for there nobody hides.
     constexpr int read_order[6] = {0, 4, 5, 1, 2, 3};
-#pragma unroll 1
-    for (uint32_t kstep = 0; kstep < p.kt; ++kstep) {
+    auto step_body = [&](uint32_t kstep, bf16x8 (&a_now)[RB], bf16x8 (&b_now)[CB], bf16x8 (&a_next)[RB], bf16x8 (&b_next)[CB]) __attribute__((always_inline)) {
         wait_vmcnt<VM_PER_STEP>();             // only the previous step's requests may still be in flight
         __builtin_amdgcn_s_waitcnt(0xC07F);    // our LDS reads of the previous step are done
         __builtin_amdgcn_s_barrier();
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {          // slab 0; reads of slab 1, then two requests for step + 3
-            acc[i >> 1][i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[i >> 1], b0[i & 1], acc[i >> 1][i & 1], 0, 0, 0);
+        for (int i = 0; i < 8; ++i) {          // slab 0; reads of slab 1, then of slab 0 of the next step (in LDS since the barrier)
+            acc[i >> 1][i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_now[i >> 1], b_now[i & 1], acc[i >> 1][i & 1], 0, 0, 0);
             if (i < 6) read_operand(kstep, 1, read_order[i], a1, b1);
-            else request_one(kstep + 3, i - 6);
+            else read_operand(kstep + 1, 0, read_order[i - 6], a_next, b_next);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {          // slab 1; reads of slab 0 of the next step (in LDS since this step's barrier)
+        for (int i = 0; i < 8; ++i) {          // slab 1; the remaining reads, then the requests for step + 3
             acc[i >> 1][i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1[i >> 1], b1[i & 1], acc[i >> 1][i & 1], 0, 0, 0);
-            if (i < 6) read_operand(kstep + 1, 0, read_order[i], a0, b0);
+            if (i < 4) read_operand(kstep + 1, 0, read_order[i + 2], a_next, b_next);
             else request_one(kstep + 3, i - 4);
             __builtin_amdgcn_sched_barrier(0);
         }
         asm volatile("" ::: "memory");         // the requests stay in this step
+    };
+    uint32_t kstep = 0;
+#pragma unroll 1
+    for (; kstep + 2 <= p.kt; kstep += 2) {
+        step_body(kstep, a0, b0, a2, b2);
+        step_body(kstep + 1, a2, b2, a0, b0);
     }
+    if (kstep < p.kt) step_body(kstep, a0, b0, a2, b2);
     wait_vmcnt<0>();                           // requests past the end have landed,
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __builtin_amdgcn_s_barrier();              // and nobody reads operands any more: the ring becomes 8 x 16 KB of staging
