@@ -152,6 +152,55 @@ def main():
                "layout": "row_major" if args.row_major else "tile", "roofline": roof}
         return leg, (run, wcopies, acopies, c)
 
+    def block_leg(name, steps, warmup, seed):
+        """A whole decode MLP block as tt-metal's model code issues it (M = 32, operands in TILE layout), every launch
+        through the C ABI: Falcon-7B dense_h_to_4h with fused GELU -> dense_4h_to_h (models/demos/falcon7b/tt/falcon_mlp.py:56-80),
+        Mistral-7B silu(x w1) * (x w3) -> w2 (models/demos/mistral7b/tt/mistral_mlp.py:43-82)."""
+        L = capi.lib()
+        stream = torch.cuda.current_stream().cuda_stream
+        m = 32
+        if name == "falcon_mlp_block":
+            gemms = [("w1", 4544, 18176, "bfp8_b", capi.ACT_GELU), ("w2", 18176, 4544, "bfp8_b", capi.ACT_NONE)]
+        else:
+            gemms = [("w1", 4096, 14336, "bfp4_b", capi.ACT_SILU), ("w3", 4096, 14336, "bfp4_b", capi.ACT_NONE),
+                     ("w2", 14336, 4096, "bfp4_b", capi.ACT_NONE)]
+        packed = {g[0]: capi.pack_tensor(FMT[g[3]], dev(workloads.weights_f32(g[1], g[2], seed + i))) for i, g in enumerate(gemms)}
+        per_block = sum(t.numel() * 4 for t in packed.values())
+        ncopies = copies_for(per_block)
+        copies = [{k: (v if j == 0 else v.clone()) for k, v in packed.items()} for j in range(ncopies)]
+        x = capi.tilize(bf16_dev(workloads.activations_bf16(m, gemms[0][1], seed + 7)))
+        hidden = gemms[0][2]
+        h1 = torch.empty(m * hidden, dtype=torch.bfloat16, device="cuda")
+        h3 = torch.empty(m * hidden, dtype=torch.bfloat16, device="cuda")
+        out = torch.empty(m * gemms[-1][2], dtype=torch.bfloat16, device="cuda")
+
+        def mm(a, w, k, n, fmt, act, c):
+            return (a.data_ptr(), capi.TILE, w.data_ptr(), FMT[fmt], 1, 1, m, k, n, None, act, c.data_ptr(), capi.TILE, capi.BFLOAT16, None, 0, stream)
+
+        plans = []
+        for cp in copies:
+            if name == "falcon_mlp_block":
+                plans.append([("mm", mm(x, cp["w1"], 4544, 18176, "bfp8_b", capi.ACT_GELU, h1)),
+                              ("mm", mm(h1, cp["w2"], 18176, 4544, "bfp8_b", capi.ACT_NONE, out))])
+            else:
+                plans.append([("mm", mm(x, cp["w1"], 4096, 14336, "bfp4_b", capi.ACT_SILU, h1)),
+                              ("mm", mm(x, cp["w3"], 4096, 14336, "bfp4_b", capi.ACT_NONE, h3)),
+                              ("el", (capi.OP_MUL, h1.data_ptr(), h3.data_ptr(), 0.0, h1.data_ptr(), h1.numel(), stream)),
+                              ("mm", mm(h1, cp["w2"], 14336, 4096, "bfp4_b", capi.ACT_NONE, out))])
+
+        def run(i):
+            for kind, call in plans[i % ncopies]:
+                capi.check(L.ttmi_matmul_bfp(*call) if kind == "mm" else L.ttmi_eltwise_bf16(*call))
+
+        ms = time_loop(run, steps, warmup)
+        nbytes = sum(workloads.gemm_bytes(m, g[1], g[2], g[3], None) for g in gemms) + (3 * m * hidden * 2 if len(gemms) == 3 else 0)
+        flops = sum(workloads.gemm_flops(m, g[1], g[2], None) for g in gemms)
+        leg = {"workload": name, "launches": len(plans[0]), "ms": round(ms, 5), "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
+               "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "algorithmic_bytes": nbytes, "flops": flops,
+               "weight_copies_rotated": ncopies, "layout": "tile", "roofline": hbm_roofline(nbytes, ms)}
+        del copies, packed
+        return leg
+
     def codec_leg(name, x_np, fmt, steps, warmup):
         x = dev(x_np)
         nbytes_in = x.numel() * 4
@@ -222,6 +271,11 @@ def main():
                     primary_keep.append(state)
                 del state
                 torch.cuda.empty_cache()
+            if not is_primary or args.legs != "none":
+                block = {"decode_falcon": "falcon_mlp_block", "decode_mistral": "mistral_mlp_block"}.get(wl)
+                if block and not args.row_major:
+                    sub.append(block_leg(block, sub_steps, warmup, 4321))
+                    torch.cuda.empty_cache()
             results[wl] = sub
         else:
             fmt = capi.BFLOAT4_B if wl == "pack_bfp4_4k" else capi.BFLOAT8_B
@@ -244,7 +298,7 @@ def main():
             primary_runs = []
             torch.cuda.empty_cache()
 
-    prim = results[args.workload]
+    prim = [l for l in results[args.workload] if "launches" not in l]     # the whole-block legs are reported, not summed
     if args.workload in gemm_sets:
         total_flops = sum(l["flops"] for l in prim)
         value, unit = total_flops / (total_ms * 1e-3) / 1e12, "TFLOP/s"

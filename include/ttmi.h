@@ -43,6 +43,10 @@ enum { TTMI_ROW_MAJOR = 0, TTMI_TILE = 1 };
 /* fused activation of ttnn.linear (ttnn/ttnn/operations/matmul.py:59-63) */
 enum { TTMI_ACT_NONE = 0, TTMI_ACT_RELU = 1, TTMI_ACT_GELU = 2, TTMI_ACT_SILU = 3 };
 
+/* elementwise operations of ttmi_eltwise_bf16: the binary ones carry the values of BinaryOpType
+ * (tt_eager/tt_dnn/op_library/eltwise_binary/eltwise_binary_op.hpp:20-38), the unary ones 16 + TTMI_ACT_* */
+enum { TTMI_OP_ADD = 0, TTMI_OP_SUB = 1, TTMI_OP_MUL = 2, TTMI_OP_RELU = 17, TTMI_OP_GELU = 18, TTMI_OP_SILU = 19 };
+
 TTMI_API const char *ttmi_last_error(void);
 TTMI_API const char *ttmi_version(void);
 
@@ -116,6 +120,15 @@ TTMI_API size_t ttmi_matmul_bfp_workspace_bytes(uint32_t batch, uint32_t m, uint
 TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch,
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
                     int c_dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/* c[i] = op(a[i], b[i]) on bf16 tensors of equal shape and layout (count elements, any layout: equal shapes have equal
+ * element order), fp32 arithmetic, one rounding to bf16: tt::tt_metal::eltwise_binary
+ * (tt_eager/tt_dnn/op_library/eltwise_binary/eltwise_binary_op.hpp:108-140) as reached from ttnn.mul / add / sub
+ * (ttnn/ttnn/operations/binary.py:321-424; Mistral's MLP multiplies gate and up projections with it,
+ * models/demos/mistral7b/tt/mistral_mlp.py:66-70).  b == NULL: op(a[i], scalar), the *_unary forms
+ * (binary.py:360-368).  Unary ops (TTMI_OP_RELU | GELU | SILU, eltwise_unary_op.hpp:17-90) ignore b and scalar.
+ * a, b, c 16-byte aligned; c may alias a or b. */
+TTMI_API int ttmi_eltwise_bf16(int op, const void *a, const void *b, float scalar, void *c, size_t count, void *stream);
 
 #ifdef __cplusplus
 }

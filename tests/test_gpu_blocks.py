@@ -1,0 +1,190 @@
+"""Callers either side of the block-float GEMMs, on the GPU: elementwise ops (ttnn.mul and friends), weight caches as tensor
+files, and the Falcon-7B / Mistral-7B MLP blocks, in the shape of the reference's own tests
+(tests/ttnn/integration_tests/falcon7b/test_falcon_mlp.py:17-95, tests/ttnn/unit_tests/test_as_tensor.py,
+tests/ttnn/unit_tests/test_dump_and_load.py, tests/ttnn/unit_tests/operations/test_mul.py).
+
+Block parity (stated here, the reference's own bar is PCC >= 0.985 against the torch model with unquantised weights):
+PCC >= 0.9999 against an fp64 evaluation that uses the weights as the oracle unpacks them and rounds the activations
+between the GEMMs to bf16 as the device does; PCC >= 0.99 against the plain torch functional model.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def device():
+    import ttnn
+
+    dev = ttnn.open_device(0)
+    yield dev
+    ttnn.close_device(dev)
+
+
+def pcc(a, b):
+    a, b = a.double().reshape(-1), b.double().reshape(-1)
+    return float(torch.corrcoef(torch.stack([a, b]))[0, 1])
+
+
+def quantised(oracle, ttnn_dtype, w):
+    """[K, N] fp32 -> the values a block-float tensor of it holds (oracle pack + unpack), fp64."""
+    x = w.float().numpy()[None]
+    words = oracle.from_torch_bfp_tiles(int(ttnn_dtype), x)
+    return torch.from_numpy(oracle.to_torch_bfp_tiles(int(ttnn_dtype), words, x.shape)[0]).double()
+
+
+def bf16_round(x):
+    return x.float().to(torch.bfloat16).double()
+
+
+# ---- elementwise ----------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(32, 64), (1, 1, 32, 18176), (2, 3, 64, 96), (7, 3)])
+@pytest.mark.parametrize("layout_name", ["TILE_LAYOUT", "ROW_MAJOR_LAYOUT"])
+def test_binary_ops_match_torch_bf16(device, shape, layout_name):
+    import ttnn
+
+    layout = getattr(ttnn, layout_name)
+    torch.manual_seed(11)
+    a = torch.randn(shape).to(torch.bfloat16)
+    b = torch.randn(shape).to(torch.bfloat16)
+    ta = ttnn.from_torch(a, layout=layout, device=device)
+    tb = ttnn.from_torch(b, layout=layout, device=device)
+    for fn, ref in ((ttnn.mul, torch.mul), (ttnn.add, torch.add), (ttnn.sub, torch.sub)):
+        out = fn(ta, tb)
+        assert out.shape == shape and out.dtype == ttnn.bfloat16 and out.layout == layout
+        want = ref(a.float(), b.float()).to(torch.bfloat16)         # fp32 arithmetic, one rounding: what torch does for bf16 too
+        assert torch.equal(ttnn.to_torch(out), want)
+    assert torch.equal(ttnn.to_torch(ttnn.mul(ta, 0.5)), (a.float() * 0.5).to(torch.bfloat16))
+    assert torch.equal(ttnn.to_torch(ttnn.multiply(ta, tb)), torch.mul(a.float(), b.float()).to(torch.bfloat16))
+
+
+def test_unary_ops(device):
+    import ttnn
+
+    torch.manual_seed(12)
+    a = (torch.randn(1, 1, 64, 160) * 3).to(torch.bfloat16)
+    ta = ttnn.from_torch(a, layout=ttnn.TILE_LAYOUT, device=device)
+    for fn, ref in ((ttnn.gelu, torch.nn.functional.gelu), (ttnn.relu, torch.relu), (ttnn.silu, torch.nn.functional.silu)):
+        got = ttnn.to_torch(fn(ta)).float()
+        want = ref(a.double())
+        assert torch.allclose(got.double(), want, rtol=2 ** -8, atol=1e-6)
+
+
+def test_block_float_operand_and_errors(oracle, device):
+    import ttnn
+
+    torch.manual_seed(13)
+    a = torch.randn(64, 64)
+    b = torch.randn(64, 64).to(torch.bfloat16)
+    ta = ttnn.from_torch(a, dtype=ttnn.bfloat8_b, layout=ttnn.TILE_LAYOUT, device=device)
+    tb = ttnn.from_torch(b, layout=ttnn.TILE_LAYOUT, device=device)
+    out = ttnn.mul(ta, tb)
+    assert out.dtype == ttnn.bfloat8_b                              # the output takes input a's dtype
+    aq = quantised(oracle, ttnn.bfloat8_b, a)
+    product = (aq.float() * b.float()).to(torch.bfloat16).float()
+    want = oracle.to_torch_bfp_tiles(3, oracle.from_torch_bfp_tiles(3, product.numpy()[None]), (1, 64, 64))[0]
+    assert np.array_equal(ttnn.to_torch(out).numpy(), want)
+    with pytest.raises(RuntimeError, match="on device"):
+        ttnn.mul(ttnn.from_torch(b, layout=ttnn.TILE_LAYOUT), tb)
+    with pytest.raises(RuntimeError, match="broadcast"):
+        ttnn.mul(tb, ttnn.from_torch(b[:1], layout=ttnn.ROW_MAJOR_LAYOUT, device=device))
+    with pytest.raises(TypeError):
+        ttnn.mul(tb, "x")
+
+
+# ---- tensor files and weight caches -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["bfloat8_b", "bfloat4_b", "bfloat16"])
+def test_dump_and_load_tilized(tmp_path, device, name):
+    import ttnn
+
+    dtype = getattr(ttnn, name)
+    torch.manual_seed(14)
+    x = torch.rand((96, 160), dtype=torch.float32).to(torch.bfloat16)
+    t = ttnn.from_torch(x, dtype=dtype, layout=ttnn.TILE_LAYOUT)
+    ttnn.dump_tensor(tmp_path / "tensor.bin", t)
+    assert (tmp_path / "tensor.bin").stat().st_size == 200 + 15 * {"bfloat8_b": 1088, "bfloat4_b": 576, "bfloat16": 2048}[name]
+    loaded = ttnn.load_tensor(tmp_path / "tensor.bin")
+    assert loaded.dtype == dtype and loaded.layout == ttnn.TILE_LAYOUT and loaded.shape == t.shape
+    assert torch.equal(loaded._buf, t._buf)
+    assert torch.equal(ttnn.to_torch(loaded), ttnn.to_torch(t))
+    with pytest.raises(RuntimeError, match="Device storage"):
+        ttnn.dump_tensor(tmp_path / "d.bin", ttnn.to_device(t, device))
+
+
+def test_as_tensor_with_cache(tmp_path, device):
+    """tests/ttnn/unit_tests/test_as_tensor.py:25-58, with a block-float weight."""
+    import ttnn
+
+    torch.manual_seed(15)
+    w = torch.rand((7, 3), dtype=torch.float32)
+    plain = ttnn.as_tensor(w.to(torch.bfloat16), layout=ttnn.TILE_LAYOUT, device=device, memory_config=ttnn.L1_MEMORY_CONFIG)
+    assert torch.allclose(ttnn.to_torch(plain), w.to(torch.bfloat16))
+    big = torch.randn(160, 96)
+    first = ttnn.as_tensor(big, dtype=ttnn.bfloat8_b, layout=ttnn.TILE_LAYOUT, device=device, cache_file_name=tmp_path / "sub" / "w")
+    file = tmp_path / "sub" / "w_dtype_BFLOAT8_B_layout_TILE.bin"
+    assert file.exists() and first.dtype == ttnn.bfloat8_b and first.layout == ttnn.TILE_LAYOUT and first.device() == device
+    second = ttnn.as_tensor(torch.zeros_like(big), dtype=ttnn.bfloat8_b, layout=ttnn.TILE_LAYOUT, device=device, cache_file_name=tmp_path / "sub" / "w")
+    assert torch.equal(second._buf, first._buf)                    # taken from the file, not from the (different) torch tensor
+    assert ttnn.is_tensor_storage_on_device(second)
+
+
+# ---- MLP blocks -------------------------------------------------------------------------------------------------------
+def falcon_reference(x, w1, w2):
+    h = bf16_round(torch.nn.functional.gelu(x @ w1))
+    return h @ w2
+
+
+@pytest.mark.parametrize("seq,hidden", [(32, 128), (128, 256), (32, 4544)])
+def test_falcon_mlp_block(oracle, device, tmp_path, seq, hidden):
+    import tt_lib
+    import ttnn
+    from blocks import TtFalconMLP, falcon_mlp_model_config
+
+    torch.manual_seed(0)
+    state = {"transformer.h.0.mlp.dense_h_to_4h.weight": torch.randn(4 * hidden, hidden) * 0.02,
+             "transformer.h.0.mlp.dense_4h_to_h.weight": torch.randn(hidden, 4 * hidden) * 0.02}
+    x = ((torch.rand(1, 1, seq, hidden) * 2) - 1).to(torch.bfloat16)
+    cache = tmp_path if hidden <= 256 else None
+    block = TtFalconMLP([device], state, "transformer.h", 0, hidden, falcon_mlp_model_config(), tt_cache_path=cache)
+    assert block.dense_h_to_4h_weights[0].dtype == tt_lib.tensor.DataType.BFLOAT8_B
+    tx = ttnn.from_torch(x, dtype=ttnn.bfloat16, layout=ttnn.TILE_LAYOUT, device=device)
+    out = block([tx])[0]
+    assert tuple(out.shape) == (1, 1, seq, hidden) and out.dtype == ttnn.bfloat16
+    got = ttnn.to_torch(out)[0, 0]
+    w1 = state["transformer.h.0.mlp.dense_h_to_4h.weight"].t()
+    w2 = state["transformer.h.0.mlp.dense_4h_to_h.weight"].t()
+    want_q = falcon_reference(x[0, 0].double(), quantised(oracle, ttnn.bfloat8_b, w1), quantised(oracle, ttnn.bfloat8_b, w2))
+    assert pcc(got, want_q) >= 0.9999
+    want = torch.nn.functional.gelu(x[0, 0].float() @ w1) @ w2         # torch_functional_falcon_mlp with unquantised weights
+    assert pcc(got, want) >= 0.99
+    if cache is not None:                                              # a second block reads the cached tensor files
+        again = TtFalconMLP([device], {k: torch.zeros_like(v) for k, v in state.items()}, "transformer.h", 0, hidden,
+                            falcon_mlp_model_config(), tt_cache_path=cache)
+        assert torch.equal(again.dense_4h_to_h_weights[0]._buf, block.dense_4h_to_h_weights[0]._buf)
+
+
+@pytest.mark.parametrize("seq,dim,hidden_dim,name", [(32, 128, 352, "bfloat8_b"), (64, 256, 704, "bfloat4_b"), (32, 4096, 14336, "bfloat4_b")])
+def test_mistral_mlp_block(oracle, device, seq, dim, hidden_dim, name):
+    import ttnn
+    from blocks import TtMistralMLP, mistral_mlp_model_config
+
+    dtype = getattr(ttnn, name)
+    torch.manual_seed(1)
+    state = {"layers.0.feed_forward.w1.weight": torch.randn(hidden_dim, dim) * 0.02,
+             "layers.0.feed_forward.w2.weight": torch.randn(dim, hidden_dim) * 0.02,
+             "layers.0.feed_forward.w3.weight": torch.randn(hidden_dim, dim) * 0.02}
+    x = torch.randn(1, 1, seq, dim).to(torch.bfloat16)
+    block = TtMistralMLP(device, None, state, None, 0, dtype, mistral_mlp_model_config())
+    out = block(ttnn.from_torch(x, dtype=ttnn.bfloat16, layout=ttnn.TILE_LAYOUT, device=device))
+    assert tuple(out.shape) == (1, 1, seq, dim)
+    got = ttnn.to_torch(out)[0, 0]
+    w1, w2, w3 = (state[f"layers.0.feed_forward.{n}.weight"].t() for n in ("w1", "w2", "w3"))
+    xd = x[0, 0].double()
+    gate = bf16_round(torch.nn.functional.silu(xd @ quantised(oracle, dtype, w1)))
+    up = bf16_round(xd @ quantised(oracle, dtype, w3))
+    want_q = bf16_round(gate * up) @ quantised(oracle, dtype, w2)
+    assert pcc(got, want_q) >= 0.9999
+    want = (torch.nn.functional.silu(x[0, 0].float() @ w1) * (x[0, 0].float() @ w3)) @ w2
+    assert pcc(got, want) >= (0.99 if name == "bfloat8_b" else 0.95)   # 3-bit mantissas: the quantisation itself costs that much

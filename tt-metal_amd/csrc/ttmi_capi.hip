@@ -121,4 +121,11 @@ int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, u
     return matmul_bfp(args, (hipStream_t)stream);
 }
 
+int ttmi_eltwise_bf16(int op, const void *a, const void *b, float scalar, void *c, size_t count, void *stream) {
+    if (count && (!a || !c)) return fail(TTMI_ERR_INVALID_ARGUMENT, "eltwise: null pointer");
+    if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15u)
+        return fail(TTMI_ERR_INVALID_ARGUMENT, "eltwise: a, b and c must be 16-byte aligned");
+    return eltwise_bf16(op, a, b, scalar, c, count, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -23,6 +23,8 @@ int codec_unpack_tensor(int fmt, const uint32_t *words, uint32_t batch, uint32_t
 int codec_relayout(bool to_tiles, const void *src, uint32_t elem, uint32_t batch, uint32_t h, uint32_t w, void *dst,
                    hipStream_t st);
 
+int eltwise_bf16(int op, const void *a, const void *b, float scalar, void *c, size_t count, hipStream_t st);
+
 struct MatmulArgs {
     const void *a; int a_layout;
     const uint32_t *b; int b_fmt;

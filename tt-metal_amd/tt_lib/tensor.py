@@ -8,6 +8,7 @@ exactly as the reference lays them out (packed uint32 words for block-float), de
 from __future__ import annotations
 
 import enum
+import struct
 from typing import Optional, Sequence
 
 import torch
@@ -346,3 +347,194 @@ def bmm(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConf
         untilize_out: bool = False) -> Tensor:
     """tt_lib.tensor.bmm: [B, C, M, K] x [B, C, K, N] (tt_lib_bindings_tensor_custom_bmm_ops.cpp:66-81, bmm_op.hpp:425)."""
     return _matmul(input_a, input_b, bcast_batch=False, op="bmm")
+
+
+# ---- fused activations and the Falcon matmuls (bmm_op.cpp:747-807) -------------------------------------------------
+class FusibleActivation(enum.IntEnum):  # UnaryOpType, tt_eager/tt_dnn/op_library/eltwise_unary/eltwise_unary_op.hpp:17-78
+    GELU = 2
+    RELU = 3
+    SILU = 48
+
+
+class FusibleActivationWithParam:
+    """UnaryWithParam (tt_lib_bindings_tensor.cpp:113-128): an activation and its parameter; for GELU the parameter selects the
+    Tensix fast-and-approximate mode, which has no counterpart here (the exact erf form is used either way)."""
+
+    def __init__(self, op_type, param: float = 0.0):
+        if isinstance(op_type, (tuple, list)):
+            op_type, param = op_type[0], (op_type[1] if len(op_type) > 1 else 0.0)
+        self.op_type, self.param = FusibleActivation(op_type), float(param)
+
+
+_FUSED = {FusibleActivation.GELU: capi.ACT_GELU, FusibleActivation.RELU: capi.ACT_RELU, FusibleActivation.SILU: capi.ACT_SILU}
+
+
+def _fused_activation_code(fused_activation) -> int:
+    if fused_activation is None:
+        return capi.ACT_NONE
+    if not isinstance(fused_activation, FusibleActivationWithParam):
+        fused_activation = FusibleActivationWithParam(fused_activation)
+    return _FUSED[fused_activation.op_type]
+
+
+def falcon_fused_qkv_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None,
+                            output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:747-750: A x B with B broadcast over the batch."""
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, output_dtype=output_dtype, op="falcon_fused_qkv_matmul")
+
+
+def falcon_selfout_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None,
+                          output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:752-755."""
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, output_dtype=output_dtype, op="falcon_selfout_matmul")
+
+
+def falcon_dense_4h_to_h_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None,
+                                output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None,
+                                packer_l1_acc: Optional[bool] = None) -> Tensor:
+    """bmm_op.cpp:757-771 (packer_l1_acc is a Tensix accumulation mode: accepted, without effect)."""
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, output_dtype=output_dtype, op="falcon_dense_4h_to_h_matmul")
+
+
+def falcon_dense_h_to_4h_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None, fused_activation=None,
+                                output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:773-791: above 1024 rows the reference accepts only [1, 1, seq, 4544] x [1, 1, 4544, 18176] without a
+    fused activation; the same conditions are rejected here."""
+    seq_len = input_a._padded[-2]
+    if seq_len > 1024:
+        if fused_activation is not None:
+            raise RuntimeError("TT_FATAL: not fused_activation.has_value()")
+        if seq_len % 32:
+            raise RuntimeError("TT_FATAL: Falcon mm's seq_len must be a multiple of 32!")
+        if tuple(input_a._padded) != (1, 1, seq_len, 4544) or tuple(input_b._padded) != (1, 1, 4544, 18176):
+            raise RuntimeError("TT_FATAL: Unsupported input shape")
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, activation=_fused_activation_code(fused_activation),
+                   output_dtype=output_dtype, op="falcon_dense_h_to_4h_matmul")
+
+
+def falcon_lm_head_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None,
+                          output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:793-807."""
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, output_dtype=output_dtype, op="falcon_lm_head_matmul")
+
+
+# ---- elementwise (eltwise_binary_op.hpp:108-140, eltwise_unary_op.hpp) ----------------------------------------------
+def _as_bf16_buffer(t: Tensor) -> "torch.Tensor":
+    """Flat bf16 device buffer in the tensor's own element order; block-float operands are expanded (exactly)."""
+    if t.storage_type() != StorageType.DEVICE:
+        raise RuntimeError("TT_FATAL: Operands to eltwise ops need to be on device!")
+    if t.dtype in _BFP:
+        words = capi.unpack_chunks(int(t.dtype), t._buf, False)      # fp32, same order as the packed data
+        return words.to(torch.bfloat16)                               # <= 7 significant bits: exact
+    if t.dtype != DataType.BFLOAT16:
+        raise RuntimeError(f"TT_FATAL: Unsupported data format {t.dtype.name} (BFLOAT16, BFLOAT8_B, BFLOAT4_B)")
+    return t._buf.reshape(-1)
+
+
+def _eltwise(op: int, a: Tensor, b=None, scalar: float = 0.0, name: str = "eltwise") -> Tensor:
+    if b is not None:
+        if tuple(a._padded) != tuple(b._padded):
+            raise RuntimeError(f"TT_FATAL: {name}: input shapes must be the same ({tuple(a._padded)} vs {tuple(b._padded)}); "
+                               "broadcast forms are not part of this build")
+        if a.layout != b.layout:
+            raise RuntimeError(f"TT_FATAL: {name}: inputs must have the same layout")
+    with torch.cuda.device(a._device.torch_device):
+        out = capi.eltwise(op, _as_bf16_buffer(a), _as_bf16_buffer(b) if b is not None else None, scalar)
+        if a.dtype in _BFP:      # output takes input a's dtype (eltwise_binary_op.hpp:124-126)
+            out = capi.pack_chunks(int(a.dtype), out.float(), False)
+        elif a.layout == Layout.ROW_MAJOR:
+            out = out.view(a._padded)
+    return a._like(out)
+
+
+def add(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    return _eltwise(capi.OP_ADD, input_a, input_b, name="add")
+
+
+def sub(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    return _eltwise(capi.OP_SUB, input_a, input_b, name="sub")
+
+
+def mul(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    return _eltwise(capi.OP_MUL, input_a, input_b, name="mul")
+
+
+def add_unary(input_a: Tensor, scalar: float, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    return _eltwise(capi.OP_ADD, input_a, None, scalar, name="add_unary")
+
+
+def mul_unary(input_a: Tensor, scalar: float, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    return _eltwise(capi.OP_MUL, input_a, None, scalar, name="mul_unary")
+
+
+def gelu(input_a: Tensor, fast_and_approx: bool = True, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    return _eltwise(capi.OP_GELU, input_a, name="gelu")
+
+
+def relu(input_a: Tensor, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    return _eltwise(capi.OP_RELU, input_a, name="relu")
+
+
+def silu(input_a: Tensor, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    return _eltwise(capi.OP_SILU, input_a, name="silu")
+
+
+# ---- tensor files (tt_eager/tensor/serialization.cpp:86-141) --------------------------------------------------------
+# File = the raw bytes of `Shape` (tt_eager/tensor/types.hpp:46-63,118-121 as the x86-64 System V ABI lays it out), then
+# DataType and Layout as 32-bit integers, then the element count as a 64-bit integer and the elements:
+#   offset   0  u64      Shape::rank_
+#            8  u32 x 8  Shape::dimensions_ (the shape WITH padding; unused entries 0)
+#           40  u64      Padding::rank_
+#           48  {u64 front, u64 back} x 8   Padding::pad_dimensions_ (back = padded - logical size)
+#          176  i32      Padding::pad_value_ (PadValue::Any = 0), 4 bytes of struct padding
+#          184  i32      DataType          188  i32  Layout
+#          192  u64      number of elements (uint32 words for block-float and UINT32, 2-byte elements for BFLOAT16 / UINT16)
+#          200  elements
+_FILE_HEADER = struct.Struct("<Q8IQ16QiiiiQ")
+_FILE_ELEMENT = {DataType.BFLOAT16: torch.bfloat16, DataType.UINT16: torch.int16, DataType.FLOAT32: torch.float32,
+                 DataType.UINT32: torch.int32, DataType.BFLOAT8_B: torch.int32, DataType.BFLOAT4_B: torch.int32}
+
+
+def dump_tensor(file_name: str, tensor: Tensor) -> None:
+    if tensor.storage_type() == StorageType.DEVICE:
+        raise RuntimeError("TT_THROW: Device storage isn't supported")     # serialization.cpp:113-115
+    rank = len(tensor._padded)
+    if rank > 8:
+        raise RuntimeError("TT_THROW: Shape supports up to 8 dimensions")
+    dims = list(tensor._padded) + [0] * (8 - rank)
+    pads = []
+    for i in range(8):
+        pads += [0, (tensor._padded[i] - tensor._shape[i]) if i < rank else 0]
+    flat = tensor._buf.contiguous().reshape(-1)
+    header = _FILE_HEADER.pack(rank, *dims, rank, *pads, 0, 0, int(tensor.dtype), int(tensor.layout), flat.numel())
+    assert len(header) == 200
+    with open(file_name, "wb") as f:
+        f.write(header)
+        f.write(flat.view(torch.uint8).numpy().tobytes())
+
+
+def load_tensor(file_name: str) -> Tensor:
+    try:
+        f = open(file_name, "rb")
+    except OSError:
+        raise RuntimeError(f'Cannot open "{file_name}"')                 # serialization.cpp:122-125
+    with f:
+        raw = f.read(200)
+        if len(raw) != 200:
+            raise RuntimeError(f'"{file_name}" is too short to hold a tensor header')
+        fields = _FILE_HEADER.unpack(raw)
+        rank, dims, pads = fields[0], fields[1:9], fields[10:26]
+        dtype, layout, count = DataType(fields[28]), Layout(fields[29]), fields[30]
+        if rank > 8 or dtype not in _FILE_ELEMENT:
+            raise RuntimeError("TT_THROW: Unsupported DataType")
+        elem = _FILE_ELEMENT[dtype]
+        nbytes = count * torch.empty(0, dtype=elem).element_size()
+        payload = f.read(nbytes)
+        if len(payload) != nbytes:
+            raise RuntimeError(f'"{file_name}" ends inside the tensor data')
+    padded = tuple(int(d) for d in dims[:rank])
+    logical = tuple(int(d) - int(pads[2 * i]) - int(pads[2 * i + 1]) for i, d in enumerate(padded))
+    buf = torch.frombuffer(bytearray(payload), dtype=torch.uint8).view(elem)
+    if layout == Layout.ROW_MAJOR and dtype not in _BFP:
+        buf = buf.view(padded)
+    return Tensor(None, _raw=(buf, logical, padded, dtype, layout, None))

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libttmi.so")
 BFLOAT16, FLOAT32, UINT32, BFLOAT8_B, BFLOAT4_B, UINT16 = 0, 1, 2, 3, 4, 6
 ROW_MAJOR, TILE = 0, 1
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_SILU = 0, 1, 2, 3
+OP_ADD, OP_SUB, OP_MUL, OP_RELU, OP_GELU, OP_SILU = 0, 1, 2, 17, 18, 19
 TILE_BYTES = {BFLOAT8_B: 1088, BFLOAT4_B: 576, BFLOAT16: 2048, UINT16: 2048, FLOAT32: 4096, UINT32: 4096}
 
 # every symbol include/ttmi.h declares
@@ -22,6 +23,7 @@ SYMBOLS = (
     "ttmi_pack_fp32_vec_as_bfp_tiles", "ttmi_unpack_bfp_tiles_into_float_vec",
     "ttmi_pack_rowmajor_as_bfp_tiles", "ttmi_unpack_bfp_tiles_as_rowmajor",
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
+    "ttmi_eltwise_bf16",
 )
 
 _lib = None
@@ -60,6 +62,8 @@ def lib() -> ctypes.CDLL:
         L.ttmi_matmul_bfp_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
         L.ttmi_matmul_bfp.restype = i32
         L.ttmi_matmul_bfp.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, sz, vp]
+        L.ttmi_eltwise_bf16.restype = i32
+        L.ttmi_eltwise_bf16.argtypes = [i32, vp, vp, ctypes.c_float, vp, sz, vp]
         _lib = L
     return _lib
 
@@ -187,3 +191,18 @@ def matmul_bfp(a, a_layout: int, b_words, b_fmt: int, batch: int, b_batch: int, 
     if c_layout == ROW_MAJOR:
         return c.view(batch, m, n)
     return c
+
+
+def eltwise(op: int, a, b=None, scalar: float = 0.0):
+    """op(a, b) (or op(a, scalar), or a unary op of a) on cuda bf16 tensors with equal element counts; returns a tensor like a."""
+    import torch
+
+    if a.dtype != torch.bfloat16 or (b is not None and b.dtype != torch.bfloat16):
+        raise RuntimeError("eltwise: operands must be bfloat16")
+    if b is not None and b.numel() != a.numel():
+        raise RuntimeError("eltwise: operands must have the same number of elements")
+    a = a.contiguous()
+    b = b.contiguous() if b is not None else None
+    out = torch.empty_like(a)
+    check(lib().ttmi_eltwise_bf16(op, _dev(a), _dev(b) if b is not None else None, float(scalar), _dev(out), a.numel(), _stream()))
+    return out
