@@ -113,4 +113,12 @@ PYBIND11_MODULE(_ttmi, m) {
           py::arg("n"), py::arg("bias") = 0, py::arg("activation") = py::none(), py::arg("c") = 0, py::arg("c_layout") = (int)TTMI_TILE,
           py::arg("c_dtype") = (int)TTMI_BFLOAT16, py::arg("workspace") = 0, py::arg("workspace_bytes") = 0, py::arg("stream") = 0,
           "ttnn.linear / ttnn.matmul with block-float weights, ttnn/cpp/ttnn/operations/matmul.hpp:44-214");
+    // ttnn.mul / add / sub and gelu / relu / silu on bf16 tensors of equal shape (ttnn/ttnn/operations/binary.py:321-424)
+    m.def("eltwise",
+          [](int op, uintptr_t a, uintptr_t b, float scalar, uintptr_t c, size_t count, uintptr_t stream) {
+              py::gil_scoped_release release;
+              check(ttmi_eltwise_bf16(op, ptr<const void>(a), ptr<const void>(b), scalar, ptr<void>(c), count, ptr<void>(stream)));
+          },
+          py::arg("op"), py::arg("a"), py::arg("b") = 0, py::arg("scalar") = 0.0f, py::arg("c") = 0, py::arg("count") = 0, py::arg("stream") = 0,
+          "c = op(a, b | scalar), eltwise_binary_op.hpp:108-140 / eltwise_unary_op.hpp:17-90");
 }
