@@ -24,6 +24,7 @@
 #include <stdlib.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "bfp_dequant.h"
 #include "ttmi_internal.h"
@@ -48,8 +49,14 @@ struct MatmulDev {
 constexpr int GROUP_TILES = 2;                       // n tiles per output group
 constexpr int GROUP_COLS = GROUP_TILES * 32;
 constexpr int WAVES = 4;
-constexpr int WGS_PER_CU = 3;                        // workgroups of 4 wavefronts per CU (registers and LDS allow 3)
-constexpr int STAGES = 3;                            // LDS ring per wavefront = units requested ahead of the arithmetic
+#ifndef TTMI_STREAM_WGS_PER_CU
+#define TTMI_STREAM_WGS_PER_CU 3
+#endif
+#ifndef TTMI_STREAM_STAGES
+#define TTMI_STREAM_STAGES 3
+#endif
+constexpr int WGS_PER_CU = TTMI_STREAM_WGS_PER_CU;   // workgroups of 4 wavefronts per CU (registers and LDS allow 3)
+constexpr int STAGES = TTMI_STREAM_STAGES;           // LDS ring per wavefront = units requested ahead of the arithmetic
 constexpr int A_LOADS = 2;                           // activation loads per unit (rows c and c + 16 of the band)
 constexpr int REDUCE_BYTES = WAVES * 32 * 64 * 4;    // every wavefront lays out its 32 accumulator registers
 constexpr size_t SLOT_BYTES = 32 * GROUP_COLS * sizeof(float);
@@ -98,6 +105,18 @@ __device__ __forceinline__ uint32_t workgroup_of(const MatmulDev &p, uint32_t un
 // with the highest index writes its sums to its own slot; that last one waits for each slot to lose its SLOT_EMPTY
 // pattern, adds the slots in workgroup order to its own sums (so the result does not depend on timing), applies the
 // epilogue, stores, and puts the empty pattern back.
+template <int... Is, typename Fn> __device__ __forceinline__ void static_for(std::integer_sequence<int, Is...>, Fn fn) {
+    (fn(std::integral_constant<int, Is>{}), ...);
+}
+// waits until at most min(younger, MOST) * PER requests are in flight
+template <int MOST, int PER> __device__ __forceinline__ void wait_for_younger(uint32_t younger) {
+    if constexpr (MOST == 0) {
+        wait_vmcnt<0>();
+    } else {
+        if (younger >= (uint32_t)MOST) wait_vmcnt<MOST * PER>(); else wait_for_younger<MOST - 1, PER>(younger);
+    }
+}
+
 template <int W, int ACT>
 __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const MatmulDev p) {
     using F = Wfmt<W>;
@@ -217,32 +236,27 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
         // units after it may still be in flight: min(STAGES - 1, total - 1 - i) of them.
         const uint32_t span = k_end - k_begin;
         const uint32_t total = span > (uint32_t)wave ? (span - wave + WAVES - 1) / WAVES : 0;
-        static_assert(STAGES == 3, "the unrolled pipeline below is written for three stages");
-        using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>; using S2 = std::integral_constant<int, 2>;
+        using Last = std::integral_constant<int, STAGES - 1>;
+        constexpr auto stages = std::make_integer_sequence<int, STAGES>{};
         uint32_t i = 0;
         if (total >= 2 * STAGES) {
             // steady state: every unit worked on here has a successor to request, so the number of requests in
             // flight at each wait is a constant the compiler can see (no conditional request on the way in)
-            fetch(S0{}); fetch(S1{}); fetch(S2{});
+            static_for(stages, [&](auto s) __attribute__((always_inline)) { fetch(s); });
 #pragma unroll 1
-            for (; i + 2 * STAGES <= total; i += STAGES) {
-                work(S0{}, S2{}, true);
-                work(S1{}, S2{}, true);
-                work(S2{}, S2{}, true);
-            }
+            for (; i + 2 * STAGES <= total; i += STAGES)
+                static_for(stages, [&](auto s) __attribute__((always_inline)) { work(s, Last{}, true); });
         } else {
-            if (total > 0) fetch(S0{});
-            if (total > 1) fetch(S1{});
-            if (total > 2) fetch(S2{});
+            static_for(stages, [&](auto s) __attribute__((always_inline)) { if (total > (uint32_t)decltype(s)::value) fetch(s); });
         }
         // at most 2 * STAGES - 1 units are left, starting in stage 0
-        auto tail = [&](auto stage_tag, uint32_t at) __attribute__((always_inline)) {
+        static_for(std::make_integer_sequence<int, 2 * STAGES - 1>{}, [&](auto j) __attribute__((always_inline)) {
+            constexpr int J = decltype(j)::value;
+            const uint32_t at = i + J;
             if (at >= total) return;
-            const uint32_t after = total - 1 - at;
-            if (after >= 2) wait_vmcnt<2 * (NLOAD + A_LOADS)>(); else if (after == 1) wait_vmcnt<NLOAD + A_LOADS>(); else wait_vmcnt<0>();
-            work(stage_tag, std::integral_constant<int, -1>{}, at + STAGES < total);
-        };
-        tail(S0{}, i); tail(S1{}, i + 1); tail(S2{}, i + 2); tail(S0{}, i + 3); tail(S1{}, i + 4);
+            wait_for_younger<STAGES - 1, NLOAD + A_LOADS>(total - 1 - at);
+            work(std::integral_constant<int, J % STAGES>{}, std::integral_constant<int, -1>{}, at + STAGES < total);
+        });
 
         wait_vmcnt<0>();   // nothing in flight any more (already true; also what the build-time ISA check keys on)
         // ---- add the four wavefronts' partial sums through LDS --------------------------------------------------
