@@ -188,3 +188,37 @@ def test_mistral_mlp_block(oracle, device, seq, dim, hidden_dim, name):
     assert pcc(got, want_q) >= 0.9999
     want = (torch.nn.functional.silu(x[0, 0].float() @ w1) * (x[0, 0].float() @ w3)) @ w2
     assert pcc(got, want) >= (0.99 if name == "bfloat8_b" else 0.95)   # 3-bit mantissas: the quantisation itself costs that much
+
+
+# ---- device-resident dtype changes ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["bfloat8_b", "bfloat4_b"])
+def test_to_layout_with_dtype_and_clone(oracle, device, name):
+    """ttnn.to_layout(.., TILE_LAYOUT, dtype=) on a bf16 device tensor (ttnn/ttnn/operations/core.py:684-711) and ttnn.clone
+    (core.py:819-839).  The Tensix packer's rounding is not pinned by the sources at hand; checked here: the result is the
+    reference's HOST packer applied once to the tile-ordered values (parity with the device op itself: unpinned)."""
+    import ttnn
+
+    dtype = getattr(ttnn, name)
+    fmt = int(dtype)
+    torch.manual_seed(21)
+    x = torch.randn(2, 64, 96).to(torch.bfloat16)
+    t = ttnn.from_torch(x, layout=ttnn.ROW_MAJOR_LAYOUT, device=device)
+    packed = ttnn.to_layout(t, ttnn.TILE_LAYOUT, dtype=dtype)
+    assert packed.dtype == dtype and packed.layout == ttnn.TILE_LAYOUT and ttnn.is_tensor_storage_on_device(packed)
+    tiles = oracle.tilize_nchw_4faces(x.float().numpy()[None])
+    want = oracle.pack_fp32_vec_as_bfp_tiles(fmt, tiles, False)
+    assert np.array_equal(packed._buf.cpu().numpy().view(np.uint32), want)
+    # clone: bf16 tiles -> block-float gives the same words; block-float -> bf16 gives the unpacked values exactly
+    tiled = ttnn.to_layout(t, ttnn.TILE_LAYOUT)
+    cloned = ttnn.clone(tiled, ttnn.DRAM_MEMORY_CONFIG, dtype)
+    assert cloned.layout == ttnn.TILE_LAYOUT and torch.equal(cloned._buf, packed._buf)
+    back = ttnn.clone(cloned, ttnn.DRAM_MEMORY_CONFIG, ttnn.bfloat16)
+    assert back.dtype == ttnn.bfloat16 and torch.equal(ttnn.to_torch(back).float(), ttnn.to_torch(cloned))
+    same = ttnn.clone(tiled, ttnn.DRAM_MEMORY_CONFIG, None)
+    assert same.dtype == ttnn.bfloat16 and torch.equal(same._buf, tiled._buf) and same._buf.data_ptr() != tiled._buf.data_ptr()
+    with pytest.raises(RuntimeError, match="Unsupported datatype conversion"):
+        ttnn.to_layout(ttnn.from_torch(x, layout=ttnn.ROW_MAJOR_LAYOUT), ttnn.TILE_LAYOUT, dtype=dtype)       # not on the device
+    with pytest.raises(RuntimeError, match="Unsupported datatype conversion"):
+        ttnn.to_layout(tiled, ttnn.ROW_MAJOR_LAYOUT, dtype=dtype)
+    with pytest.raises(RuntimeError, match="on device"):
+        ttnn.clone(ttnn.from_torch(x), ttnn.DRAM_MEMORY_CONFIG, dtype)

@@ -538,3 +538,55 @@ def load_tensor(file_name: str) -> Tensor:
     if layout == Layout.ROW_MAJOR and dtype not in _BFP:
         buf = buf.view(padded)
     return Tensor(None, _raw=(buf, logical, padded, dtype, layout, None))
+
+
+# ---- device-resident dtype changes (tt_eager/tt_dnn/op_library/copy/copy_op.hpp:42-44, tilize/tilize_op.hpp:71-73) -------
+# On Tensix the conversion happens in the packer of a data-movement kernel, whose rounding is not stated in the sources at
+# hand; here the values pass through the host packers' arithmetic (one pack of the tile-ordered values), which is what
+# the reference's own host-side typecast of a block-float tensor does.
+def typecast(input_tensor: Tensor, dtype: DataType, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    dtype = DataType(dtype)
+    if input_tensor.storage_type() != StorageType.DEVICE:
+        raise RuntimeError("TT_FATAL: Operands to copy need to be on device!")
+    if dtype == input_tensor.dtype:
+        return input_tensor._like(input_tensor._buf.clone())
+    floats = (DataType.BFLOAT16, DataType.FLOAT32) + _BFP
+    if input_tensor.dtype not in floats or dtype not in floats:
+        raise RuntimeError(f"TT_FATAL: typecast between {input_tensor.dtype.name} and {dtype.name} is not supported")
+    if (input_tensor.dtype in _BFP or dtype in _BFP) and input_tensor.layout != Layout.TILE:
+        raise RuntimeError("TT_FATAL: block-float tensors on device are in TILE layout")
+    with torch.cuda.device(input_tensor._device.torch_device):
+        if input_tensor.dtype in _BFP:
+            values = capi.unpack_chunks(int(input_tensor.dtype), input_tensor._buf, False)      # fp32 in tile order, exact
+        else:
+            values = input_tensor._buf.reshape(-1).float()
+        if dtype in _BFP:
+            out = capi.pack_chunks(int(dtype), values, False)
+        else:
+            out = values.to(_TORCH[dtype])
+            if input_tensor.layout == Layout.ROW_MAJOR:
+                out = out.view(input_tensor._padded)
+    return input_tensor._like(out, dtype=dtype)
+
+
+def clone(input_tensor: Tensor, output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    if output_dtype is None or DataType(output_dtype) == input_tensor.dtype:
+        if input_tensor.storage_type() != StorageType.DEVICE:
+            raise RuntimeError("TT_FATAL: Operands to copy need to be on device!")
+        return input_tensor._like(input_tensor._buf.clone())
+    return typecast(input_tensor, output_dtype, output_mem_config)
+
+
+def tilize(input_tensor: Tensor, output_mem_config: Optional[MemoryConfig] = None, use_multicore: bool = False,
+           output_dtype: Optional[DataType] = None) -> Tensor:
+    """tilize_op.hpp:71-73: ROW_MAJOR -> TILE on the device, optionally into another dtype (bf16 -> block-float)."""
+    if input_tensor.storage_type() != StorageType.DEVICE:
+        raise RuntimeError("TT_FATAL: Operands to tilize need to be on device!")
+    if input_tensor.layout != Layout.ROW_MAJOR:
+        raise RuntimeError("TT_FATAL: Can only tilize row major data")
+    if input_tensor._padded[-1] % 32 or (len(input_tensor._padded) > 1 and input_tensor._padded[-2] % 32):
+        raise RuntimeError("TT_FATAL: tilize needs height and width to be multiples of 32")
+    tiles = input_tensor.to(Layout.TILE)
+    if output_dtype is None or DataType(output_dtype) == tiles.dtype:
+        return tiles
+    return typecast(tiles, output_dtype, output_mem_config)

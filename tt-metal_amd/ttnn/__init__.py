@@ -115,7 +115,7 @@ def is_tensor_storage_on_device(tensor: Tensor) -> bool:
     return tensor.storage_type() in (DEVICE_STORAGE_TYPE, MULTI_DEVICE_STORAGE_TYPE)
 
 
-from .core import from_torch, to_torch, to_layout, to_device, from_device, reshape, deallocate, unsqueeze_to_4D  # noqa: E402
+from .core import from_torch, to_torch, to_layout, to_device, from_device, reshape, deallocate, unsqueeze_to_4D, clone  # noqa: E402
 from .matmul import matmul, linear  # noqa: E402
 from .elementwise import mul, multiply, add, sub, subtract, gelu, relu, silu  # noqa: E402
 from .files import load_tensor, dump_tensor, as_tensor, get_memory_config  # noqa: E402

@@ -6,6 +6,7 @@ from typing import Optional, Tuple, Union
 import torch
 
 import ttnn
+import tt_lib.tensor as ttl_tensor
 from tt_lib.tensor import DataType, Layout, Tensor, Device, _BFP, _TORCH, _pad32, _run_on_gpu
 from ttmi import capi
 
@@ -88,8 +89,14 @@ def to_layout(tensor: Tensor, layout: Layout, dtype: Optional[DataType] = None, 
     """core.py:609-803: TILE pads the last two dimensions to multiples of 32 with zeros and keeps the logical shape."""
     if layout not in (ttnn.ROW_MAJOR_LAYOUT, ttnn.TILE_LAYOUT):
         raise RuntimeError(f"Unsupported layout: {layout}")
+    if tensor.layout == layout and (dtype is None or dtype == tensor.dtype):
+        return tensor
     if dtype is not None and dtype != tensor.dtype:
-        raise RuntimeError("ttnn.to_layout: changing dtype with the layout is not supported by this build")
+        # core.py:684-685, 706-711: only on the device and only towards TILE_LAYOUT (tilize with an output dtype)
+        if not ttnn.is_tensor_storage_on_device(tensor) or layout != ttnn.TILE_LAYOUT:
+            raise RuntimeError(f"Unsupported datatype conversion to {dtype}")
+        tiles = to_layout(tensor, layout) if tensor.layout != layout else tensor
+        return ttl_tensor.typecast(tiles, dtype)
     if tensor.layout == layout:
         return tensor
     logical, padded = tuple(tensor._shape), tuple(tensor._padded)
@@ -135,3 +142,10 @@ def unsqueeze_to_4D(tensor: Tensor) -> Tensor:
         raise RuntimeError("Tensor cannot have more than 4 dimensions!")
     lead = (1,) * (4 - rank)
     return tensor.reshape(ttnn.Shape(lead + tuple(tensor._shape), lead + tuple(tensor._padded)))
+
+
+def clone(tensor: Tensor, memory_config=None, dtype: Optional[DataType] = None) -> Tensor:
+    """core.py:819-839: a copy of a device tensor, optionally in another dtype; the layout stays."""
+    if not isinstance(tensor, Tensor) or not ttnn.is_tensor_storage_on_device(tensor):
+        raise RuntimeError("ttnn.clone: Tensor must be on device!")
+    return ttl_tensor.clone(tensor, output_mem_config=memory_config, output_dtype=dtype)
