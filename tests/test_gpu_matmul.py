@@ -208,6 +208,40 @@ def test_expanded_weights_in_a_caller_workspace(oracle, monkeypatch):
                         workspace=torch.empty(need - 256, dtype=torch.uint8, device="cuda"))
 
 
+def test_decode_gemm_in_a_hip_graph(oracle):
+    """A caller that captures the stream: with its own workspace the call records kernels only (the slots are marked empty by
+    a fill kernel, no memset node).  Replayed several times with eager work and synchronisation in between, every replay
+    must give the eager result."""
+    m, k, n = 32, 2048, 320
+    a_bits = workloads.activations_bf16(m, k, seed=90)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=91), BFP8)
+    a = bf16_dev(a_bits)
+    need = capi.lib().ttmi_matmul_bfp_workspace_bytes(1, m, k, n, BFP8)
+    assert need > 0
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    eager = capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n, workspace=ws).clone()
+    check_against_reference(eager.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+    out = torch.zeros(m * n, dtype=torch.bfloat16, device="cuda")
+    L = capi.lib()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            capi.check(L.ttmi_matmul_bfp(a.data_ptr(), capi.ROW_MAJOR, words.data_ptr(), BFP8, 1, 1, m, k, n, None, capi.ACT_NONE,
+                                         out.data_ptr(), capi.ROW_MAJOR, capi.BFLOAT16, ws.data_ptr(), need, side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(4):
+        out.zero_()
+        ws.fill_(replay)                                        # the workspace may hold anything between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(1, m, n).view(torch.int16), eager.view(torch.int16)), replay
+        other = capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)      # eager work between the replays
+        assert torch.equal(other.view(torch.int16), eager.view(torch.int16))
+
+
 @pytest.mark.parametrize("name,m,k,n,fmt,batch", workloads.DECODE_FALCON + workloads.DECODE_MISTRAL)
 def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch):
     a_bits = workloads.activations_bf16(m, k, seed=80)

@@ -105,6 +105,12 @@ __device__ __forceinline__ uint32_t workgroup_of(const MatmulDev &p, uint32_t un
 // with the highest index writes its sums to its own slot; that last one waits for each slot to lose its SLOT_EMPTY
 // pattern, adds the slots in workgroup order to its own sums (so the result does not depend on timing), applies the
 // epilogue, stores, and puts the empty pattern back.
+// every word of a caller's workspace becomes SLOT_EMPTY
+__global__ __launch_bounds__(256) void fill_slots_kernel(u32x4 *slots, uint32_t chunks) {
+    const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < chunks; i += gridDim.x * 256) slots[i] = empty;
+}
+
 template <int... Is, typename Fn> __device__ __forceinline__ void static_for(std::integer_sequence<int, Is...>, Fn fn) {
     (fn(std::integral_constant<int, Is>{}), ...);
 }
@@ -468,8 +474,11 @@ int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) {
     } else if (x.workspace) {
         if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
         if (reinterpret_cast<uintptr_t>(x.workspace) & 255u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 256-byte aligned");
-        // a caller's buffer may hold anything: mark every slot of this launch empty
-        if (int rc = check_hip(hipMemsetAsync(x.workspace, 0xff, need, st), "hipMemsetAsync(slots)")) return rc;
+        // a caller's buffer may hold anything: mark every slot of this launch empty (with a kernel, not a memset node:
+        // the caller may be capturing the stream into a graph)
+        const uint32_t chunks = (uint32_t)(need / 16);
+        hipLaunchKernelGGL(fill_slots_kernel, dim3((chunks + 255) / 256 < 2048 ? (chunks + 255) / 256 : 2048), dim3(256), 0, st, (u32x4 *)x.workspace, chunks);
+        if (int rc = check_launch("fill_slots_kernel")) return rc;
         slots = x.workspace;
     } else if (int rc = own_slots(need, &slots)) {
         return rc;
