@@ -222,3 +222,33 @@ def test_to_layout_with_dtype_and_clone(oracle, device, name):
         ttnn.to_layout(tiled, ttnn.ROW_MAJOR_LAYOUT, dtype=dtype)
     with pytest.raises(RuntimeError, match="on device"):
         ttnn.clone(ttnn.from_torch(x), ttnn.DRAM_MEMORY_CONFIG, dtype)
+
+
+@pytest.mark.parametrize("name", ["bfloat16", "bfloat8_b", "bfloat4_b"])
+def test_getitem_prefix_on_device(oracle, device, name):
+    """ttnn.Tensor.__getitem__ (ttnn/ttnn/operations/core.py:56-114): a prefix of a device tensor keeps whole tiles, so a
+    block-float result equals the corresponding tiles of the source, and its values equal the torch slice of the source's."""
+    import ttnn
+
+    dtype = getattr(ttnn, name)
+    torch.manual_seed(22)
+    x = torch.randn(2, 3, 96, 160).to(torch.bfloat16)
+    t = ttnn.from_torch(x, dtype=dtype, layout=ttnn.TILE_LAYOUT, device=device)
+    full = ttnn.to_torch(t)
+    part = t[:1, :2, :40, :70]
+    assert tuple(part.shape) == (1, 2, 40, 70) and tuple(part.shape.with_tile_padding()) == (1, 2, 64, 96)
+    assert part.dtype == dtype and part.layout == ttnn.TILE_LAYOUT and ttnn.is_tensor_storage_on_device(part)
+    assert torch.equal(ttnn.to_torch(part), full[:1, :2, :40, :70])
+    if name != "bfloat16":      # the tiles themselves: tile (r, c) of slice (0, ch) of the source
+        per_tile = {"bfloat8_b": 272, "bfloat4_b": 144}[name]
+        src = t._buf.view(2, 3, 3, 5, per_tile)
+        assert torch.equal(part._buf.view(1, 2, 2, 3, per_tile), src[:1, :2, :2, :3])
+    assert t[:2] is not None and tuple(t[:2].shape) == (2, 3, 96, 160)
+    row_major = ttnn.from_torch(x, layout=ttnn.ROW_MAJOR_LAYOUT, device=device)
+    assert torch.equal(ttnn.to_torch(row_major[:2, :1, :5, :9]), x[:2, :1, :5, :9])
+    with pytest.raises(RuntimeError, match="cannot slice"):
+        t[:, :, 32:64, :]
+    with pytest.raises(RuntimeError, match="cannot slice"):
+        ttnn.from_torch(x, layout=ttnn.ROW_MAJOR_LAYOUT)[:1]
+    with pytest.raises(RuntimeError, match="Too many slices"):
+        t[:1, :1, :1, :1, :1]

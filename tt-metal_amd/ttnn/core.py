@@ -149,3 +149,58 @@ def clone(tensor: Tensor, memory_config=None, dtype: Optional[DataType] = None) 
     if not isinstance(tensor, Tensor) or not ttnn.is_tensor_storage_on_device(tensor):
         raise RuntimeError("ttnn.clone: Tensor must be on device!")
     return ttl_tensor.clone(tensor, output_mem_config=memory_config, output_dtype=dtype)
+
+
+def _getitem(input_tensor: Tensor, slices) -> Tensor:
+    """ttnn.Tensor.__getitem__ (core.py:56-114): prefixes of a device tensor of rank <= 4.  In TILE layout the reference's
+    `unpad` copies whole tiles up to the tile-rounded end and the logical shape is set by a reshape, so block-float tiles
+    keep their bytes (nothing is re-quantised); the same happens here."""
+    input_rank = len(input_tensor._shape)
+    if isinstance(slices, int):
+        slices = (slice(None, slices, None),)
+    elif isinstance(slices, slice):
+        slices = (slices,)
+    elif slices is Ellipsis:
+        raise RuntimeError("Ellipsis is not supported!")
+    normalized = []
+    for s in slices:
+        if isinstance(s, int):
+            normalized.append(slice(None, s, None))
+        elif isinstance(s, slice):
+            normalized.append(s)
+        else:
+            raise RuntimeError("Invalid slice type!")
+    if len(normalized) > input_rank:
+        raise RuntimeError(f"Too many slices for tensor of rank {input_rank}")
+    normalized += [slice(None, None, None)] * (input_rank - len(normalized))
+    if not (ttnn.is_tensor_storage_on_device(input_tensor) and input_rank <= 4):
+        raise RuntimeError("ttnn.Tensor.__getitem__: cannot slice the given tensor on the device!")
+    t4 = unsqueeze_to_4D(input_tensor)
+    normalized = [slice(None, None, None)] * (4 - input_rank) + normalized
+    for s in normalized:
+        if s.start not in (None, 0) or s.step not in (None, 1):
+            raise RuntimeError("ttnn.Tensor.__getitem__: cannot slice the given tensor on the device!")
+    end = [s.stop if s.stop is not None else t4._shape[i] for i, s in enumerate(normalized)]
+    for i, e in enumerate(end):
+        if e < 0 or e > t4._shape[i]:
+            raise RuntimeError("ttnn.Tensor.__getitem__: slice end outside the tensor")
+    padded_end = list(end)
+    if t4.layout == Layout.TILE:
+        padded_end[-1], padded_end[-2] = _pad32(end[-1]), _pad32(end[-2])
+    full = tuple(t4._padded)
+    buf = t4._buf
+    if tuple(padded_end) != full:
+        if t4.layout == Layout.TILE:
+            per_tile = capi.TILE_BYTES[int(t4.dtype)] // buf.element_size()
+            tiles = buf.view(full[0], full[1], full[2] // 32, full[3] // 32, per_tile)
+            buf = tiles[:padded_end[0], :padded_end[1], :padded_end[2] // 32, :padded_end[3] // 32].contiguous().view(-1)
+        else:
+            buf = buf.view(full)[:padded_end[0], :padded_end[1], :padded_end[2], :padded_end[3]].contiguous()
+    out_shape = tuple(end[-input_rank:])
+    out_padded = tuple(padded_end[-input_rank:])
+    if t4.layout == Layout.ROW_MAJOR and t4.dtype not in _BFP:
+        buf = buf.reshape(out_padded)
+    return Tensor(None, _raw=(buf, out_shape, out_padded, t4.dtype, t4.layout, t4._device))
+
+
+Tensor.__getitem__ = _getitem
