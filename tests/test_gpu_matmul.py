@@ -132,12 +132,9 @@ def test_linear_bias_and_activation(oracle, activation):
     assert torch.allclose(c[0].cpu().double(), ref, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("stream_k", ["0", "1"])
 @pytest.mark.parametrize("workgroups", ["1", "3", "7", "64", "512", "4096"])
-def test_any_number_of_workgroups_gives_the_same_bits(oracle, workgroups, stream_k, monkeypatch):
-    """The k range of an output may be shared between workgroups in any way — cut into equal parts per output, or dealt out
-    evenly across output boundaries; partial sums are added in a fixed order."""
-    monkeypatch.setenv("TTMI_MATMUL_STREAMK", stream_k)
+def test_any_number_of_workgroups_gives_the_same_bits(oracle, workgroups, monkeypatch):
+    """The k range of an output may be shared between workgroups in any way; partial sums are added in a fixed order."""
     m, k, n = 40, 1024, 288
     a_bits = workloads.activations_bf16(m, k, seed=71)
     words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=72), BFP8)

@@ -85,7 +85,7 @@ __device__ __forceinline__ uint32_t not_empty(uint32_t bits) { return bits == SL
 //   split > 0   every output group is cut into `split` nearly equal k ranges, one per workgroup (P = groups * split):
 //               one output per workgroup, at most `split` partial sums to add
 //   split == 0  "stream-K": the U units are dealt out contiguously, the first `extra` workgroups take share + 1 units,
-//               the rest `share`; a range may end one output and begin the next
+//               the rest `share`; a range may end one output and begin the next (the host does not choose this)
 __device__ __forceinline__ uint32_t range_start(const MatmulDev &p, uint32_t i) {
     if (p.split) return (i / p.split) * p.kt + ((i % p.split) * p.kt) / p.split;
     return i * p.share + min(i, p.extra);
@@ -202,102 +202,6 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
     const uint32_t unit_end = range_start(p, me + 1);
     const uint32_t my_first_og = unit / p.kt;
 
-    // Adds the partial sums of the other contributors to output group `og` (all of lower index) to `sums`, in workgroup
-    // order, and leaves their slots empty for the next launch.
-    auto collect = [&](uint32_t og, float (&sums)[2][4]) __attribute__((always_inline)) {
-        const uint32_t lo = og * p.kt;
-        const uint32_t first = workgroup_of(p, lo), last = workgroup_of(p, lo + p.kt - 1);
-        float sum[2][4];
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) sum[r][j] = 0.f;
-        const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
-        for (uint32_t w0 = first; w0 < last; w0 += 4) {          // four contributors' loads in flight at a time
-            u32x4 part[4][2];
-            float4 *other[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t w = min(w0 + u, last - 1);
-                const uint32_t which = range_start(p, w) >= lo ? 0u : 1u;      // first or second output of w
-                other[u] = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(2 * w + which) * 8 + wave * 2) * 64 + lane;
-            }
-            uint32_t spins = 0;
-            bool waiting;
-            do {
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-#pragma unroll
-                    for (int r = 0; r < 2; ++r) part[u][r] = slot_load_issue(other[u] + r * 64);
-                asm volatile("s_waitcnt vmcnt(0)" : "+v"(part[0][0]), "+v"(part[0][1]), "+v"(part[1][0]), "+v"(part[1][1]),
-                             "+v"(part[2][0]), "+v"(part[2][1]), "+v"(part[3][0]), "+v"(part[3][1])::"memory");
-                bool missing = false;
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-#pragma unroll
-                    for (int r = 0; r < 2; ++r)
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) missing |= part[u][r][j] == SLOT_EMPTY;
-                waiting = __ballot(missing) != 0 && ++spins < SLOT_SPIN_LIMIT;
-                if (waiting) __builtin_amdgcn_s_sleep(4);
-            } while (waiting);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (w0 + u >= last) break;
-#pragma unroll
-                for (int r = 0; r < 2; ++r) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) sum[r][j] += __uint_as_float(part[u][r][j]);
-                    slot_store(other[u] + r * 64, empty);                       // ready for the next launch
-                }
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) sums[r][j] = sum[r][j] + sums[r][j];
-    };
-    // Epilogue and store of output group `og`: this wavefront's two rows of the band, this lane's four columns.
-    auto store = [&](uint32_t og, const float (&sums)[2][4]) __attribute__((always_inline)) {
-        const uint32_t ng = og % p.ngroups, band = og / p.ngroups;
-        const uint32_t mt = band % p.mt, bb = band / p.mt;
-        const uint32_t nt0 = ng * GROUP_TILES;
-        const uint32_t n_valid = min((uint32_t)GROUP_TILES, p.nt - nt0);
-        if (t_of_lane < (int)n_valid) {
-            const uint32_t n_col = (nt0 + t_of_lane) * 32 + fc * 16 + q * 4;   // first of this lane's 4 columns
-#pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const uint32_t row_in_band = (wave >> 1) * 16 + g * 4 + (wave & 1) * 2 + r;
-                const uint32_t row = mt * 32 + row_in_band;
-                if (row >= p.m) continue;
-                float v[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float x = sums[r][j] * F::unscale;
-                    if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
-                    v[j] = apply_activation<ACT>(x);
-                }
-                uint64_t elem;   // element offset of the 4-column run in C
-                if (p.c_tiled) {
-                    const uint64_t tile = ((uint64_t)bb * p.mt + mt) * p.nt + nt0 + t_of_lane;
-                    elem = tile * 1024 + ((row_in_band >> 4) * 2 + fc) * 256 + (row_in_band & 15) * 16 + q * 4;
-                } else {
-                    elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
-                }
-                if (p.c_f32) {
-                    *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
-                } else {
-                    const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
-                    const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
-                    *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
-                }
-            }
-        }
-    };
-    bool holding = false;          // a collection put off until this workgroup has handed over its own later part
-    uint32_t held_og = 0;
-    float held[2][4] = {};
-
     while (unit < unit_end) {
         // ---- one segment: output group og, k-tiles [k_begin, k_end) ---------------------------------------
         const uint32_t og = unit / p.kt;
@@ -390,14 +294,15 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
 
         // ---- outputs shared with other workgroups ----------------------------------------------------------
         // Contributors are the workgroups first..last whose ranges meet this output's k range.  The last one (the
-        // highest index: every other contributor was dispatched before it) collects the others' partial sums and adds
-        // them in workgroup order, its own last: the result does not depend on timing.  Wavefront w of every contributor
-        // holds the same rows, so the hand-over is wavefront to wavefront and needs no workgroup barrier.  A workgroup
-        // whose range goes on into the next output hands that part over FIRST and collects afterwards: then nobody's
-        // hand-over waits for anybody, and a collector only ever waits for workgroups that do not wait themselves.
+        // highest index: every other contributor was dispatched before it and waits for nobody, so it will finish)
+        // collects the others' partial sums and adds them in workgroup order, its own last: the result does not
+        // depend on timing.  Wavefront w of every contributor holds the same rows, so the hand-over is wavefront to
+        // wavefront and needs no workgroup barrier.
         bool store_now = true;
         if (k_begin != 0 || k_end != p.kt) {
-            if (me != workgroup_of(p, og * p.kt + p.kt - 1)) {
+            const uint32_t lo = og * p.kt;
+            const uint32_t first = workgroup_of(p, lo), last = workgroup_of(p, lo + p.kt - 1);
+            if (me != last) {
                 float4 *slot = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(2 * me + (og == my_first_og ? 0 : 1)) * 8 + wave * 2) * 64 + lane;
 #pragma unroll
                 for (int r = 0; r < 2; ++r) {
@@ -407,24 +312,90 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
                     slot_store(slot + r * 64, v);
                 }
                 store_now = false;
-            } else if (unit < unit_end) {
+            } else {
+                float sum[2][4];
 #pragma unroll
                 for (int r = 0; r < 2; ++r)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) held[r][j] = mine[r][j];
-                held_og = og;
-                holding = true;
-                store_now = false;
-            } else {
-                collect(og, mine);
+                    for (int j = 0; j < 4; ++j) sum[r][j] = 0.f;
+                const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
+                for (uint32_t w0 = first; w0 < last; w0 += 4) {          // four contributors' loads in flight at a time
+                    u32x4 part[4][2];
+                    float4 *other[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const uint32_t w = min(w0 + u, last - 1);
+                        const uint32_t which = range_start(p, w) >= lo ? 0u : 1u;      // first or second output of w
+                        other[u] = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(2 * w + which) * 8 + wave * 2) * 64 + lane;
+                    }
+                    uint32_t spins = 0;
+                    bool waiting;
+                    do {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int r = 0; r < 2; ++r) part[u][r] = slot_load_issue(other[u] + r * 64);
+                        asm volatile("s_waitcnt vmcnt(0)" : "+v"(part[0][0]), "+v"(part[0][1]), "+v"(part[1][0]), "+v"(part[1][1]),
+                                     "+v"(part[2][0]), "+v"(part[2][1]), "+v"(part[3][0]), "+v"(part[3][1])::"memory");
+                        bool missing = false;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) missing |= part[u][r][j] == SLOT_EMPTY;
+                        waiting = __ballot(missing) != 0 && ++spins < SLOT_SPIN_LIMIT;
+                        if (waiting) __builtin_amdgcn_s_sleep(4);
+                    } while (waiting);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (w0 + u >= last) break;
+#pragma unroll
+                        for (int r = 0; r < 2; ++r) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) sum[r][j] += __uint_as_float(part[u][r][j]);
+                            slot_store(other[u] + r * 64, empty);                       // ready for the next launch
+                        }
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) mine[r][j] = sum[r][j] + mine[r][j];
             }
         }
-        if (store_now) store(og, mine);
+
+        if (store_now && t_of_lane < (int)n_valid) {
+            const uint32_t n_col = (nt0 + t_of_lane) * 32 + fc * 16 + q * 4;   // first of this lane's 4 columns
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint32_t row_in_band = (wave >> 1) * 16 + g * 4 + (wave & 1) * 2 + r;
+                const uint32_t row = mt * 32 + row_in_band;
+                if (row >= p.m) continue;
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float x = mine[r][j] * F::unscale;
+                    if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
+                    v[j] = apply_activation<ACT>(x);
+                }
+                uint64_t elem;   // element offset of the 4-column run in C
+                if (p.c_tiled) {
+                    const uint64_t tile = ((uint64_t)bb * p.mt + mt) * p.nt + nt0 + t_of_lane;
+                    elem = tile * 1024 + ((row_in_band >> 4) * 2 + fc) * 256 + (row_in_band & 15) * 16 + q * 4;
+                } else {
+                    elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
+                }
+                if (p.c_f32) {
+                    *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                    const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
+                    const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
+                    *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
+                }
+            }
+        }
         __syncthreads();   // LDS is reused by the next segment
-    }
-    if (holding) {
-        collect(held_og, held);
-        store(held_og, held);
     }
 }
 
@@ -449,26 +420,14 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     // workgroups to aim for: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone nearly get there,
     // x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot reset)
     const uint64_t resident = env_u32("TTMI_MATMUL_WGS", d.groups >= 256 ? 768 : 512);
-    // Aligned split: every output's k range is cut into equally many parts (every wavefront keeping >= 2 k-tiles); cheap
-    // (one output per workgroup) but the number of workgroups is a multiple of the number of outputs.  When that leaves
-    // more than a fifth of the chip's slots empty the units are instead dealt out evenly across output boundaries
-    // ("stream-K", split == 0): every workgroup streams the same number of bytes, at the price of a second start-up for
-    // the workgroups whose range crosses an output boundary (measured: Falcon h_to_4h, 568 of 768 slots, 33.3 -> 31.3 us;
-    // Mistral gate, 448 of 512 slots, 21.4 -> 22.2 us).  TTMI_MATMUL_STREAMK=0|1 forces one.
+    // cut every output's k range into as many parts as keeps the chip full, every wavefront keeping >= 2 k-tiles
+    // (the kernel can also deal the units out evenly across output boundaries, split == 0, but a workgroup that is
+    // consumer of one output and producer of the next would then make its successor wait: not offered)
     uint64_t parts = d.groups >= resident ? 1 : resident / d.groups;
     const uint64_t most = d.kt / (2 * WAVES) ? d.kt / (2 * WAVES) : 1;
     if (parts > most) parts = most;
-    const char *force = getenv("TTMI_MATMUL_STREAMK");
-    const uint64_t evenly = d.units < resident ? d.units : resident;
-    bool stream_k = d.groups < resident && d.groups * parts * 10 < resident * 8 && d.units / evenly >= 2 * WAVES;
-    if (force && (force[0] == '0' || force[0] == '1')) stream_k = force[0] == '1';
-    if (stream_k) {
-        d.split = 0;
-        d.workgroups = (uint32_t)evenly;
-    } else {
-        d.split = (uint32_t)parts;
-        d.workgroups = (uint32_t)(d.groups * parts);
-    }
+    d.split = (uint32_t)parts;
+    d.workgroups = (uint32_t)(d.groups * parts);
     return d;
 }
 
