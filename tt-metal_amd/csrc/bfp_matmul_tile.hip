@@ -250,36 +250,17 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
         iteration(I0{}, std::false_type{});
     }
 
-    // ---- epilogue: acc[rb][cb][i] is row rb*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the wavefront's 64
-    if (t_of_lane >= (int)n_valid) return;
-    const uint32_t col_in_tile = fc * 16 + q * 4 + half * 2;
-    const uint32_t n_col = (nt0 + t_of_lane) * 32 + col_in_tile;
-    float bias_v[2] = {0.f, 0.f};
-    if (p.bias) {
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb) bias_v[cb] = __uint_as_float((uint32_t)p.bias[n_col + cb] << 16);
-    }
-#pragma unroll
-    for (int rb = 0; rb < MB; ++rb) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t row = m0 + rb * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
-            if (row >= p.m) continue;
-            const float v0 = apply_activation<ACT>(acc[rb][0][i] * F::unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * F::unscale + bias_v[1]);
-            uint64_t elem;
-            if (p.c_tiled) {
-                const uint64_t tile = ((uint64_t)bb * ((p.m + 31) / 32) + (row >> 5)) * p.nt + nt0 + t_of_lane;
-                elem = tile * 1024 + (((row >> 4) & 1) * 2 + fc) * 256 + (row & 15) * 16 + q * 4 + half * 2;
-            } else {
-                elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
-            }
-            if (p.c_f32) {
-                *reinterpret_cast<float2 *>(p.c + elem * 4) = make_float2(v0, v1);
-            } else {
-                *reinterpret_cast<uint32_t *>(p.c + elem * 2) = f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
-            }
-        }
-    }
+    // ---- epilogue: acc[rb][cb][i] is row rb*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the wavefront's 64;
+    // the ring is idle now and becomes the staging of store_wave_part (4 KB per 32 rows and wavefront)
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    StoreTarget o;
+    o.c = p.c; o.bias = p.bias; o.m = p.m; o.n = p.n; o.nt = p.nt; o.slice = bb;
+    o.row0 = m0; o.nt0 = nt0;
+    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32;
+    static_assert(MB == 4 && TILE_STAGES * STAGE_BYTES >= 4 * 16384, "the epilogue stages 128 rows x 64 columns per wavefront in the ring");
+    store_wave_part<ACT>(acc, o, lds + wave * 16384, lane);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -464,36 +445,17 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
     while (step + 1 < total) iteration(std::true_type{});
     iteration(std::false_type{});
 
-    // ---- epilogue: acc[rb][cb][i] is row wr*128 + rb*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the group's 64
-    if (t_of_lane >= (int)n_valid) return;
-    const uint32_t col_in_tile = fc * 16 + q * 4 + half * 2;
-    const uint32_t n_col = (nt0 + t_of_lane) * 32 + col_in_tile;
-    float bias_v[2] = {0.f, 0.f};
-    if (p.bias) {
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb) bias_v[cb] = __uint_as_float((uint32_t)p.bias[n_col + cb] << 16);
-    }
-#pragma unroll
-    for (int rb = 0; rb < MB; ++rb) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t row = m0 + wr * 128 + rb * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
-            if (row >= p.m) continue;
-            const float v0 = apply_activation<ACT>(acc[rb][0][i] * F::unscale + bias_v[0]), v1 = apply_activation<ACT>(acc[rb][1][i] * F::unscale + bias_v[1]);
-            uint64_t elem;
-            if (p.c_tiled) {
-                const uint64_t tile = ((uint64_t)bb * ((p.m + 31) / 32) + (row >> 5)) * p.nt + nt0 + t_of_lane;
-                elem = tile * 1024 + (((row >> 4) & 1) * 2 + fc) * 256 + (row & 15) * 16 + q * 4 + half * 2;
-            } else {
-                elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
-            }
-            if (p.c_f32) {
-                *reinterpret_cast<float2 *>(p.c + elem * 4) = make_float2(v0, v1);
-            } else {
-                *reinterpret_cast<uint32_t *>(p.c + elem * 2) = f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
-            }
-        }
-    }
+    // ---- epilogue: acc[rb][cb][i] is row wr*128 + rb*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the group's 64;
+    // the ring and the operand buffers are idle now and become the staging of store_wave_part (16 KB per wavefront)
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    StoreTarget o;
+    o.c = p.c; o.bias = p.bias; o.m = p.m; o.n = p.n; o.nt = p.nt; o.slice = bb;
+    o.row0 = m0 + wr * 128; o.nt0 = nt0;
+    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32;
+    static_assert(OPS_BASE + 2 * OPS_BYTES >= 8 * 16384, "staging of the epilogue does not fit into LDS");
+    store_wave_part<ACT>(acc, o, lds + wave * 16384, lane);
 }
 
 template <int W>
