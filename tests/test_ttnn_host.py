@@ -80,3 +80,51 @@ def test_matmul_validation_on_host_tensors():
         ttnn.matmul(ttnn.from_torch(torch.zeros(32, dtype=torch.bfloat16)), a)
     with pytest.raises(RuntimeError, match="must be of type"):
         ttnn.matmul(ttnn.from_torch(torch.zeros(32, 32, dtype=torch.float32)), a)
+
+
+def _host_tile_tensor(shape, dtype=tt_lib.tensor.DataType.BFLOAT16):
+    """A host tensor that claims TILE layout (no conversion needed to build it: only metadata is checked below)."""
+    n = 1
+    for s in shape:
+        n *= s
+    return tt_lib.tensor.Tensor(None, _raw=(torch.zeros(n, dtype=torch.bfloat16), tuple(shape), tuple(shape), dtype, tt_lib.tensor.Layout.TILE, None))
+
+
+def test_elementwise_argument_checks_need_no_gpu():
+    """ttnn/ttnn/operations/binary.py:352-368: first operand a device tensor, second a tensor or a number."""
+    host = _host_tile_tensor((32, 32))
+    with pytest.raises(RuntimeError, match="must be on device"):
+        ttnn.mul(host, host)
+    with pytest.raises(TypeError, match="first argument"):
+        ttnn.mul(torch.zeros(2), host)
+    with pytest.raises(RuntimeError, match="must be on device"):
+        ttnn.gelu(host)
+    assert ttnn.multiply is ttnn.mul and ttnn.subtract is ttnn.sub
+
+
+def test_falcon_matmul_shape_rules():
+    """bmm_op.cpp:773-784: above 1024 rows falcon_dense_h_to_4h_matmul takes no fused activation and only the model's shapes."""
+    gelu = [tt_lib.tensor.FusibleActivation.GELU, True]
+    assert tt_lib.tensor.FusibleActivationWithParam(gelu).op_type == tt_lib.tensor.FusibleActivation.GELU
+    assert int(tt_lib.tensor.FusibleActivation.GELU) == 2 and int(tt_lib.tensor.FusibleActivation.SILU) == 48     # UnaryOpType values
+    a = _host_tile_tensor((1, 1, 2048, 64))
+    w = _host_tile_tensor((1, 1, 64, 128), tt_lib.tensor.DataType.BFLOAT8_B)
+    with pytest.raises(RuntimeError, match="fused_activation"):
+        tt_lib.tensor.falcon_dense_h_to_4h_matmul(a, w, fused_activation=gelu)
+    with pytest.raises(RuntimeError, match="Unsupported input shape"):
+        tt_lib.tensor.falcon_dense_h_to_4h_matmul(a, w)
+    with pytest.raises(RuntimeError, match="need to be on device"):
+        tt_lib.tensor.falcon_dense_4h_to_h_matmul(_host_tile_tensor((1, 1, 32, 64)), w)
+
+
+def test_as_tensor_and_clone_argument_checks():
+    with pytest.raises(RuntimeError, match="must be of type"):
+        ttnn.as_tensor(torch.zeros(4, 4, dtype=torch.float64))
+    with pytest.raises(RuntimeError, match="must be of rank"):
+        ttnn.as_tensor(torch.zeros(()))
+    with pytest.raises(RuntimeError, match="on device"):
+        ttnn.clone(_host_tile_tensor((32, 32)), None, ttnn.bfloat8_b)
+    with pytest.raises(RuntimeError, match="Unsupported datatype conversion"):
+        ttnn.to_layout(ttnn.from_torch(torch.zeros(32, 32, dtype=torch.bfloat16)), ttnn.TILE_LAYOUT, dtype=ttnn.bfloat8_b)
+    with pytest.raises(RuntimeError, match="cannot slice"):
+        ttnn.from_torch(torch.zeros(4, 4))[:2]
