@@ -159,7 +159,7 @@ def test_caller_workspace(oracle):
         capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP4, 1, 1, m, k, n, workspace=small)
 
 
-@pytest.mark.parametrize("kernel", ["stream", "tile", "tile256", "expanded"])
+@pytest.mark.parametrize("kernel", ["stream", "wide", "tile", "tile256", "expanded"])
 @pytest.mark.parametrize("fmt", [BFP8, BFP4])
 @pytest.mark.parametrize("batch,b_batch,m,k,n", [(1, 1, 256, 128, 256), (1, 1, 300, 96, 288), (2, 1, 130, 160, 96), (1, 1, 288, 224, 96),
                                                  (2, 2, 512, 64, 544), (1, 1, 40, 32, 2080)])

@@ -160,6 +160,51 @@ __device__ __forceinline__ void staged_operands(uint32_t exp_at, uint32_t mant_a
     bop[3] = weights_operand8<3>(words, mags, scale);
 }
 
+// The same in two steps, for kernels that read several slabs before they wait: what one lane reads from LDS for 8 k rows
+// of one face (8 exponent bytes, 8 mantissa words) ...
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+struct SlabRaw { u32x2 e01, w01, w23, w45, w67; };
+
+// ... requested here (inline assembly for the reason given at staged_operands; EXP_OFF / MANT_OFF are compile-time byte
+// offsets; the caller waits with wait_slabs before it touches the result) ...
+template <int W, int EXP_OFF, int MANT_OFF> __device__ __forceinline__ void slab_read(uint32_t exp_at, uint32_t mant_at, SlabRaw &r) {
+    constexpr int R = Wfmt<W>::row_bytes / 4;
+    const uint32_t mant = mant_at + MANT_OFF;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(r.e01) : "v"(exp_at), "n"(EXP_OFF));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w01) : "v"(mant), "n"(0 * R), "n"(1 * R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w23) : "v"(mant), "n"(2 * R), "n"(3 * R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w45) : "v"(mant), "n"(4 * R), "n"(5 * R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w67) : "v"(mant), "n"(6 * R), "n"(7 * R));
+}
+__device__ __forceinline__ void wait_slabs(SlabRaw &a, SlabRaw &b) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.e01), "+v"(a.w01), "+v"(a.w23), "+v"(a.w45), "+v"(a.w67),
+                                          "+v"(b.e01), "+v"(b.w01), "+v"(b.w23), "+v"(b.w45), "+v"(b.w67)::"memory");
+}
+// ... and expanded into the four B operands (byte j of every word = operand j, as above).
+template <int W> __device__ __forceinline__ void slab_expand(const SlabRaw &r, int q, bf16x8 (&bop)[4]) {
+    uint32_t words[8] = {r.w01[0], r.w01[1], r.w23[0], r.w23[1], r.w45[0], r.w45[1], r.w67[0], r.w67[1]};
+    uint32_t mags[8];
+    float scale[8];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(((r.e01[jj >> 2] >> (8 * (jj & 3))) & 0xffu) << 23);
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+        if (W == 7) {
+            mags[jj] = words[jj] & 0x7f7f7f7fu;
+        } else {
+            uint32_t v = (words[jj] >> (16 * (q & 1))) & 0xffffu;
+            v = (v | (v << 8)) & 0x00ff00ffu;
+            v = (v | (v << 4)) & 0x0f0f0f0fu;
+            words[jj] = v << 4;
+            mags[jj] = v & 0x07070707u;
+        }
+    }
+    bop[0] = weights_operand8<0>(words, mags, scale);
+    bop[1] = weights_operand8<1>(words, mags, scale);
+    bop[2] = weights_operand8<2>(words, mags, scale);
+    bop[3] = weights_operand8<3>(words, mags, scale);
+}
+
 // Epilogue of the tiled GEMM kernels for one wavefront: a 128-row x 64-column part of C (one 64-column weight group) whose
 // accumulators lie as v_mfma_f32_32x32x16 leaves them, with the column order of the weight expansion:
 //   acc[rb][cb][i] = row 32 rb + 8 (i / 4) + 4 kh + i % 4, column 32 t + 16 fc + 4 q + 2 half + cb of the 64, for lane

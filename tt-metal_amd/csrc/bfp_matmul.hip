@@ -400,6 +400,289 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// Wide streaming kernel: the same scheme with units of 32 k rows x 128 columns (4 adjacent packed tiles) and
+// v_mfma_f32_32x32x16_bf16.  Against the 64-column kernel every activation load, every ring move and every matrix
+// instruction serves twice as many weights.
+//   lane (c32 = lane % 32, kh = lane / 32) holds, for operand j of slab s (k rows 16s..16s+15 of the k-tile),
+//   column 4*c32 + j of the group and k rows 16s + 8kh .. + 7: byte j of 8 mantissa words of face row s of tile
+//   c32 / 8.  The activations are the A operand of the same instruction: row c32 of the band, the same 8 k.
+//   One workgroup = one k range of one output group (split >= 1); after the loop acc[j][i] is row 8(i/4) + 4kh + i%4,
+//   column 4*c32 + j.  Wavefront w keeps rows 8w..8w+7 of the workgroup's sums.
+// A stage of the LDS ring holds the two tile pairs of a unit, each laid out as Wfmt describes; the second pair is
+// shifted by PAIR_PAD bytes so that the 64 lanes of one ds_read2_b32 fall into 64 different banks.
+// ---------------------------------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+constexpr int WIDE_TILES = 4;
+constexpr int WIDE_COLS = WIDE_TILES * 32;
+#ifndef TTMI_WIDE_WGS_PER_CU
+#define TTMI_WIDE_WGS_PER_CU 2
+#endif
+#ifndef TTMI_WIDE_STAGES
+#define TTMI_WIDE_STAGES 3
+#endif
+constexpr int WIDE_WGS_PER_CU = TTMI_WIDE_WGS_PER_CU;
+constexpr int WIDE_STAGES = TTMI_WIDE_STAGES;
+constexpr int WIDE_REDUCE_BYTES = WAVES * 64 * 64 * 4;     // every wavefront lays out its 64 accumulator registers
+constexpr size_t WIDE_SLOT_BYTES = 32 * WIDE_COLS * sizeof(float);
+
+template <int W, int ACT>
+__global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const MatmulDev p) {
+    using F = Wfmt<W>;
+    constexpr int PAIR_PAD = W == 7 ? 64 : 128;
+    constexpr int PAIR_STRIDE = F::stage_bytes + PAIR_PAD;
+    constexpr int UNIT_BYTES = 2 * PAIR_STRIDE;
+    constexpr int WAVE_LDS = WIDE_STAGES * UNIT_BYTES;
+    constexpr int LDS_BYTES = WIDE_REDUCE_BYTES > WAVES * WAVE_LDS ? WIDE_REDUCE_BYTES : WAVES * WAVE_LDS;
+    constexpr int NLOAD = F::loads;
+    constexpr int PER = 2 * NLOAD + 2;                 // vector-memory requests per unit
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
+
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c32 = lane & 31, kh = lane >> 5;
+    const int t_of_lane = c32 >> 3, pair = t_of_lane >> 1, t_in = t_of_lane & 1, fc = (c32 >> 2) & 1, q = c32 & 3;
+
+    uint32_t chunk_of[NLOAD];
+    stage_chunks<W>(lane, chunk_of);
+    // this lane's LDS addresses for slab 0 of stage 0; slab 1 is 32 bytes (exponents) / 4 faces (mantissas) further
+    const uint32_t exp_at = lds_base + wave * WAVE_LDS + pair * PAIR_STRIDE + F::exp_base + t_in * 64 + fc * 16 + kh * 8;
+    const uint32_t mant_at = lds_base + wave * WAVE_LDS + pair * PAIR_STRIDE + (t_in * 2 + fc) * F::face_stride + (kh * 8) * F::row_bytes +
+                             (W == 7 ? q * 4 : (q >> 1) * 4);
+
+    // ---- this workgroup's output group and k range ---------------------------------------------------------
+    const uint32_t me = blockIdx.x;
+    const uint32_t og = me / p.split, part = me - og * p.split;
+    const uint32_t k_begin = (part * p.kt) / p.split, k_end = ((part + 1) * p.kt) / p.split;
+    const uint32_t ng = og % p.ngroups, band = og / p.ngroups;
+    const uint32_t mt = band % p.mt, bb = band / p.mt;
+    const uint32_t nt0 = ng * WIDE_TILES;
+    const uint32_t n_valid = min((uint32_t)WIDE_TILES, p.nt - nt0);
+
+    // tiles past the matrix edge repeat the last chunk that exists and are never stored
+    const uint32_t chunks_valid = n_valid * F::chunks;
+    uint32_t src_off[2][NLOAD];
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+        for (int l = 0; l < NLOAD; ++l) src_off[pr][l] = min(pr * 2 * F::chunks + chunk_of[l], chunks_valid - 1) * 16;
+    const uint8_t *wptr = p.b + ((uint64_t)(p.b_batch == 1 ? 0 : bb) * p.kt * p.nt + (uint64_t)(k_begin + wave) * p.nt + nt0) * F::tile_bytes;
+    const uint64_t w_step = (uint64_t)WAVES * p.nt * F::tile_bytes;
+    // activations of one unit for this lane: row c32 of the band, k = kt*32 + 16s + 8kh .. + 7 for s = 0, 1;
+    // rows past M read row M-1 and are never stored
+    const uint8_t *aptr;
+    uint32_t a_second, a_step;
+    if (p.a_tiled) {
+        aptr = p.a + (((uint64_t)bb * p.mt + mt) * p.kt + k_begin + wave) * 2048 + (c32 >> 4) * 1024 + (c32 & 15) * 32 + kh * 16;
+        a_second = 512; a_step = WAVES * 2048;
+    } else {
+        const uint32_t r0 = min(mt * 32 + c32, p.m - 1);
+        aptr = p.a + (((uint64_t)bb * p.m + r0) * p.k + (k_begin + wave) * 32 + kh * 8) * 2;
+        a_second = 32; a_step = WAVES * 64;
+    }
+
+    f32x16 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+    u32x4 a_ring[WIDE_STAGES][2] = {};
+
+    // Requests one unit: its 4 packed tiles straight into LDS stage S, its activations into a_ring[S] (inline assembly
+    // for the loads and their waits, as in the 64-column kernel).
+    auto fetch = [&](auto stage_tag) __attribute__((always_inline)) {
+        constexpr int S = decltype(stage_tag)::value;
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+            for (int l = 0; l < NLOAD; ++l)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[pr][l]),
+                                                 (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * UNIT_BYTES + pr * PAIR_STRIDE + l * 1024),
+                                                 16, 0, 0);
+        wptr += w_step;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][0]) : "v"(aptr) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][1]) : "v"(aptr + a_second) : "memory");
+        aptr += a_step;
+    };
+    auto work = [&](auto stage_tag, auto younger_tag, bool refill) __attribute__((always_inline)) {
+        constexpr int S = decltype(stage_tag)::value;
+        constexpr int YOUNGER = decltype(younger_tag)::value;
+        if (YOUNGER >= 0) wait_vmcnt<(YOUNGER < 0 ? 0 : YOUNGER) * PER>();   // < 0: the caller has waited
+        asm volatile("" : "+v"(a_ring[S][0]), "+v"(a_ring[S][1]) :: "memory");
+        u32x4 a_now[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                uint32_t moved;
+                asm volatile("v_mov_b32 %0, %1" : "=v"(moved) : "v"(a_ring[S][s][e]));
+                a_now[s][e] = moved;
+            }
+        SlabRaw raw0, raw1;
+        slab_read<W, S * UNIT_BYTES, S * UNIT_BYTES>(exp_at, mant_at, raw0);
+        slab_read<W, S * UNIT_BYTES + 32, S * UNIT_BYTES + 4 * F::face_stride>(exp_at, mant_at, raw1);
+        wait_slabs(raw0, raw1);
+        if (refill) fetch(stage_tag);
+        bf16x8 bop[4];
+        slab_expand<W>(raw0, q, bop);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[0]), bop[j], acc[j], 0, 0, 0);
+        slab_expand<W>(raw1, q, bop);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[1]), bop[j], acc[j], 0, 0, 0);
+    };
+
+    // This wavefront's units: k_begin + wave, + WAVES, ...; unit i lives in stage i % STAGES and is requested STAGES
+    // units ahead (see the 64-column kernel for the bookkeeping of requests in flight).
+    const uint32_t span = k_end - k_begin;
+    const uint32_t total = span > (uint32_t)wave ? (span - wave + WAVES - 1) / WAVES : 0;
+    using Last = std::integral_constant<int, WIDE_STAGES - 1>;
+    constexpr auto stages = std::make_integer_sequence<int, WIDE_STAGES>{};
+    uint32_t i = 0;
+    if (total >= 2 * WIDE_STAGES) {
+        static_for(stages, [&](auto s) __attribute__((always_inline)) { fetch(s); });
+#pragma unroll 1
+        for (; i + 2 * WIDE_STAGES <= total; i += WIDE_STAGES)
+            static_for(stages, [&](auto s) __attribute__((always_inline)) { work(s, Last{}, true); });
+    } else {
+        static_for(stages, [&](auto s) __attribute__((always_inline)) { if (total > (uint32_t)decltype(s)::value) fetch(s); });
+    }
+    static_for(std::make_integer_sequence<int, 2 * WIDE_STAGES - 1>{}, [&](auto j) __attribute__((always_inline)) {
+        constexpr int J = decltype(j)::value;
+        const uint32_t at = i + J;
+        if (at >= total) return;
+        wait_for_younger<WIDE_STAGES - 1, PER>(total - 1 - at);
+        work(std::integral_constant<int, J % WIDE_STAGES>{}, std::integral_constant<int, -1>{}, at + WIDE_STAGES < total);
+    });
+
+    wait_vmcnt<0>();   // nothing in flight any more (already true; also what the build-time ISA check keys on)
+    // ---- add the four wavefronts' partial sums through LDS ------------------------------------------------------
+    // Every wavefront writes its 64 accumulator registers as 16 float4 (acc[j][4q4 .. 4q4+3]); wavefront w then keeps
+    // q4 = w: rows 8w + 4kh + r (r = 0..3), columns 4*c32 + j.
+    __syncthreads();
+    float4 *red = reinterpret_cast<float4 *>(lds);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+            red[(wave * 16 + j * 4 + q4) * 64 + lane] = make_float4(acc[j][4 * q4], acc[j][4 * q4 + 1], acc[j][4 * q4 + 2], acc[j][4 * q4 + 3]);
+    __syncthreads();
+    float mine[4][4];   // [r][j]
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int sw = 0; sw < WAVES; ++sw) {
+            const float4 x = red[(sw * 16 + j * 4 + wave) * 64 + lane];
+            v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
+        }
+        mine[0][j] = v.x; mine[1][j] = v.y; mine[2][j] = v.z; mine[3][j] = v.w;
+    }
+
+    // ---- outputs shared with other workgroups ----------------------------------------------------------------
+    // The `split` workgroups of an output add their partial sums along a radix-4 tree over r = split - 1 - part: a
+    // workgroup whose r has zeros in its lowest base-4 digits collects, digit position by digit position, from
+    // r + s, r + 2s, r + 3s (s = 4^position) while they exist, adding them in that order; at its lowest non-zero digit
+    // it publishes its sums in its slot and is done.  r = 0 (the highest index) ends with the complete sum and stores.
+    // Whoever waits, waits for workgroups of lower index only: they were dispatched earlier and wait for nobody
+    // dispatched later, so they finish.  The order of the additions is fixed, the result does not depend on timing.
+    // Slots work as in the 64-column kernel (SLOT_EMPTY until written, put back by the reader), one per workgroup;
+    // wavefront w of every workgroup holds the same rows, so the hand-over is wavefront to wavefront.
+    bool store_now = true;
+    if (p.split > 1) {
+        const uint32_t first = og * p.split, r_me = p.split - 1 - part;
+        const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
+        const u32x4 nothing = {0u, 0u, 0u, 0u};
+        for (uint32_t s = 1; s < p.split; s *= 4) {
+            if ((r_me / s) & 3u) break;
+            if (r_me + s >= p.split) break;
+            u32x4 got[3][4];
+            float4 *other[3];
+#pragma unroll
+            for (int u = 0; u < 3; ++u) {
+                const uint32_t r_other = min(r_me + (u + 1) * s, p.split - 1);
+                other[u] = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(first + p.split - 1 - r_other) * 16 + wave * 4) * 64 + lane;
+            }
+            uint32_t spins = 0;
+            bool waiting;
+            do {
+#pragma unroll
+                for (int u = 0; u < 3; ++u)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        got[u][r] = nothing;
+                        if (r_me + (u + 1) * s < p.split) got[u][r] = slot_load_issue(other[u] + r * 64);
+                    }
+#pragma unroll
+                for (int u = 0; u < 3; ++u)      // one wait; every loaded register is an operand of some statement here
+                    asm volatile("s_waitcnt vmcnt(0)" : "+v"(got[u][0]), "+v"(got[u][1]), "+v"(got[u][2]), "+v"(got[u][3])::"memory");
+                bool missing = false;
+#pragma unroll
+                for (int u = 0; u < 3; ++u)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) missing |= got[u][r][j] == SLOT_EMPTY;
+                waiting = __ballot(missing) != 0 && ++spins < SLOT_SPIN_LIMIT;
+                if (waiting) __builtin_amdgcn_s_sleep(4);
+            } while (waiting);
+#pragma unroll
+            for (int u = 0; u < 3; ++u) {
+                if (r_me + (u + 1) * s >= p.split) break;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) mine[r][j] += __uint_as_float(got[u][r][j]);
+                    slot_store(other[u] + r * 64, empty);                       // ready for the next launch
+                }
+            }
+        }
+        if (r_me != 0) {
+            float4 *slot = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)me * 16 + wave * 4) * 64 + lane;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                u32x4 v;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[r][j]));
+                slot_store(slot + r * 64, v);
+            }
+            store_now = false;
+        }
+    }
+
+
+    if (store_now && t_of_lane < (int)n_valid) {
+        const uint32_t n_col = (nt0 + t_of_lane) * 32 + fc * 16 + q * 4;   // first of this lane's 4 columns
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t row_in_band = wave * 8 + kh * 4 + r;
+            const uint32_t row = mt * 32 + row_in_band;
+            if (row >= p.m) continue;
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float x = mine[r][j] * F::unscale;
+                if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
+                v[j] = apply_activation<ACT>(x);
+            }
+            uint64_t elem;   // element offset of the 4-column run in C
+            if (p.c_tiled) {
+                const uint64_t tile = ((uint64_t)bb * p.mt + mt) * p.nt + nt0 + t_of_lane;
+                elem = tile * 1024 + ((row_in_band >> 4) * 2 + fc) * 256 + (row_in_band & 15) * 16 + q * 4;
+            } else {
+                elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
+            }
+            if (p.c_f32) {
+                *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+                const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
+                const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
+                *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // host side: decomposition, workspace, launch
 // ---------------------------------------------------------------------------------------------------------
 static uint32_t env_u32(const char *name, uint32_t fallback) {
@@ -411,15 +694,17 @@ static uint32_t env_u32(const char *name, uint32_t fallback) {
 
 struct Decomposition { uint32_t mt, kt, nt, ngroups, workgroups, split; uint64_t groups, units; };
 
-static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
+static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, bool wide) {
     Decomposition d{};
+    const uint32_t group_tiles = wide ? WIDE_TILES : GROUP_TILES;
     d.mt = (m + 31) / 32; d.kt = k / 32; d.nt = n / 32;
-    d.ngroups = (d.nt + GROUP_TILES - 1) / GROUP_TILES;
+    d.ngroups = (d.nt + group_tiles - 1) / group_tiles;
     d.groups = (uint64_t)batch * d.mt * d.ngroups;
     d.units = d.groups * d.kt;
-    // workgroups to aim for: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone nearly get there,
-    // x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot reset)
-    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", d.groups >= 256 ? 768 : 512);
+    // workgroups to aim for.  64-column kernel: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone
+    // nearly get there, x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot
+    // reset); 128-column kernel: 256 CUs x 2.
+    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", wide ? 256 * WIDE_WGS_PER_CU : d.groups >= 256 ? 768 : 512);
     // cut every output's k range into as many parts as keeps the chip full, every wavefront keeping >= 2 k-tiles
     // (the kernel can also deal the units out evenly across output boundaries, split == 0, but a workgroup that is
     // consumer of one output and producer of the next would then make its successor wait: not offered)
@@ -455,8 +740,13 @@ static int own_slots(size_t bytes, void **slots) {
     return TTMI_OK;
 }
 
-int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) {
-    const Decomposition d = decompose(x.batch, x.m, x.k, x.n);
+static size_t slot_bytes_needed(const Decomposition &d, bool wide) {
+    if (d.split == 1) return 0;                     // every output belongs to one workgroup: no slot is touched
+    return wide ? (size_t)d.workgroups * WIDE_SLOT_BYTES : (size_t)2 * d.workgroups * SLOT_BYTES;
+}
+
+static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
+    const Decomposition d = decompose(x.batch, x.m, x.k, x.n, wide);
     MatmulDev p{};
     p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
@@ -467,10 +757,9 @@ int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) {
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
     if (d.units > 0x7fffffffull || d.groups * (d.split ? d.split : 1) > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
-    const size_t need = (size_t)2 * d.workgroups * SLOT_BYTES;
+    const size_t need = slot_bytes_needed(d, wide);
     void *slots = nullptr;
-    if (d.split == 1) {
-        // every output belongs to one workgroup: no slot is touched
+    if (need == 0) {
     } else if (x.workspace) {
         if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
         if (reinterpret_cast<uintptr_t>(x.workspace) & 255u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 256-byte aligned");
@@ -484,7 +773,9 @@ int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) {
         return rc;
     }
     p.slots = (float *)slots;
-#define TTMI_LAUNCH(W, ACT) hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
+#define TTMI_LAUNCH(W, ACT)                                                                                     \
+    if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p);        \
+    else hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
 #define TTMI_LAUNCH_ACT(W)                                              \
     switch (x.activation) {                                             \
         case TTMI_ACT_RELU: TTMI_LAUNCH(W, TTMI_ACT_RELU); break;       \
@@ -495,37 +786,47 @@ int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) {
     if (x.b_fmt == TTMI_BFLOAT8_B) { TTMI_LAUNCH_ACT(7) } else { TTMI_LAUNCH_ACT(3) }
 #undef TTMI_LAUNCH_ACT
 #undef TTMI_LAUNCH
-    return check_launch("matmul_stream_kernel");
+    return check_launch(wide ? "matmul_wide_kernel" : "matmul_stream_kernel");
 }
 
-// Which kernel a shape goes to.  Up to 127 rows the weights are streamed once per 32-row band (HBM-bound); taller
-// activations are MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows on (two or more 256-row blocks
-// share every weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
-// TTMI_MATMUL_KERNEL=stream|tile|expanded overrides the choice (for tests and measurements).
-enum class Kernel { Stream, Tile, Expanded };
-static Kernel choose_kernel(uint32_t m) {
+int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) { return launch_streaming(x, st, false); }
+int matmul_bfp_wide(const MatmulArgs &x, hipStream_t st) { return launch_streaming(x, st, true); }
+
+// Which kernel a shape goes to.  Up to 127 rows the weights are streamed once per 32-row band (HBM-bound): in
+// 128-column units when that fills the chip with at most three k ranges per output (measured: beyond that the
+// hand-over of partial sums costs more than the wider unit saves), in 64-column units otherwise (twice the output groups, so half the k ranges per output).  Taller activations are
+// MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows on (two or more 256-row blocks share every
+// weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
+// TTMI_MATMUL_KERNEL=stream|wide|tile|expanded overrides the choice (for tests and measurements).
+enum class Kernel { Stream, Wide, Tile, Expanded };
+static Kernel choose_kernel(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
     const char *force = getenv("TTMI_MATMUL_KERNEL");
     if (force && force[0] == 's') return Kernel::Stream;
+    if (force && force[0] == 'w') return Kernel::Wide;
     if (force && force[0] == 't') return Kernel::Tile;
     if (force && force[0] == 'e') return Kernel::Expanded;
-    return m >= 512 ? Kernel::Expanded : m >= 128 ? Kernel::Tile : Kernel::Stream;
+    if (m >= 512) return Kernel::Expanded;
+    if (m >= 128) return Kernel::Tile;
+    return decompose(batch, m, k, n, true).split <= 3 ? Kernel::Wide : Kernel::Stream;
 }
 
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int) {
     if (!batch || !m || !k || !n) return 0;
-    switch (choose_kernel(m)) {
+    const Kernel kernel = choose_kernel(batch, m, k, n);
+    switch (kernel) {
         case Kernel::Expanded: return matmul_expanded_workspace_bytes(batch, k, n);   // as if every slice had weights of its own
         case Kernel::Tile: return 0;
         default: break;
     }
-    const Decomposition d = decompose(batch, m, k, n);
-    return d.split == 1 ? 0 : (size_t)2 * d.workgroups * SLOT_BYTES;
+    const bool wide = kernel == Kernel::Wide;
+    return slot_bytes_needed(decompose(batch, m, k, n, wide), wide);
 }
 
 int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
-    switch (choose_kernel(x.m)) {
+    switch (choose_kernel(x.batch, x.m, x.k, x.n)) {
         case Kernel::Expanded: return matmul_bfp_expanded(x, st);
         case Kernel::Tile: return matmul_bfp_tiled(x, st);
+        case Kernel::Wide: return matmul_bfp_wide(x, st);
         default: return matmul_bfp_stream(x, st);
     }
 }

@@ -36,6 +36,7 @@ struct MatmulArgs {
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
 int matmul_bfp(const MatmulArgs &args, hipStream_t st);         // streaming kernel (decode shapes) or the tiled one
 int matmul_bfp_stream(const MatmulArgs &args, hipStream_t st);
+int matmul_bfp_wide(const MatmulArgs &args, hipStream_t st);     // the streaming kernel with 128-column units
 int matmul_bfp_tiled(const MatmulArgs &args, hipStream_t st);
 int matmul_bfp_expanded(const MatmulArgs &args, hipStream_t st);   // expand the weights to bf16 once, then a bf16 GEMM
 size_t matmul_expanded_workspace_bytes(uint32_t b_batch, uint32_t k, uint32_t n);
