@@ -4,7 +4,7 @@ bfp_matmul.hip issues some global loads as inline assembly and waits for them wi
 compiler's waits would drain the prefetch pipeline.  The compiler therefore believes that a loaded register holds its
 value as soon as the load has issued.  That is only safe if it never copies, moves, reads or reuses such a register
 between the load and the point where the data is taken over.  This script reads the device assembly of the file,
-builds the control-flow graph of each streaming kernel and propagates the set of registers with a load in flight:
+builds the control-flow graph of each streaming kernel (64- and 128-column) and propagates the set of registers with a load in flight:
 
   ring loads   (inline global_load_dwordx4 without sc1: activations in flight across loop iterations) are in flight
                until an inline `v_mov_b32 vX, vN` reads register N
@@ -158,16 +158,16 @@ def _check_kernel(name, body, problems):
             problems.append(f)
 
 
-def check(path: str, kernel_substring: str = "matmul_stream_kernel") -> int:
+def check(path: str, kernel_substrings=("matmul_stream_kernel", "matmul_wide_kernel")) -> int:
     problems, checked = [], 0
     with open(path) as f:
         lines = f.read().split("\n")
     for name, body in _kernels(lines):
-        if kernel_substring in name:
+        if any(k in name for k in kernel_substrings):
             checked += 1
             _check_kernel(name, body, problems)
     if not checked:
-        problems.append(f"no kernel matching '{kernel_substring}' in {path}")
+        problems.append(f"no kernel matching {kernel_substrings} in {path}")
     for p in problems[:40]:
         print("check_isa:", p, file=sys.stderr)
     if len(problems) > 40:

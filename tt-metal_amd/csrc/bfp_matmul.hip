@@ -39,6 +39,7 @@ struct MatmulDev {
     float *slots;            // 2 slots of 32x64 fp32 per workgroup, for outputs shared between workgroups (see SLOT_EMPTY)
     uint32_t batch, b_batch, m, k, n;
     uint32_t mt, kt, nt, ngroups;
+    uint32_t groups;         // batch * mt * ngroups
     uint32_t workgroups;     // P
     uint32_t units;          // U = batch * mt * ngroups * kt
     uint32_t share, extra;   // U = P * share + extra: the first `extra` workgroups take share + 1 units
@@ -113,6 +114,15 @@ __global__ __launch_bounds__(256) void fill_slots_kernel(u32x4 *slots, uint32_t 
 
 template <int... Is, typename Fn> __device__ __forceinline__ void static_for(std::integer_sequence<int, Is...>, Fn fn) {
     (fn(std::integral_constant<int, Is>{}), ...);
+}
+// step(J) for J = FROM, FROM + 1, ... while first + J < total and J < COUNT
+template <int FROM, int COUNT, typename Step> __device__ __forceinline__ void nested_steps(uint32_t first, uint32_t total, Step step) {
+    if constexpr (FROM < COUNT) {
+        if (first + FROM < total) {
+            step(std::integral_constant<int, FROM>{});
+            nested_steps<FROM + 1, COUNT>(first, total, step);
+        }
+    }
 }
 // waits until at most min(younger, MOST) * PER requests are in flight
 template <int MOST, int PER> __device__ __forceinline__ void wait_for_younger(uint32_t younger) {
@@ -261,7 +271,8 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
             const uint32_t at = i + J;
             if (at >= total) return;
             wait_for_younger<STAGES - 1, NLOAD + A_LOADS>(total - 1 - at);
-            work(std::integral_constant<int, J % STAGES>{}, std::integral_constant<int, -1>{}, at + STAGES < total);
+            // a unit requested from here would be number J + STAGES of the tail: only the first STAGES - 1 steps can have one
+            work(std::integral_constant<int, J % STAGES>{}, std::integral_constant<int, -1>{}, J + STAGES < 2 * STAGES - 1 && at + STAGES < total);
         });
 
         wait_vmcnt<0>();   // nothing in flight any more (already true; also what the build-time ISA check keys on)
@@ -438,7 +449,7 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
 
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: branches on it are uniform
     const int c32 = lane & 31, kh = lane >> 5;
     const int t_of_lane = c32 >> 3, pair = t_of_lane >> 1, t_in = t_of_lane & 1, fc = (c32 >> 2) & 1, q = c32 & 3;
 
@@ -485,7 +496,19 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
-    u32x4 a_ring[WIDE_STAGES][2] = {};
+    // The ring registers are cleared by instructions the compiler cannot see through: entries it knows to be zero it
+    // would keep in a shared constant register and copy loaded entries around at joins, while their loads are in flight.
+    u32x4 a_ring[WIDE_STAGES][2];
+#pragma unroll
+    for (int s = 0; s < WIDE_STAGES; ++s)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                uint32_t zero;
+                asm volatile("v_mov_b32 %0, 0" : "=v"(zero));
+                a_ring[s][h][e] = zero;
+            }
 
     // Requests one unit: its 4 packed tiles straight into LDS stage S, its activations into a_ring[S] (inline assembly
     // for the loads and their waits, as in the 64-column kernel).
@@ -534,27 +557,29 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     // This wavefront's units: k_begin + wave, + WAVES, ...; unit i lives in stage i % STAGES and is requested STAGES
     // units ahead (see the 64-column kernel for the bookkeeping of requests in flight).
     const uint32_t span = k_end - k_begin;
-    const uint32_t total = span > (uint32_t)wave ? (span - wave + WAVES - 1) / WAVES : 0;
+    const bool computes = og < p.groups;             // the last `split` workgroups of a shared launch only collect
+    const uint32_t total = computes && span > (uint32_t)wave ? (span - wave + WAVES - 1) / WAVES : 0;
     using Last = std::integral_constant<int, WIDE_STAGES - 1>;
     constexpr auto stages = std::make_integer_sequence<int, WIDE_STAGES>{};
     uint32_t i = 0;
-    if (total >= 2 * WIDE_STAGES) {
-        static_for(stages, [&](auto s) __attribute__((always_inline)) { fetch(s); });
+    static_for(stages, [&](auto s) __attribute__((always_inline)) { if (total > (uint32_t)decltype(s)::value) fetch(s); });
+    // steady state: every unit worked on here has a successor to request, so the number of requests in flight at each
+    // wait is a constant the compiler can see
 #pragma unroll 1
-        for (; i + 2 * WIDE_STAGES <= total; i += WIDE_STAGES)
-            static_for(stages, [&](auto s) __attribute__((always_inline)) { work(s, Last{}, true); });
-    } else {
-        static_for(stages, [&](auto s) __attribute__((always_inline)) { if (total > (uint32_t)decltype(s)::value) fetch(s); });
-    }
-    static_for(std::make_integer_sequence<int, 2 * WIDE_STAGES - 1>{}, [&](auto j) __attribute__((always_inline)) {
+    for (; i + 2 * WIDE_STAGES <= total; i += WIDE_STAGES)
+        static_for(stages, [&](auto s) __attribute__((always_inline)) { work(s, Last{}, true); });
+    // at most 2 * STAGES - 1 units are left, starting in stage 0; the steps are nested (step J + 1 inside step J) so that
+    // a step that does not happen takes all later ones with it
+    nested_steps<0, 2 * WIDE_STAGES - 1>(i, total, [&](auto j) __attribute__((always_inline)) {
         constexpr int J = decltype(j)::value;
         const uint32_t at = i + J;
-        if (at >= total) return;
         wait_for_younger<WIDE_STAGES - 1, PER>(total - 1 - at);
-        work(std::integral_constant<int, J % WIDE_STAGES>{}, std::integral_constant<int, -1>{}, at + WIDE_STAGES < total);
+        // a unit requested from here would be number J + STAGES of the tail: only the first STAGES - 1 steps can have one
+        work(std::integral_constant<int, J % WIDE_STAGES>{}, std::integral_constant<int, -1>{}, J + WIDE_STAGES < 2 * WIDE_STAGES - 1 && at + WIDE_STAGES < total);
     });
 
     wait_vmcnt<0>();   // nothing in flight any more (already true; also what the build-time ISA check keys on)
+    __builtin_amdgcn_sched_barrier(0);   // and nothing of what follows is scheduled in front of it
     // ---- add the four wavefronts' partial sums through LDS ------------------------------------------------------
     // Every wavefront writes its 64 accumulator registers as 16 float4 (acc[j][4q4 .. 4q4+3]); wavefront w then keeps
     // q4 = w: rows 8w + 4kh + r (r = 0..3), columns 4*c32 + j.
@@ -578,107 +603,120 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         mine[0][j] = v.x; mine[1][j] = v.y; mine[2][j] = v.z; mine[3][j] = v.w;
     }
 
-    // ---- outputs shared with other workgroups ----------------------------------------------------------------
-    // The `split` workgroups of an output add their partial sums along a radix-4 tree over r = split - 1 - part: a
-    // workgroup whose r has zeros in its lowest base-4 digits collects, digit position by digit position, from
-    // r + s, r + 2s, r + 3s (s = 4^position) while they exist, adding them in that order; at its lowest non-zero digit
-    // it publishes its sums in its slot and is done.  r = 0 (the highest index) ends with the complete sum and stores.
-    // Whoever waits, waits for workgroups of lower index only: they were dispatched earlier and wait for nobody
-    // dispatched later, so they finish.  The order of the additions is fixed, the result does not depend on timing.
-    // Slots work as in the 64-column kernel (SLOT_EMPTY until written, put back by the reader), one per workgroup;
-    // wavefront w of every workgroup holds the same rows, so the hand-over is wavefront to wavefront.
-    bool store_now = true;
-    if (p.split > 1) {
-        const uint32_t first = og * p.split, r_me = p.split - 1 - part;
-        const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
-        const u32x4 nothing = {0u, 0u, 0u, 0u};
-        for (uint32_t s = 1; s < p.split; s *= 4) {
-            if ((r_me / s) & 3u) break;
-            if (r_me + s >= p.split) break;
-            u32x4 got[3][4];
-            float4 *other[3];
+    // ---- store, or hand over ------------------------------------------------------------------------------------
+    // A chunk = 4 adjacent columns of one row = what one lane holds per r: chunk number (w * 4 + r) * 64 + lane, 1024
+    // per output group.  Stores chunk `idx` of output group `group` (sums still carry the common factor).
+    auto store_chunk = [&](uint32_t group, uint32_t idx, const float (&sums)[4]) __attribute__((always_inline)) {
+        const uint32_t lane_of = idx & 63, r_of = (idx >> 6) & 3, w_of = idx >> 8;
+        const uint32_t c32_of = lane_of & 31, t_of = c32_of >> 3, fc_of = (c32_of >> 2) & 1, q_of = c32_of & 3;
+        const uint32_t band_of = group / p.ngroups, mt_of = band_of % p.mt, bb_of = band_of / p.mt;
+        const uint32_t nt_of = (group % p.ngroups) * WIDE_TILES + t_of;
+        const uint32_t row_in_band = w_of * 8 + (lane_of >> 5) * 4 + r_of, row = mt_of * 32 + row_in_band;
+        if (nt_of >= p.nt || row >= p.m) return;
+        const uint32_t n_col = nt_of * 32 + fc_of * 16 + q_of * 4;           // first of the 4 columns
+        float v[4];
 #pragma unroll
-            for (int u = 0; u < 3; ++u) {
-                const uint32_t r_other = min(r_me + (u + 1) * s, p.split - 1);
-                other[u] = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)(first + p.split - 1 - r_other) * 16 + wave * 4) * 64 + lane;
-            }
-            uint32_t spins = 0;
-            bool waiting;
+        for (int j = 0; j < 4; ++j) {
+            float x = sums[j] * F::unscale;
+            if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
+            v[j] = apply_activation<ACT>(x);
+        }
+        uint64_t elem;   // element offset of the 4-column run in C
+        if (p.c_tiled) {
+            const uint64_t tile = ((uint64_t)bb_of * p.mt + mt_of) * p.nt + nt_of;
+            elem = tile * 1024 + ((row_in_band >> 4) * 2 + fc_of) * 256 + (row_in_band & 15) * 16 + q_of * 4;
+        } else {
+            elem = ((uint64_t)bb_of * p.m + row) * p.n + n_col;
+        }
+        if (p.c_f32) {
+            *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+            const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
+            const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
+            *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
+        }
+    };
+
+    if (p.split == 1) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) store_chunk(og, (wave * 4 + r) * 64 + lane, mine[r]);
+        return;
+    }
+    // Outputs shared between `split` workgroups.  Every workgroup publishes its 1024 chunks in its slot; the sums of
+    // output group g are then formed by the `split` workgroups of group g + 1 (after the last group: by `split`
+    // workgroups launched for nothing else), workgroup j of them taking chunks [1024 j / split, 1024 (j + 1) / split)
+    // from every contributor, in contributor order (so the result does not depend on timing), storing them and putting
+    // SLOT_EMPTY back.  The work of collecting is spread evenly, every chunk is read by exactly one thread, and
+    // whoever waits, waits for workgroups of lower index only: they were dispatched earlier and wait for nobody
+    // dispatched later, so they finish.
+    float4 *const all_slots = reinterpret_cast<float4 *>(p.slots);
+    if (computes) {
+        float4 *slot = all_slots + ((uint64_t)me * 16 + wave * 4) * 64 + lane;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            u32x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[r][j]));
+            slot_store(slot + r * 64, v);
+        }
+    }
+    if (og == 0) return;
+    const uint32_t target = og - 1;
+    const uint32_t lo = (part * 1024u) / p.split, hi = ((part + 1) * 1024u) / p.split;
+    const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
+    for (uint32_t idx0 = lo; idx0 < hi; idx0 += 256) {
+        const bool active = idx0 + threadIdx.x < hi;                       // idle lanes re-read the last chunk and drop it
+        const uint32_t idx = active ? idx0 + threadIdx.x : hi - 1;
+        float4 *const at = all_slots + (uint64_t)target * p.split * 1024 + idx;   // contributor c: at + c * 1024
+        uint32_t spins = 0;
+        bool waiting;
+        // cheap poll first (one contributor), then everything, checked word by word
+        do {
+            u32x4 probe = slot_load_issue(at + (uint64_t)(p.split - 1) * 1024);
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(probe)::"memory");
+            const bool missing = active && (probe[0] == SLOT_EMPTY || probe[1] == SLOT_EMPTY || probe[2] == SLOT_EMPTY || probe[3] == SLOT_EMPTY);
+            waiting = __ballot(missing) != 0 && ++spins < SLOT_SPIN_LIMIT;
+            if (waiting) __builtin_amdgcn_s_sleep(8);
+        } while (waiting);
+        float sums[4] = {0.f, 0.f, 0.f, 0.f};
+        // N contributors at a time, N a compile-time constant: loads under a condition would have the compiler merge
+        // loaded and unloaded registers (that is, copy them) while the loads are in flight
+        auto collect = [&](auto count_tag, uint32_t c0) __attribute__((always_inline)) {
+            constexpr int N = decltype(count_tag)::value;
+            u32x4 got[N];
             do {
 #pragma unroll
-                for (int u = 0; u < 3; ++u)
+                for (int u = 0; u < N; ++u) got[u] = slot_load_issue(at + (uint64_t)(c0 + u) * 1024);
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        got[u][r] = nothing;
-                        if (r_me + (u + 1) * s < p.split) got[u][r] = slot_load_issue(other[u] + r * 64);
-                    }
-#pragma unroll
-                for (int u = 0; u < 3; ++u)      // one wait; every loaded register is an operand of some statement here
-                    asm volatile("s_waitcnt vmcnt(0)" : "+v"(got[u][0]), "+v"(got[u][1]), "+v"(got[u][2]), "+v"(got[u][3])::"memory");
+                for (int u = 0; u < N; ++u) asm volatile("s_waitcnt vmcnt(0)" : "+v"(got[u])::"memory");
                 bool missing = false;
 #pragma unroll
-                for (int u = 0; u < 3; ++u)
+                for (int u = 0; u < N; ++u)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) missing |= got[u][r][j] == SLOT_EMPTY;
-                waiting = __ballot(missing) != 0 && ++spins < SLOT_SPIN_LIMIT;
+                    for (int j = 0; j < 4; ++j) missing |= got[u][j] == SLOT_EMPTY;
+                waiting = __ballot(missing && active) != 0 && ++spins < SLOT_SPIN_LIMIT;
                 if (waiting) __builtin_amdgcn_s_sleep(4);
             } while (waiting);
 #pragma unroll
-            for (int u = 0; u < 3; ++u) {
-                if (r_me + (u + 1) * s >= p.split) break;
+            for (int u = 0; u < N; ++u) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) mine[r][j] += __uint_as_float(got[u][r][j]);
-                    slot_store(other[u] + r * 64, empty);                       // ready for the next launch
-                }
+                for (int j = 0; j < 4; ++j) sums[j] += __uint_as_float(got[u][j]);
+                if (active) slot_store(at + (uint64_t)(c0 + u) * 1024, empty);          // ready for the next launch
             }
+        };
+        uint32_t c0 = 0;
+        for (; c0 + 8 <= p.split; c0 += 8) collect(std::integral_constant<int, 8>{}, c0);
+        switch (p.split - c0) {
+            case 1: collect(std::integral_constant<int, 1>{}, c0); break;
+            case 2: collect(std::integral_constant<int, 2>{}, c0); break;
+            case 3: collect(std::integral_constant<int, 3>{}, c0); break;
+            case 4: collect(std::integral_constant<int, 4>{}, c0); break;
+            case 5: collect(std::integral_constant<int, 5>{}, c0); break;
+            case 6: collect(std::integral_constant<int, 6>{}, c0); break;
+            case 7: collect(std::integral_constant<int, 7>{}, c0); break;
+            default: break;
         }
-        if (r_me != 0) {
-            float4 *slot = reinterpret_cast<float4 *>(p.slots) + ((uint64_t)me * 16 + wave * 4) * 64 + lane;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                u32x4 v;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[r][j]));
-                slot_store(slot + r * 64, v);
-            }
-            store_now = false;
-        }
-    }
-
-
-    if (store_now && t_of_lane < (int)n_valid) {
-        const uint32_t n_col = (nt0 + t_of_lane) * 32 + fc * 16 + q * 4;   // first of this lane's 4 columns
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t row_in_band = wave * 8 + kh * 4 + r;
-            const uint32_t row = mt * 32 + row_in_band;
-            if (row >= p.m) continue;
-            float v[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float x = mine[r][j] * F::unscale;
-                if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
-                v[j] = apply_activation<ACT>(x);
-            }
-            uint64_t elem;   // element offset of the 4-column run in C
-            if (p.c_tiled) {
-                const uint64_t tile = ((uint64_t)bb * p.mt + mt) * p.nt + nt0 + t_of_lane;
-                elem = tile * 1024 + ((row_in_band >> 4) * 2 + fc) * 256 + (row_in_band & 15) * 16 + q * 4;
-            } else {
-                elem = ((uint64_t)bb * p.m + row) * p.n + n_col;
-            }
-            if (p.c_f32) {
-                *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
-            } else {
-                const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
-                const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
-                *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
-            }
-        }
+        if (active) store_chunk(target, idx, sums);
     }
 }
 
@@ -701,14 +739,17 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     d.ngroups = (d.nt + group_tiles - 1) / group_tiles;
     d.groups = (uint64_t)batch * d.mt * d.ngroups;
     d.units = d.groups * d.kt;
-    // workgroups to aim for.  64-column kernel: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone
-    // nearly get there, x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot
-    // reset); 128-column kernel: 256 CUs x 2.
-    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", wide ? 256 * WIDE_WGS_PER_CU : d.groups >= 256 ? 768 : 512);
-    // cut every output's k range into as many parts as keeps the chip full, every wavefront keeping >= 2 k-tiles
-    // (the kernel can also deal the units out evenly across output boundaries, split == 0, but a workgroup that is
-    // consumer of one output and producer of the next would then make its successor wait: not offered)
-    uint64_t parts = d.groups >= resident ? 1 : resident / d.groups;
+    // Workgroups to aim for, every output's k range being cut into as many parts as get there (every wavefront keeping
+    // >= 2 k-tiles).  64-column kernel: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone nearly get
+    // there, x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot reset; the kernel
+    // can also deal the units out evenly across output boundaries, split == 0, but a workgroup that is consumer of one
+    // output and producer of the next would then make its successor wait: not offered).  128-column kernel: two
+    // workgroups per CU (all it can hold, the collecting workgroups included) when that takes few parts per output, one
+    // per CU when the outputs are few (measured: many short k ranges cost more than the second workgroup gains).
+    const bool few = d.groups < 100;
+    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", wide ? (few ? 256 : 512) : d.groups >= 256 ? 768 : 512);
+    uint64_t parts = d.groups >= resident ? 1 : wide && !few ? resident / (d.groups + 1) : resident / d.groups;
+    if (parts == 0) parts = 1;
     const uint64_t most = d.kt / (2 * WAVES) ? d.kt / (2 * WAVES) : 1;
     if (parts > most) parts = most;
     d.split = (uint32_t)parts;
@@ -750,7 +791,7 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     MatmulDev p{};
     p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
-    p.mt = d.mt; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
+    p.mt = d.mt; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.groups = (uint32_t)d.groups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
     p.share = p.units / p.workgroups; p.extra = p.units % p.workgroups; p.split = d.split;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE;
     p.c_f32 = x.c_dtype == TTMI_FLOAT32;
@@ -774,7 +815,7 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     }
     p.slots = (float *)slots;
 #define TTMI_LAUNCH(W, ACT)                                                                                     \
-    if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p);        \
+    if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
     else hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
 #define TTMI_LAUNCH_ACT(W)                                              \
     switch (x.activation) {                                             \
@@ -792,14 +833,13 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
 int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) { return launch_streaming(x, st, false); }
 int matmul_bfp_wide(const MatmulArgs &x, hipStream_t st) { return launch_streaming(x, st, true); }
 
-// Which kernel a shape goes to.  Up to 127 rows the weights are streamed once per 32-row band (HBM-bound): in
-// 128-column units when that fills the chip with at most three k ranges per output (measured: beyond that the
-// hand-over of partial sums costs more than the wider unit saves), in 64-column units otherwise (twice the output groups, so half the k ranges per output).  Taller activations are
-// MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows on (two or more 256-row blocks share every
-// weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
+// Which kernel a shape goes to.  Up to 127 rows the weights are streamed once per 32-row band (HBM-bound): one band in
+// 128-column units, several bands in 64-column units (measured: 43 against 46 us for 64 rows of the Falcon shape).
+// Taller activations are MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows on (two or more
+// 256-row blocks share every weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
 // TTMI_MATMUL_KERNEL=stream|wide|tile|expanded overrides the choice (for tests and measurements).
 enum class Kernel { Stream, Wide, Tile, Expanded };
-static Kernel choose_kernel(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
+static Kernel choose_kernel(uint32_t m) {
     const char *force = getenv("TTMI_MATMUL_KERNEL");
     if (force && force[0] == 's') return Kernel::Stream;
     if (force && force[0] == 'w') return Kernel::Wide;
@@ -807,12 +847,12 @@ static Kernel choose_kernel(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) 
     if (force && force[0] == 'e') return Kernel::Expanded;
     if (m >= 512) return Kernel::Expanded;
     if (m >= 128) return Kernel::Tile;
-    return decompose(batch, m, k, n, true).split <= 3 ? Kernel::Wide : Kernel::Stream;
+    return m <= 32 ? Kernel::Wide : Kernel::Stream;
 }
 
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int) {
     if (!batch || !m || !k || !n) return 0;
-    const Kernel kernel = choose_kernel(batch, m, k, n);
+    const Kernel kernel = choose_kernel(m);
     switch (kernel) {
         case Kernel::Expanded: return matmul_expanded_workspace_bytes(batch, k, n);   // as if every slice had weights of its own
         case Kernel::Tile: return 0;
@@ -823,7 +863,7 @@ size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n
 }
 
 int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
-    switch (choose_kernel(x.batch, x.m, x.k, x.n)) {
+    switch (choose_kernel(x.m)) {
         case Kernel::Expanded: return matmul_bfp_expanded(x, st);
         case Kernel::Tile: return matmul_bfp_tiled(x, st);
         case Kernel::Wide: return matmul_bfp_wide(x, st);
