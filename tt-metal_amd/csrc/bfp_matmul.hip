@@ -670,8 +670,8 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         float4 *const at = all_slots + (uint64_t)target * p.split * 1024 + idx;   // contributor c: at + c * 1024
         uint32_t spins = 0;
         bool waiting;
-        // cheap poll first (one contributor), then everything, checked word by word
-        do {
+        // workgroups with nothing else to do poll cheaply first (one contributor); then everything, checked word by word
+        if (!computes) do {
             u32x4 probe = slot_load_issue(at + (uint64_t)(p.split - 1) * 1024);
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(probe)::"memory");
             const bool missing = active && (probe[0] == SLOT_EMPTY || probe[1] == SLOT_EMPTY || probe[2] == SLOT_EMPTY || probe[3] == SLOT_EMPTY);
