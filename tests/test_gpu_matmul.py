@@ -163,10 +163,12 @@ def test_caller_workspace(oracle):
 @pytest.mark.parametrize("kernel", ["stream", "wide", "tile", "tile256", "expanded"])
 @pytest.mark.parametrize("fmt", [BFP8, BFP4])
 @pytest.mark.parametrize("batch,b_batch,m,k,n", [(1, 1, 256, 128, 256), (1, 1, 300, 96, 288), (2, 1, 130, 160, 96), (1, 1, 288, 224, 96),
-                                                 (2, 2, 512, 64, 544), (1, 1, 40, 32, 2080)])
+                                                 (2, 2, 512, 64, 544), (1, 1, 40, 32, 2080),
+                                                 (2, 2, 32, 1024, 224), (3, 1, 24, 768, 160)])
 def test_every_kernel_on_every_shape(oracle, kernel, fmt, batch, b_batch, m, k, n, monkeypatch):
     """Each GEMM kernel forced onto shapes it would not be chosen for: ragged row blocks, odd tile counts, one k step,
-    more than eight 256-column blocks, shared and per-slice weights; TILE layout in and out, bias and activation."""
+    more than eight 256-column blocks, shared and per-slice weights, k ranges long enough for the streaming kernels to
+    share outputs between workgroups (with batches and ragged column groups); TILE layout in and out, bias and activation."""
     monkeypatch.setenv("TTMI_MATMUL_KERNEL", kernel[:4])
     if kernel == "tile256":
         monkeypatch.setenv("TTMI_MATMUL_BM", "256")
