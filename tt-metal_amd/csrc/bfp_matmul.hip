@@ -429,11 +429,11 @@ constexpr int WIDE_COLS = WIDE_TILES * 32;
 #define TTMI_WIDE_WGS_PER_CU 2
 #endif
 #ifndef TTMI_WIDE_STAGES
-#define TTMI_WIDE_STAGES 3
+#define TTMI_WIDE_STAGES 2      // measured: 2 beats 3 by 1.5 us on the Falcon h_to_4h shape (less code, fewer registers), 4 leaves one workgroup per CU
 #endif
 constexpr int WIDE_WGS_PER_CU = TTMI_WIDE_WGS_PER_CU;
 constexpr int WIDE_STAGES = TTMI_WIDE_STAGES;
-constexpr int WIDE_REDUCE_BYTES = WAVES * 64 * 64 * 4;     // every wavefront lays out its 64 accumulator registers
+constexpr int WIDE_REDUCE_BYTES = WAVES * 32 * 64 * 4;     // every wavefront lays out half of its 64 accumulator registers
 constexpr size_t WIDE_SLOT_BYTES = 32 * WIDE_COLS * sizeof(float);
 
 template <int W, int ACT>
@@ -581,26 +581,32 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     wait_vmcnt<0>();   // nothing in flight any more (already true; also what the build-time ISA check keys on)
     __builtin_amdgcn_sched_barrier(0);   // and nothing of what follows is scheduled in front of it
     // ---- add the four wavefronts' partial sums through LDS ------------------------------------------------------
-    // Every wavefront writes its 64 accumulator registers as 16 float4 (acc[j][4q4 .. 4q4+3]); wavefront w then keeps
-    // q4 = w: rows 8w + 4kh + r (r = 0..3), columns 4*c32 + j.
-    __syncthreads();
+    // In two passes (operands j = 0, 1, then 2, 3; 32 KB each) every wavefront writes its accumulator registers as
+    // float4 (acc[j][4q4 .. 4q4+3]); wavefront w then keeps q4 = w: rows 8w + 4kh + r (r = 0..3), columns 4*c32 + j.
     float4 *red = reinterpret_cast<float4 *>(lds);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4)
-            red[(wave * 16 + j * 4 + q4) * 64 + lane] = make_float4(acc[j][4 * q4], acc[j][4 * q4 + 1], acc[j][4 * q4 + 2], acc[j][4 * q4 + 3]);
-    __syncthreads();
     float mine[4][4];   // [r][j]
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int pass = 0; pass < 2; ++pass) {
+        __syncthreads();
 #pragma unroll
-        for (int sw = 0; sw < WAVES; ++sw) {
-            const float4 x = red[(sw * 16 + j * 4 + wave) * 64 + lane];
-            v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
+        for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int j = pass * 2 + jj;
+                red[(wave * 8 + jj * 4 + q4) * 64 + lane] = make_float4(acc[j][4 * q4], acc[j][4 * q4 + 1], acc[j][4 * q4 + 2], acc[j][4 * q4 + 3]);
+            }
+        __syncthreads();
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = pass * 2 + jj;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int sw = 0; sw < WAVES; ++sw) {
+                const float4 x = red[(sw * 8 + jj * 4 + wave) * 64 + lane];
+                v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
+            }
+            mine[0][j] = v.x; mine[1][j] = v.y; mine[2][j] = v.z; mine[3][j] = v.w;
         }
-        mine[0][j] = v.x; mine[1][j] = v.y; mine[2][j] = v.z; mine[3][j] = v.w;
     }
 
     // ---- store, or hand over ------------------------------------------------------------------------------------
@@ -747,7 +753,7 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     // workgroups per CU (all it can hold, the collecting workgroups included) when that takes few parts per output, one
     // per CU when the outputs are few (measured: many short k ranges cost more than the second workgroup gains).
     const bool few = d.groups < 100;
-    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", wide ? (few ? 256 : 512) : d.groups >= 256 ? 768 : 512);
+    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", wide ? (few ? 256 : 256 * WIDE_WGS_PER_CU) : d.groups >= 256 ? 768 : 512);
     uint64_t parts = d.groups >= resident ? 1 : wide && !few ? resident / (d.groups + 1) : resident / d.groups;
     if (parts == 0) parts = 1;
     const uint64_t most = d.kt / (2 * WAVES) ? d.kt / (2 * WAVES) : 1;
