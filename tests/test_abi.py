@@ -39,6 +39,26 @@ def test_size_helpers_need_no_gpu():
     assert L.ttmi_tiled_size_bytes(3, 6, 7, 3) == 6 * 1088
 
 
+def test_matmul_workspace_sizes_follow_the_decomposition(monkeypatch):
+    """What a caller has to bring for a GEMM of its own stream: 16 KB of partial-sum slots per computing workgroup of the
+    128-column kernel (one band of rows), nothing when every output has a workgroup of its own, the expanded weights
+    (2 bytes each) from 512 rows on."""
+    from ttmi import capi
+
+    if not os.path.exists(capi.LIB_PATH):
+        pytest.skip("libttmi.so not built")
+    for name in ("TTMI_MATMUL_KERNEL", "TTMI_MATMUL_WGS", "TTMI_MATMUL_BM"):
+        monkeypatch.delenv(name, raising=False)
+    ws = capi.lib().ttmi_matmul_bfp_workspace_bytes
+    assert ws(1, 32, 4544, 18176, 3) == 142 * 3 * 16384        # 142 groups of 128 columns, 512 // 143 = 3 k ranges each
+    assert ws(1, 32, 18176, 4544, 3) == 36 * 7 * 16384         # 36 groups (the last one half empty), 256 // 36 = 7
+    assert ws(1, 32, 64, 4096, 3) == 0                         # 2 k-tiles: never shared
+    assert ws(1, 64, 4544, 18176, 3) == 0                      # two bands, 64-column kernel: 568 groups fill the chip
+    assert ws(1, 256, 4096, 4096, 3) == 0                      # fused tiled kernels
+    assert ws(1, 2048, 4096, 14336, 3) == 4096 * 14336 * 2     # expanded weights
+    assert ws(0, 32, 64, 64, 3) == 0
+
+
 def test_argument_validation_returns_errors_without_launching():
     from ttmi import capi
 
