@@ -245,6 +245,34 @@ def test_decode_gemm_in_a_hip_graph(oracle):
         assert torch.equal(other.view(torch.int16), eager.view(torch.int16))
 
 
+def test_decode_gemms_on_two_streams_at_once(oracle):
+    """Two decode GEMMs, each with a workspace of its own, queued on two streams without waiting for each other: neither
+    grid is resident as a whole while the other runs, and the hand-over of partial sums must neither stall nor mix.  Every
+    result equals the one computed alone."""
+    shapes = [(32, 4096, 1024, BFP8, 92), (32, 2048, 4096, BFP4, 94)]
+    L = capi.lib()
+    jobs = []
+    for m, k, n, fmt, seed in shapes:
+        a = bf16_dev(workloads.activations_bf16(m, k, seed=seed))
+        words = capi.pack_tensor(fmt, dev(workloads.weights_f32(k, n, seed=seed + 1)))
+        need = L.ttmi_matmul_bfp_workspace_bytes(1, m, k, n, fmt)
+        assert need > 0
+        alone = capi.matmul_bfp(a, capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n).clone()
+        jobs.append(dict(m=m, k=k, n=n, fmt=fmt, a=a, words=words, need=need, alone=alone, stream=torch.cuda.Stream(),
+                         ws=torch.full((need,), 0x33, dtype=torch.uint8, device="cuda"),
+                         outs=[torch.zeros(m * n, dtype=torch.bfloat16, device="cuda") for _ in range(12)]))
+    torch.cuda.synchronize()
+    for rep in range(12):
+        for j in jobs:
+            capi.check(L.ttmi_matmul_bfp(j["a"].data_ptr(), capi.ROW_MAJOR, j["words"].data_ptr(), j["fmt"], 1, 1, j["m"], j["k"], j["n"],
+                                         None, capi.ACT_NONE, j["outs"][rep].data_ptr(), capi.ROW_MAJOR, capi.BFLOAT16,
+                                         j["ws"].data_ptr(), j["need"], j["stream"].cuda_stream))
+    torch.cuda.synchronize()
+    for j in jobs:
+        for rep, out in enumerate(j["outs"]):
+            assert torch.equal(out.view(1, j["m"], j["n"]).view(torch.int16), j["alone"].view(torch.int16)), (j["n"], rep)
+
+
 @pytest.mark.parametrize("name,m,k,n,fmt,batch", workloads.DECODE_FALCON + workloads.DECODE_MISTRAL)
 def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch):
     a_bits = workloads.activations_bf16(m, k, seed=80)
