@@ -48,10 +48,12 @@ template <int ACT> __device__ __forceinline__ float apply_activation(float x) {
     return x;
 }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
-    uint32_t u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+// two floats -> two bf16 in one word (lo in the low half), round to nearest even: one v_cvt_pk_bf16_f32 on gfx950
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_rne(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // v_cvt_f32_ubyteN: byte N of a word as float, one instruction (the compiler otherwise extracts the field first)
@@ -253,7 +255,7 @@ __device__ __forceinline__ void store_wave_part(const Acc (&acc)[4][2], const St
                 else elem = (o.slice * o.m + row) * o.n + o.nt0 * 32 + col;
                 *reinterpret_cast<float2 *>(o.c + elem * 4) = make_float2(v0, v1);
             } else {
-                const uint32_t both = f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
+                const uint32_t both = f32x2_to_bf16x2_rne(v0, v1);
                 const uint32_t at = o.c_tiled ? rb * 4096 + t * 2048 + (((r32 >> 4) & 1) * 2 + fc) * 512 + (r32 & 15) * 32 + q * 8 + half * 4
                                               : (rb * 32 + r32) * 128 + col * 2;
                 *reinterpret_cast<uint32_t *>(lds_wave + at) = both;

@@ -23,6 +23,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <mutex>
+
 #include <type_traits>
 #include <utility>
 
@@ -400,8 +402,8 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
                 if (p.c_f32) {
                     *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
                 } else {
-                    const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
-                    const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
+                    const uint32_t lo16 = f32x2_to_bf16x2_rne(v[0], v[1]);
+                    const uint32_t hi16 = f32x2_to_bf16x2_rne(v[2], v[3]);
                     *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
                 }
             }
@@ -637,8 +639,8 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         if (p.c_f32) {
             *reinterpret_cast<float4 *>(p.c + elem * 4) = make_float4(v[0], v[1], v[2], v[3]);
         } else {
-            const uint32_t lo16 = f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
-            const uint32_t hi16 = f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
+            const uint32_t lo16 = f32x2_to_bf16x2_rne(v[0], v[1]);
+            const uint32_t hi16 = f32x2_to_bf16x2_rne(v[2], v[3]);
             *reinterpret_cast<uint2 *>(p.c + elem * 2) = make_uint2(lo16, hi16);
         }
     };
@@ -769,6 +771,8 @@ struct Scratch { void *ptr = nullptr; size_t bytes = 0; };
 static Scratch g_slots[64];
 
 static int own_slots(size_t bytes, void **slots) {
+    static std::mutex guard;                     // host threads may call in at the same time
+    std::lock_guard<std::mutex> lock(guard);
     int dev = 0;
     if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
     if (dev < 0 || dev >= 64) return fail(TTMI_ERR_UNSUPPORTED, "device index %d out of range", dev);

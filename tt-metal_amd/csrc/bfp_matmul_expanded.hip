@@ -15,6 +15,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "bfp_dequant.h"
 #include "ttmi_internal.h"
 
@@ -244,6 +246,8 @@ struct Expanded { void *ptr = nullptr; size_t bytes = 0; };
 static Expanded g_expanded[64];
 
 static int own_expanded(size_t bytes, void **out) {
+    static std::mutex guard;                     // host threads may call in at the same time
+    std::lock_guard<std::mutex> lock(guard);
     int dev = 0;
     if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
     if (dev < 0 || dev >= 64) return fail(TTMI_ERR_UNSUPPORTED, "device index %d out of range", dev);

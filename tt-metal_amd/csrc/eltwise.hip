@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(const uint16_t *a, const u
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const float b0 = (BINARY && b) ? bf16_lo(vb[j]) : scalar, b1 = (BINARY && b) ? bf16_hi(vb[j]) : scalar;
-            out[j] = f32_to_bf16_rne(eltwise_apply<OP>(bf16_lo(va[j]), b0)) | ((uint32_t)f32_to_bf16_rne(eltwise_apply<OP>(bf16_hi(va[j]), b1)) << 16);
+            out[j] = f32x2_to_bf16x2_rne(eltwise_apply<OP>(bf16_lo(va[j]), b0), eltwise_apply<OP>(bf16_hi(va[j]), b1));
         }
         reinterpret_cast<u32x4 *>(c)[i] = out;
     }
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(const uint16_t *a, const u
     if (tail < count) {
         const float x = __uint_as_float((uint32_t)a[tail] << 16);
         const float y = (BINARY && b) ? __uint_as_float((uint32_t)b[tail] << 16) : scalar;
-        c[tail] = f32_to_bf16_rne(eltwise_apply<OP>(x, y));
+        c[tail] = (uint16_t)f32x2_to_bf16x2_rne(eltwise_apply<OP>(x, y), 0.f);
     }
 }
 
