@@ -87,3 +87,15 @@ def test_a_listing_without_the_kernel_or_without_its_loads_fails(tmp_path):
     f.write_text("_Z5otherv:\n\ts_endpgm\n.Lfunc_end0:\n")
     assert check_isa.check(str(f)) == 1
     assert run(tmp_path, "\tv_add_u32_e32 v1, v2, v3\n") == 1
+
+
+def test_inline_lds_reads_are_in_flight_until_lgkmcnt_zero(tmp_path, capsys):
+    ring = asm("global_load_dwordx4 v[8:11], v[0:1], off") + "\ts_waitcnt vmcnt(0)\n"   # the kernel must have ring loads
+    good = ring + asm("ds_read2_b32 v[40:41], v5 offset0:0 offset1:4", "s_waitcnt lgkmcnt(0)") + "\tv_add_u32_e32 v42, v40, v41\n"
+    assert run(tmp_path, good) == 0
+    bad = ring + asm("ds_read2_b32 v[40:41], v5 offset0:0 offset1:4") + "\tv_mov_b32_e32 v50, v41\n" + asm("s_waitcnt lgkmcnt(0)")
+    assert run(tmp_path, bad) == 1
+    assert "v_mov_b32_e32 v50, v41" in capsys.readouterr().err
+    # the compiler's own combined wait releases them as well
+    also_good = ring + asm("ds_read_b64 v[40:41], v5 offset:32") + "\ts_waitcnt vmcnt(0) lgkmcnt(0)\n\tv_add_u32_e32 v42, v40, v41\n"
+    assert run(tmp_path, also_good) == 0

@@ -11,6 +11,8 @@ builds the control-flow graph of each streaming kernel (64- and 128-column) and 
   slot loads   (inline global_load_dwordx4 ... sc1: partial sums of other workgroups) are in flight until the next
                `s_waitcnt vmcnt(0)`
   any `s_waitcnt vmcnt(0)` ends every flight (the kernel drains the ring that way when its k range is done)
+  LDS reads    (inline ds_read*: staged tiles, read behind the compiler's back for the same reason) are in flight until
+               the next `s_waitcnt` with lgkmcnt(0), the kernel's own or the compiler's
 
 and fails the build if any compiler-generated instruction mentions a register while it is in flight, or if a register is
 still in flight when the kernel ends.
@@ -111,12 +113,16 @@ def _check_kernel(name, body, problems):
         problems.append(f"{name}: no hand-written activation loads found (has the kernel changed?)")
 
     def run(block, state, report):
-        ring, slot = set(state[0]), set(state[1])
+        ring, slot, lds = set(state[0]), set(state[1]), set(state[2])
         for text, asm in block["instrs"]:
+            if text.startswith("s_waitcnt") and "lgkmcnt(0)" in text:           # every LDS read has returned
+                lds.clear()
             if asm:
                 if text.startswith("global_load_dwordx4"):
                     dest = _regs(text.split(",")[0])
                     (slot if "sc1" in text else ring).update(dest)
+                elif text.startswith("ds_read"):
+                    lds.update(_regs(text.split(",")[0]))
                 elif text.startswith("v_mov_b32"):
                     ring -= _regs(text.split(",")[-1])
                 elif text.startswith("s_waitcnt vmcnt(0)"):
@@ -128,14 +134,14 @@ def _check_kernel(name, body, problems):
                 slot.clear()
                 continue
             if report is not None:
-                hit = _regs(text) & (ring | slot)
+                hit = _regs(text) & (ring | slot | lds)
                 if hit:
                     report.append(f"{name}: compiler instruction touches registers {sorted(hit)} while a hand-scheduled load into them is in flight: {text}")
-            if text.startswith("s_endpgm") and report is not None and (ring or slot):
-                report.append(f"{name}: registers {sorted(ring | slot)} still have a load in flight at s_endpgm")
-        return frozenset(ring), frozenset(slot)
+            if text.startswith("s_endpgm") and report is not None and (ring or slot or lds):
+                report.append(f"{name}: registers {sorted(ring | slot | lds)} still have a load in flight at s_endpgm")
+        return frozenset(ring), frozenset(slot), frozenset(lds)
 
-    empty = (frozenset(), frozenset())
+    empty = (frozenset(), frozenset(), frozenset())
     state_in = [None] * len(blocks)
     state_in[0] = empty
     work = [0]
@@ -143,7 +149,7 @@ def _check_kernel(name, body, problems):
         i = work.pop()
         out = run(blocks[i], state_in[i], None)
         for j in succs[i]:
-            merged = out if state_in[j] is None else (state_in[j][0] | out[0], state_in[j][1] | out[1])
+            merged = out if state_in[j] is None else tuple(a | b for a, b in zip(state_in[j], out))
             if merged != state_in[j]:
                 state_in[j] = merged
                 work.append(j)
