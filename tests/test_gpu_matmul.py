@@ -245,6 +245,24 @@ def test_decode_gemm_in_a_hip_graph(oracle):
         assert torch.equal(other.view(torch.int16), eager.view(torch.int16))
 
 
+@pytest.mark.parametrize("kernel", ["stream", "wide"])
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_row_exponents_over_the_whole_range(oracle, kernel, fmt, monkeypatch):
+    """Weight rows scaled by 2^s, s in [-100, 100], against activation columns scaled by 2^-s: every shared exponent from
+    about 20 to 230 occurs, the products stay of order one, and the result must not care (scales are exact powers of two)."""
+    monkeypatch.setenv("TTMI_MATMUL_KERNEL", kernel)
+    rng = np.random.default_rng(97)
+    m, k, n = 32, 512, 256
+    shift = rng.integers(-100, 101, size=k)
+    a = workloads.bf16_bits_to_f32(workloads.activations_bf16(m, k, seed=98)) * np.exp2(-shift)[None, :].astype(np.float32)
+    w = workloads.weights_f32(k, n, seed=99) * np.exp2(shift)[:, None].astype(np.float32)
+    a_bits = workloads.f32_to_bf16_bits_rne(a.astype(np.float32))
+    assert np.array_equal(workloads.bf16_bits_to_f32(a_bits), a.astype(np.float32))          # still exact in bf16
+    words, w_unpacked = pack_weights(oracle, w.astype(np.float32), fmt)
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n, out_dtype=torch.float32)
+    check_against_reference(c.cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k, bf16_out=False)
+
+
 def test_decode_gemms_on_two_streams_at_once(oracle):
     """Two decode GEMMs, each with a workspace of its own, queued on two streams without waiting for each other: neither
     grid is resident as a whole while the other runs, and the hand-over of partial sums must neither stall nor mix.  Every
