@@ -259,14 +259,29 @@ __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__
         else if (lane_bytes == 4) lo = reinterpret_cast<const uint32_t *>(row)[at.q];
         else { const uint2 v = reinterpret_cast<const uint2 *>(row)[at.q]; lo = v.x; hi = v.y; }
         uint32_t bits[EPL];
+        // Where the result is an ordinary float, i.e. W <= E < 248, the unpacker's normalisation (count leading zeros, shift,
+        // assemble) is the float arithmetic mantissa * 2^(E - 126 - W), exact because the mantissa has at most 7 bits:
+        // convert, multiply by a power of two, put the sign on.  Rows outside that range (non-zero values below 2^-120, where
+        // the reference's exponent subtraction wraps, or near overflow) take the integer route, a wavefront at a time.
+        // (a row of zeros, E = 0 with no mantissa bit set, is ordinary: it comes out as signed zeros either way)
+        constexpr uint32_t all_mantissas = W == 7 ? 0x7f7f7f7fu : 0x77777777u;
+        const bool tiny = shared < (uint32_t)W;
+        const bool odd_rows = __ballot((tiny && ((lo | hi) & all_mantissas) != 0) || shared >= 248u) != 0;
+        const float two_to = tiny ? 0.f : __uint_as_float((shared - (uint32_t)W + 1u) << 23);
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
             const int sh = (W + 1) * e;
-            const uint32_t code = (sh < 32 ? (lo >> sh) : (hi >> (sh - 32))) & ((2u << W) - 1u);
-            bits[e] = from_code<W>(code, shared);
-            // to_torch runs unpack -> untilize -> pack -> unpack: a sign-only value (code 0x80 / 0x8, which no
-            // packer writes) is packed to code 0 on the way and comes out as +0.0f
-            if (MODE == SRC_TENSOR && (bits[e] & 0x7fffffffu) == 0) bits[e] = 0;
+            const uint32_t field = sh < 32 ? (lo >> sh) : (hi >> (sh - 32));            // the code in its low W + 1 bits
+            if (!odd_rows) {
+                const float magnitude = (float)(field & ((1u << W) - 1u)) * two_to;
+                bits[e] = __float_as_uint(magnitude) | ((field << (31 - W)) & 0x80000000u);
+                // to_torch runs unpack -> untilize -> pack -> unpack: a sign-only value (code 0x80 / 0x8, which no
+                // packer writes) is packed to code 0 on the way and comes out as +0.0f; -0 + 0 is +0, all else stays
+                if (MODE == SRC_TENSOR) bits[e] = __float_as_uint(__uint_as_float(bits[e]) + 0.0f);
+            } else {
+                bits[e] = from_code<W>(field & ((2u << W) - 1u), shared);
+                if (MODE == SRC_TENSOR && (bits[e] & 0x7fffffffu) == 0) bits[e] = 0;
+            }
         }
         uint4 v;
         if (ELEM == 4) v = make_uint4(bits[0], bits[1], bits[2], bits[3]);
