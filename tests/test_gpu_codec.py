@@ -60,6 +60,40 @@ def test_from_torch_and_to_torch_paths_bit_exact(oracle, fmt, shape):
         assert np.array_equal(back16.view(torch.int16).cpu().numpy().view(np.uint16), (want_back.view(np.uint32) >> 16).astype(np.uint16))
 
 
+def rounding_boundaries(fmt, shape, seed, exponents):
+    """Face rows whose shared exponent is one of `exponents` and whose elements sit on and next to the packer's rounding
+    boundaries: t = m + d, d in {0, 1/2 - 2^-16, 1/2, 1/2 + 2^-16, 1 - 2^-16}, m = 0 .. 2^W, in units of the row's code step
+    2^(E - 126 - W); the first element of every row is the largest code, which pins E.  All values are exact in fp32."""
+    w = 7 if fmt == BFP8 else 3
+    rng = np.random.default_rng(seed)
+    n = int(np.prod(shape))
+    rows = -(-n // 16)
+    e = rng.choice(np.asarray(exponents), size=rows)
+    m = rng.integers(0, (1 << w) + 1, size=(rows, 16)).astype(np.float64)
+    d = rng.choice(np.array([0.0, 0.5 - 2.0 ** -16, 0.5, 0.5 + 2.0 ** -16, 1.0 - 2.0 ** -16]), size=(rows, 16))
+    t = np.minimum(m + d, float((1 << w)) - 2.0 ** -16)                 # stay inside the row's binade
+    t[:, 0] = float((1 << w) - 1)
+    sign = rng.choice(np.array([-1.0, 1.0]), size=(rows, 16))
+    x = sign * t * np.exp2(e.astype(np.float64) - 126 - w)[:, None]
+    x32 = x.astype(np.float32)
+    assert np.array_equal(x32.astype(np.float64), x)
+    return x32.reshape(-1)[:n].reshape(shape)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("exponents", [(32, 33, 100, 127, 128, 200, 254), (31, 32, 127), (8, 20, 31, 40)])
+def test_rounding_boundaries_bit_exact(oracle, fmt, exponents):
+    """Ties, near-ties and code saturation in rows of every exponent range: rows the kernels take the float way (32 <= E <
+    255), rows they take the integer way, and tensors where both kinds of wavefront occur."""
+    shape = (1, 2, 64, 160)                                  # width 160: face rows are contiguous runs of 16 columns
+    x = rounding_boundaries(fmt, shape, 24, exponents)
+    want = oracle.from_torch_bfp_tiles(fmt, x)
+    got = capi.pack_tensor(fmt, dev(x))
+    assert np.array_equal(words_np(got), want)
+    back = capi.unpack_tensor(fmt, got, shape)
+    assert np.array_equal(back.cpu().numpy().view(np.uint32), oracle.to_torch_bfp_tiles(fmt, want, shape).view(np.uint32))
+
+
 @pytest.mark.parametrize("fmt", [BFP8, BFP4])
 @pytest.mark.parametrize("shape", [(1, 1, 64, 96), (2, 1, 5, 40), (1, 1, 32, 24)])
 def test_bf16_source_bit_exact(oracle, fmt, shape):
