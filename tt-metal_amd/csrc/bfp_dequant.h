@@ -88,6 +88,38 @@ __device__ __forceinline__ bf16x8 weights_operand8(const uint32_t (&words)[8], c
     return __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
 }
 
+// BFLOAT4_B, four operands from 8 mantissa words of 8 k rows (lane uses the half of each word that q selects): a code is
+// sign + a 3-bit integer, which fp8 (e4m3) holds exactly, and gfx950 converts two fp8 bytes to two bf16 times a power of two
+// in one instruction (v_cvt_scalef32_pk_bf16_fp8: the scale is the exponent of a float, i.e. exactly the row scale used
+// here; checked on the hardware for every code and exponent).  Per row: spread the nibbles, look the magnitudes up in a
+// byte table (v_perm_b32), put the signs on top, two conversions; per pair of rows four v_perm_b32 bring (row, row + 1) of a
+// column together.  About 3 instructions per weight instead of 5.5 for convert-and-scale; the values are the same except in
+// rows with E = 0, which contribute their mantissa times 2^-129 instead of nothing.
+__device__ __forceinline__ void bfp4_operands(const uint32_t (&words)[8], int q, const float (&scale)[8], bf16x8 (&bop)[4]) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    uint32_t lo[8], hi[8];         // (columns 0, 1) and (columns 2, 3) of row jj as bf16 pairs
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+        uint32_t v = (words[jj] >> (16 * (q & 1))) & 0xffffu;
+        v = (v | (v << 8)) & 0x00ff00ffu;
+        v = (v | (v << 4)) & 0x0f0f0f0fu;                                   // one code per byte
+        // e4m3 bytes of 0..7: 00 38 40 44 48 4A 4C 4E
+        const uint32_t fp8 = ((v << 4) & 0x80808080u) | __builtin_amdgcn_perm(0x4E4C4A48u, 0x44403800u, v & 0x07070707u);
+        lo[jj] = __builtin_bit_cast(uint32_t, (bf16x2_t)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(fp8, scale[jj], false));
+        hi[jj] = __builtin_bit_cast(uint32_t, (bf16x2_t)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(fp8, scale[jj], true));
+    }
+    uint32_t packed[4][4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        packed[0][p] = __builtin_amdgcn_perm(lo[2 * p + 1], lo[2 * p], 0x05040100u);
+        packed[1][p] = __builtin_amdgcn_perm(lo[2 * p + 1], lo[2 * p], 0x07060302u);
+        packed[2][p] = __builtin_amdgcn_perm(hi[2 * p + 1], hi[2 * p], 0x05040100u);
+        packed[3][p] = __builtin_amdgcn_perm(hi[2 * p + 1], hi[2 * p], 0x07060302u);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bop[j] = __builtin_bit_cast(bf16x8, make_uint4(packed[j][0], packed[j][1], packed[j][2], packed[j][3]));
+}
+
 // Fills `chunk_of[l]` with the global chunk (16 bytes, counted from the start of a 2-tile run) that lands in this
 // lane's slot of direct-to-LDS load l, for the stage layout described at Wfmt.
 template <int W> __device__ __forceinline__ void stage_chunks(int lane, uint32_t (&chunk_of)[Wfmt<W>::loads]) {
@@ -143,23 +175,16 @@ __device__ __forceinline__ void staged_operands(uint32_t exp_at, uint32_t mant_a
     float scale[8];
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(e[jj] << 23);
+    if constexpr (W == 3) {
+        bfp4_operands(words, q, scale, bop);
+    } else {
 #pragma unroll
-    for (int jj = 0; jj < 8; ++jj) {
-        if (W == 7) {
-            mags[jj] = words[jj] & 0x7f7f7f7fu;
-        } else {
-            // four 4-bit codes -> one code per byte; sign bit moved from bit 3 to bit 7 of its byte
-            uint32_t v = (words[jj] >> (16 * (q & 1))) & 0xffffu;
-            v = (v | (v << 8)) & 0x00ff00ffu;
-            v = (v | (v << 4)) & 0x0f0f0f0fu;
-            words[jj] = v << 4;
-            mags[jj] = v & 0x07070707u;
-        }
+        for (int jj = 0; jj < 8; ++jj) mags[jj] = words[jj] & 0x7f7f7f7fu;
+        bop[0] = weights_operand8<0>(words, mags, scale);
+        bop[1] = weights_operand8<1>(words, mags, scale);
+        bop[2] = weights_operand8<2>(words, mags, scale);
+        bop[3] = weights_operand8<3>(words, mags, scale);
     }
-    bop[0] = weights_operand8<0>(words, mags, scale);
-    bop[1] = weights_operand8<1>(words, mags, scale);
-    bop[2] = weights_operand8<2>(words, mags, scale);
-    bop[3] = weights_operand8<3>(words, mags, scale);
 }
 
 // The same in two steps, for kernels that read several slabs before they wait: what one lane reads from LDS for 8 k rows
@@ -182,41 +207,14 @@ __device__ __forceinline__ void wait_slabs(SlabRaw &a, SlabRaw &b) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.e01), "+v"(a.w01), "+v"(a.w23), "+v"(a.w45), "+v"(a.w67),
                                           "+v"(b.e01), "+v"(b.w01), "+v"(b.w23), "+v"(b.w45), "+v"(b.w67)::"memory");
 }
-// ... and expanded into the four B operands (byte j of every word = operand j, as above).
-// BFLOAT4_B takes a shorter way: a code is sign + a 3-bit integer, which fp8 (e4m3) holds exactly, and gfx950 converts two
-// fp8 bytes to two bf16 times a power of two in one instruction (v_cvt_scalef32_pk_bf16_fp8: the scale is the exponent of
-// a float, i.e. exactly the row scale used here; checked on the hardware for every code and exponent).  Per row: spread
-// the nibbles, look the magnitudes up in a byte table (v_perm_b32), put the signs on top, two conversions; per pair of rows
-// four v_perm_b32 bring (row, row + 1) of a column together.  About 3 instructions per weight instead of 5.5; the values
-// are the same except in rows with E = 0, which now contribute their mantissa times 2^-129 instead of nothing.
+// ... and expanded into the four B operands (byte j of every word = operand j, as above; BFLOAT4_B through bfp4_operands).
 template <int W> __device__ __forceinline__ void slab_expand(const SlabRaw &r, int q, bf16x8 (&bop)[4]) {
-    uint32_t words[8] = {r.w01[0], r.w01[1], r.w23[0], r.w23[1], r.w45[0], r.w45[1], r.w67[0], r.w67[1]};
+    const uint32_t words[8] = {r.w01[0], r.w01[1], r.w23[0], r.w23[1], r.w45[0], r.w45[1], r.w67[0], r.w67[1]};
     float scale[8];
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(((r.e01[jj >> 2] >> (8 * (jj & 3))) & 0xffu) << 23);
     if constexpr (W == 3) {
-        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-        uint32_t lo[8], hi[8];         // (columns 0, 1) and (columns 2, 3) of row jj as bf16 pairs
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-            uint32_t v = (words[jj] >> (16 * (q & 1))) & 0xffffu;
-            v = (v | (v << 8)) & 0x00ff00ffu;
-            v = (v | (v << 4)) & 0x0f0f0f0fu;                                   // one code per byte
-            // e4m3 bytes of 0..7: 00 38 40 44 48 4A 4C 4E
-            const uint32_t fp8 = ((v << 4) & 0x80808080u) | __builtin_amdgcn_perm(0x4E4C4A48u, 0x44403800u, v & 0x07070707u);
-            lo[jj] = __builtin_bit_cast(uint32_t, (bf16x2_t)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(fp8, scale[jj], false));
-            hi[jj] = __builtin_bit_cast(uint32_t, (bf16x2_t)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(fp8, scale[jj], true));
-        }
-        uint32_t packed[4][4];
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            packed[0][p] = __builtin_amdgcn_perm(lo[2 * p + 1], lo[2 * p], 0x05040100u);
-            packed[1][p] = __builtin_amdgcn_perm(lo[2 * p + 1], lo[2 * p], 0x07060302u);
-            packed[2][p] = __builtin_amdgcn_perm(hi[2 * p + 1], hi[2 * p], 0x05040100u);
-            packed[3][p] = __builtin_amdgcn_perm(hi[2 * p + 1], hi[2 * p], 0x07060302u);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) bop[j] = __builtin_bit_cast(bf16x8, make_uint4(packed[j][0], packed[j][1], packed[j][2], packed[j][3]));
+        bfp4_operands(words, q, scale, bop);
     } else {
         uint32_t mags[8];
 #pragma unroll
