@@ -291,6 +291,33 @@ def test_decode_gemms_on_two_streams_at_once(oracle):
             assert torch.equal(out.view(1, j["m"], j["n"]).view(torch.int16), j["alone"].view(torch.int16)), (j["n"], rep)
 
 
+def test_full_size_decode_gemms_on_three_streams():
+    """The same at full size: together the three grids are more than twice what the GPU holds at one time, so workgroups
+    of every launch wait for slots while others of the same launch already poll for their partial sums.  That costs time
+    (whoever waits, waits for lower workgroup indices only, so it ends), never results."""
+    L = capi.lib()
+    jobs = []
+    for m, k, n, fmt, seed in [(32, 4544, 18176, BFP8, 1), (32, 18176, 4544, BFP8, 2), (32, 4096, 14336, BFP4, 3)]:
+        gen = torch.Generator(device="cuda").manual_seed(seed)
+        a = capi.tilize(torch.randn(m, k, device="cuda", generator=gen).bfloat16())
+        w = capi.pack_tensor(fmt, torch.randn(k, n, device="cuda", generator=gen) * 0.02)
+        need = L.ttmi_matmul_bfp_workspace_bytes(1, m, k, n, fmt)
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        alone = capi.matmul_bfp(a, capi.TILE, w, fmt, 1, 1, m, k, n, c_layout=capi.TILE).clone()
+        jobs.append(dict(m=m, k=k, n=n, fmt=fmt, a=a, w=w, need=need, ws=ws, alone=alone, stream=torch.cuda.Stream(),
+                         outs=[torch.empty(m * n, dtype=torch.bfloat16, device="cuda") for _ in range(8)]))
+    torch.cuda.synchronize()
+    for rep in range(8):
+        for j in jobs:
+            capi.check(L.ttmi_matmul_bfp(j["a"].data_ptr(), capi.TILE, j["w"].data_ptr(), j["fmt"], 1, 1, j["m"], j["k"], j["n"], None,
+                                         capi.ACT_NONE, j["outs"][rep].data_ptr(), capi.TILE, capi.BFLOAT16, j["ws"].data_ptr(), j["need"],
+                                         j["stream"].cuda_stream))
+    torch.cuda.synchronize()
+    for j in jobs:
+        for rep, out in enumerate(j["outs"]):
+            assert torch.equal(out.view(torch.int16), j["alone"].reshape(-1).view(torch.int16)), (j["n"], rep)
+
+
 @pytest.mark.parametrize("name,m,k,n,fmt,batch", workloads.DECODE_FALCON + workloads.DECODE_MISTRAL)
 def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch):
     a_bits = workloads.activations_bf16(m, k, seed=80)
