@@ -245,8 +245,8 @@ struct StoreTarget {
     int c_tiled, c_f32;
 };
 
-template <int ACT, typename Acc>
-__device__ __forceinline__ void store_wave_part(const Acc (&acc)[4][2], const StoreTarget &o, uint8_t *lds_wave, int lane) {
+template <int ACT, typename Acc, int RB>
+__device__ __forceinline__ void store_wave_part(const Acc (&acc)[RB][2], const StoreTarget &o, uint8_t *lds_wave, int lane) {
     const int c = lane & 31, kh = lane >> 5;
     const int c16 = c & 15, half = c >> 4;
     const int t = c16 >> 3, fc = (c16 >> 2) & 1, q = c16 & 3;
@@ -261,7 +261,7 @@ __device__ __forceinline__ void store_wave_part(const Acc (&acc)[4][2], const St
     }
     const uint32_t mt = (o.m + 31) / 32;
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb) {
+    for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const uint32_t r32 = (i >> 2) * 8 + kh * 4 + (i & 3);
@@ -284,7 +284,7 @@ __device__ __forceinline__ void store_wave_part(const Acc (&acc)[4][2], const St
     if (o.c_f32) return;
     if (o.c_tiled) {
 #pragma unroll
-        for (int rb = 0; rb < 4; ++rb) {
+        for (int rb = 0; rb < RB; ++rb) {
             const uint32_t row = o.row0 + rb * 32;
             if (row >= o.m) break;
             uint8_t *dst = o.c + ((o.slice * mt + (row >> 5)) * o.nt + o.nt0) * 2048;
@@ -296,7 +296,7 @@ __device__ __forceinline__ void store_wave_part(const Acc (&acc)[4][2], const St
     } else {
         const uint32_t chunk = lane & 7;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
+        for (int j = 0; j < 4 * RB; ++j) {
             const uint32_t r = j * 8 + (lane >> 3), row = o.row0 + r;
             if (row < o.m && chunk < tiles * 4)
                 *reinterpret_cast<u32x4 *>(o.c + ((o.slice * o.m + row) * o.n + o.nt0 * 32) * 2 + chunk * 16) =

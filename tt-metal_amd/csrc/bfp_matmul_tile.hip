@@ -2,9 +2,9 @@
 //
 // Two kernels share the staging and the weight expansion:
 //   matmul_tile_kernel   4 wavefronts, (32*MB)-row x 256-column block of C; used with MB = 4 (128 rows) when 256-row
-//                        blocks would leave CUs idle or M is not a multiple of 256
-//   matmul_tile8_kernel  8 wavefronts, 256 x 256 block; the two wavefronts of a column group split the weight
-//                        expansion and exchange operands through LDS (described at the kernel)
+//                        blocks would leave CUs idle or M is not a multiple of 256, for long k ranges
+//   matmul_tile8_kernel  8 wavefronts, 256 x 256 block (or 128 x 256, for short k ranges); the two wavefronts of a
+//                        column group split the weight expansion and exchange operands through LDS (described at the kernel)
 //   staging    the k loop advances one packed tile row (32 rows of W) at a time through a ring of LDS stages filled by
 //              direct global->LDS loads
 //   math       v_mfma_f32_32x32x16_bf16, fp32 accumulation
@@ -264,27 +264,27 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// 256 x 256 block with EIGHT wavefronts (two per SIMD).  A single wavefront per SIMD cannot issue the weight
+// 256 x 256 block (MB = 4; MB = 2: 128 x 256) with EIGHT wavefronts (two per SIMD).  A single wavefront per SIMD cannot issue the weight
 // expansion and the MFMAs of a 256-row block fast enough; two can, if the expansion is not done twice.  Wavefront
-// (wc = w % 4, wr = w / 4) owns rows 128*wr .. +127 and columns 64*wc .. +63 of the block.  The two wavefronts of a
+// (wc = w % 4, wr = w / 4) owns rows 32*MB*wr .. and columns 64*wc .. +63 of the block.  The two wavefronts of a
 // column group share the work of expanding its weights: wr expands slab wr (k rows 16*wr .. +15) of the NEXT k step
 // into bf16 B operands and leaves them in LDS, exactly as its lanes would hold them in registers; after the step's
 // barrier both read all four operands of the group (2 slabs x 2 operands, one ds_read_b128 each).
-//   LDS   ring of TILE_STAGES stages [A: 256 rows x 64 B][packed W: 4 column groups], then two operand buffers
+//   LDS   ring of TILE_STAGES stages [A: 64*MB rows x 64 B][packed W: 4 column groups], then two operand buffers
 //         [column group][slab][operand][lane] x 16 B (step parity)
 //   step  wait for the own direct-to-LDS loads of step i+1, barrier, request step i+3, then interleaved:
-//         (a) operands of step i and A from LDS -> 16 MFMAs (32x32x16), (b) expand slab wr of step i+1 -> LDS
-template <int W, int ACT>
+//         (a) operands of step i and A from LDS -> 4*MB MFMAs (32x32x16), (b) expand slab wr of step i+1 -> LDS
+template <int W, int ACT, int MB>                          // MB = 32-row blocks per wavefront: 4 (256-row block) or 2 (128-row block)
 __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
     using F = Wfmt<W>;
-    constexpr int MB = 4;                                  // 32-row blocks per wavefront
-    constexpr int A_BYTES = 256 * 64;
+    constexpr int BM = 64 * MB;                            // rows of the block
+    constexpr int A_BYTES = BM * 64;
     constexpr int STAGE_BYTES = A_BYTES + 4 * F::stage_bytes;
     constexpr int OPS_BYTES = 4 * 2 * 2 * 64 * 16;         // one operand buffer
     constexpr int OPS_BASE = TILE_STAGES * STAGE_BYTES;
     constexpr int NLOAD = F::loads;
     constexpr int W_LOADS0 = (NLOAD + 1) / 2, W_LOADS1 = NLOAD - W_LOADS0;   // packed-weight loads issued by wr = 0 / wr = 1
-    constexpr int A_LOADS = 2;                             // 16 loads of 16 rows each over 8 wavefronts
+    constexpr int A_LOADS = MB / 2;                        // BM / 16 loads of 16 rows each over 8 wavefronts
     __shared__ __attribute__((aligned(1024))) uint8_t lds[OPS_BASE + 2 * OPS_BYTES];
 
     const int lane = threadIdx.x & 63;
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
     const uint32_t tm = idx % p.tiles_m; idx /= p.tiles_m;
     const uint32_t tn = idx % p.tiles_n;
     const uint32_t bb = idx / p.tiles_n;
-    const uint32_t m0 = tm * 256;
+    const uint32_t m0 = tm * BM;
     const uint32_t nt0 = tn * (TILE_COLS / 32) + wc * 2;               // first packed tile column of this column group
     const uint32_t n_valid = nt0 >= p.nt ? 0u : min(2u, p.nt - nt0);
 
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
     uint32_t a_step;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
-        const uint32_t row_in_block = wave * 32 + i * 16 + (lane >> 2);
+        const uint32_t row_in_block = wave * (BM / 8) + i * 16 + (lane >> 2);
         const uint32_t row = min(m0 + row_in_block, p.m - 1);
         const uint32_t kq = (lane & 3) ^ ((lane >> 4) & 3);              // XOR swizzle of the row's four 16-byte chunks
         if (p.a_tiled) a_off[i] = (row >> 5) * p.kt * 2048 + (((row >> 4) & 1) * 2 + (kq >> 1)) * 512 + (row & 15) * 32 + (kq & 1) * 16;
@@ -331,7 +331,7 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(a_base + a_off[i]),
-                                             (__attribute__((address_space(3))) void *)(base + (wave * 32 + i * 16) * 64), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void *)(base + (wave * (BM / 8) + i * 16) * 64), 16, 0, 0);
         if (wr == 0) {
 #pragma unroll
             for (int l = 0; l < W_LOADS0; ++l)
@@ -353,9 +353,9 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
                               (kh * 8) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);
     const uint32_t ops_write_off = OPS_BASE + ((wc * 2 + wr) * 2) * 1024 + lane * 16;         // + parity * OPS_BYTES, + operand * 1024
     const uint32_t ops_partner_off = OPS_BASE + ((wc * 2 + (1 - wr)) * 2) * 1024 + lane * 16;  // the other slab's operands
-    // A operand of MFMA (row block rb, slab s): row wr*128 + rb*32 + c, 16-byte chunk 2s + kh of that row (+ rb * 2048)
-    const uint32_t a_own_off = (wr * 128 + c) * 64 + (((2 * wr + kh) ^ ((c >> 2) & 3)) * 16);
-    const uint32_t a_partner_off = (wr * 128 + c) * 64 + (((2 * (1 - wr) + kh) ^ ((c >> 2) & 3)) * 16);
+    // A operand of MFMA (row block rb, slab s): row wr*32*MB + rb*32 + c, 16-byte chunk 2s + kh of that row (+ rb * 2048)
+    const uint32_t a_own_off = (wr * 32 * MB + c) * 64 + (((2 * wr + kh) ^ ((c >> 2) & 3)) * 16);
+    const uint32_t a_partner_off = (wr * 32 * MB + c) * 64 + (((2 * (1 - wr) + kh) ^ ((c >> 2) & 3)) * 16);
 
     f32x16 acc[MB][2];
 #pragma unroll
@@ -445,26 +445,26 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
     while (step + 1 < total) iteration(std::true_type{});
     iteration(std::false_type{});
 
-    // ---- epilogue: acc[rb][cb][i] is row wr*128 + rb*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the group's 64;
-    // the ring and the operand buffers are idle now and become the staging of store_wave_part (16 KB per wavefront)
+    // ---- epilogue: acc[rb][cb][i] is row wr*32*MB + rb*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the group's 64;
+    // the ring and the operand buffers are idle now and become the staging of store_wave_part (4 KB per 32 rows and wavefront)
     wait_vmcnt<0>();
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __builtin_amdgcn_s_barrier();
     StoreTarget o;
     o.c = p.c; o.bias = p.bias; o.m = p.m; o.n = p.n; o.nt = p.nt; o.slice = bb;
-    o.row0 = m0 + wr * 128; o.nt0 = nt0;
+    o.row0 = m0 + wr * 32 * MB; o.nt0 = nt0;
     o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32;
-    static_assert(OPS_BASE + 2 * OPS_BYTES >= 8 * 16384, "staging of the epilogue does not fit into LDS");
-    store_wave_part<ACT>(acc, o, lds + wave * 16384, lane);
+    static_assert(OPS_BASE + 2 * OPS_BYTES >= 8 * MB * 4096, "staging of the epilogue does not fit into LDS");
+    store_wave_part<ACT>(acc, o, lds + wave * (MB * 4096), lane);
 }
 
-template <int W>
+template <int W, int MB>
 static void launch_tile8_act(const TileDev &p, int activation, uint32_t blocks, hipStream_t st) {
     switch (activation) {
-        case TTMI_ACT_RELU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_RELU>), dim3(blocks), dim3(512), 0, st, p); break;
-        case TTMI_ACT_GELU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_GELU>), dim3(blocks), dim3(512), 0, st, p); break;
-        case TTMI_ACT_SILU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_SILU>), dim3(blocks), dim3(512), 0, st, p); break;
-        default: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_NONE>), dim3(blocks), dim3(512), 0, st, p); break;
+        case TTMI_ACT_RELU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_RELU, MB>), dim3(blocks), dim3(512), 0, st, p); break;
+        case TTMI_ACT_GELU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_GELU, MB>), dim3(blocks), dim3(512), 0, st, p); break;
+        case TTMI_ACT_SILU: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_SILU, MB>), dim3(blocks), dim3(512), 0, st, p); break;
+        default: hipLaunchKernelGGL((matmul_tile8_kernel<W, TTMI_ACT_NONE, MB>), dim3(blocks), dim3(512), 0, st, p); break;
     }
 }
 
@@ -489,11 +489,15 @@ int matmul_bfp_tiled(const MatmulArgs &x, hipStream_t st) {
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
     p.kt = x.k / 32; p.nt = x.n / 32;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE; p.c_f32 = x.c_dtype == TTMI_FLOAT32;
-    // 256-row blocks when they fill the chip, 128-row blocks otherwise (fewer idle CUs, half the accumulators)
+    // 256-row blocks when they fill the chip, 128-row blocks otherwise (fewer idle CUs, half the accumulators).
+    // TTMI_MATMUL_BM forces a form: "256", "128" (eight wavefronts) or "4" (128 rows, four wavefronts).
     const uint32_t tiles_n = (x.n + TILE_COLS - 1) / TILE_COLS;
     const uint64_t big = (uint64_t)x.batch * ((x.m + 255) / 256) * tiles_n;
     const char *force_bm = getenv("TTMI_MATMUL_BM");
     const bool use_256 = force_bm ? force_bm[0] == '2' : (x.m > 128 && big >= 256 && x.m % 256 == 0);
+    // 128-row blocks: eight wavefronts (each 64 rows) measure 6 % better than four for short k ranges (batched bmm,
+    // k = 1024: epilogue and start-up are spread over twice as many wavefronts), four 1-2 % better for k = 4096
+    const bool four_waves = force_bm ? force_bm[0] == '4' : x.k > 2048;
     const uint32_t bm = use_256 ? 256 : 128;
     p.tiles_m = (x.m + bm - 1) / bm; p.tiles_n = tiles_n;
     const uint64_t blocks = (uint64_t)x.batch * p.tiles_m * p.tiles_n;
@@ -503,11 +507,13 @@ int matmul_bfp_tiled(const MatmulArgs &x, hipStream_t st) {
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
     if (x.b_fmt == TTMI_BFLOAT8_B) {
-        if (use_256) launch_tile8_act<7>(p, x.activation, (uint32_t)blocks, st);
-        else launch_tile_act<7, 4>(p, x.activation, (uint32_t)blocks, st);
+        if (use_256) launch_tile8_act<7, 4>(p, x.activation, (uint32_t)blocks, st);
+        else if (four_waves) launch_tile_act<7, 4>(p, x.activation, (uint32_t)blocks, st);
+        else launch_tile8_act<7, 2>(p, x.activation, (uint32_t)blocks, st);
     } else {
-        if (use_256) launch_tile8_act<3>(p, x.activation, (uint32_t)blocks, st);
-        else launch_tile_act<3, 4>(p, x.activation, (uint32_t)blocks, st);
+        if (use_256) launch_tile8_act<3, 4>(p, x.activation, (uint32_t)blocks, st);
+        else if (four_waves) launch_tile_act<3, 4>(p, x.activation, (uint32_t)blocks, st);
+        else launch_tile8_act<3, 2>(p, x.activation, (uint32_t)blocks, st);
     }
     return check_launch("matmul_tile_kernel");
 }
