@@ -275,7 +275,9 @@ __device__ __forceinline__ void store_wave_part(const Acc (&acc)[RB][2], const S
                 *reinterpret_cast<float2 *>(o.c + elem * 4) = make_float2(v0, v1);
             } else {
                 const uint32_t both = f32x2_to_bf16x2_rne(v0, v1);
-                const uint32_t at = o.c_tiled ? rb * 4096 + t * 2048 + (((r32 >> 4) & 1) * 2 + fc) * 512 + (r32 & 15) * 32 + q * 8 + half * 4
+                // TILE layout: tile t and face column fc move a lane by 2048 and 512 bytes, i.e. onto the same banks; they are
+                // XOR-ed into the two 16-byte-chunk bits that are the same for all lanes (r32 % 4), and out again below
+                const uint32_t at = o.c_tiled ? rb * 4096 + t * 2048 + (((r32 >> 4) & 1) * 2 + fc) * 512 + (((r32 & 15) * 32) ^ (t * 32 + fc * 64)) + q * 8 + half * 4
                                               : (rb * 32 + r32) * 128 + col * 2;
                 *reinterpret_cast<uint32_t *>(lds_wave + at) = both;
             }
@@ -291,7 +293,8 @@ __device__ __forceinline__ void store_wave_part(const Acc (&acc)[RB][2], const S
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 if ((uint32_t)j < tiles * 2)
-                    *reinterpret_cast<u32x4 *>(dst + j * 1024 + lane * 16) = *reinterpret_cast<const u32x4 *>(lds_wave + rb * 4096 + j * 1024 + lane * 16);
+                    *reinterpret_cast<u32x4 *>(dst + j * 1024 + lane * 16) =
+                        *reinterpret_cast<const u32x4 *>(lds_wave + rb * 4096 + j * 1024 + ((lane * 16) ^ ((j >> 1) * 32 + ((lane >> 5) & 1) * 64)));
         }
     } else {
         const uint32_t chunk = lane & 7;
