@@ -160,7 +160,7 @@ def test_caller_workspace(oracle):
         capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP4, 1, 1, m, k, n, workspace=small)
 
 
-@pytest.mark.parametrize("kernel", ["stream", "wide", "tile", "tile256", "tile4waves", "expanded"])
+@pytest.mark.parametrize("kernel", ["stream", "wide", "tile", "tile256", "tile4waves", "tile384", "expanded"])
 @pytest.mark.parametrize("fmt", [BFP8, BFP4])
 @pytest.mark.parametrize("batch,b_batch,m,k,n", [(1, 1, 256, 128, 256), (1, 1, 300, 96, 288), (2, 1, 130, 160, 96), (1, 1, 288, 224, 96),
                                                  (2, 2, 512, 64, 544), (1, 1, 40, 32, 2080),
@@ -174,6 +174,8 @@ def test_every_kernel_on_every_shape(oracle, kernel, fmt, batch, b_batch, m, k, 
         monkeypatch.setenv("TTMI_MATMUL_BM", "256")
     if kernel == "tile4waves":
         monkeypatch.setenv("TTMI_MATMUL_BM", "4")
+    if kernel == "tile384":                                  # 384-row x 64-column blocks, twelve wavefronts
+        monkeypatch.setenv("TTMI_MATMUL_BM", "384")
     a_bits = workloads.activations_bf16(m, k, seed=75, batch=batch)
     w = workloads.weights_f32(k, n, seed=76, batch=b_batch)
     words, w_unpacked = pack_weights(oracle, w, fmt)

@@ -458,6 +458,228 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
     store_wave_part<ACT>(acc, o, lds + wave * (MB * 4096), lane);
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// (32*NW)-row x 64-column block with NW wavefronts, one 32-row band each, for batched GEMMs whose row ranges are short
+// and few (BERT-like bmm: 384 rows per slice): with 128 x 256 blocks such a problem occupies half the CUs with
+// workgroups that expand every weight once per 128 rows.  Here a workgroup owns ALL rows of a slice for one 64-column
+// group, so every weight is expanded once: wavefronts 0..7 each expand a quarter of a slab of the NEXT k step into the
+// operand buffer (one wavefront expanding a whole slab makes the others wait for it at every barrier), and after the
+// step's barrier every wavefront reads the four operands (2 slabs x 2).
+//   A     nobody but its wavefront reads a band of 32 rows, so A goes from memory straight into registers in the layout of
+//         the MFMA's A operand, six k steps ahead (a ring through LDS holds at most two to three steps of 24 KB in flight,
+//         and with 1.5 to 2 us of latency that, not any pipe, set the step time)
+//   LDS   ring of 6 stages [packed W of the group], then two operand buffers [slab][operand][lane] x 16 B (step parity)
+//   step  wait for the own loads of step i+1, barrier, operands of step i from LDS -> 4 MFMAs (32x32x16); wavefronts 0..7
+//         expand their part of step i+1 between the two slabs; request step i+6
+template <int W, int ACT, int NW>
+__global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p) {
+    using F = Wfmt<W>;
+    constexpr int BM = 32 * NW;
+    constexpr int D = 6;                                   // k steps requested ahead (A into registers, packed W into the ring)
+    constexpr int STAGE_BYTES = F::stage_bytes;
+    constexpr int OPS_BYTES = 2 * 2 * 64 * 16;             // one operand buffer
+    constexpr int OPS_BASE = D * STAGE_BYTES;
+    constexpr int LDS_BYTES = OPS_BASE + 2 * OPS_BYTES > NW * 4096 ? OPS_BASE + 2 * OPS_BYTES : NW * 4096;
+    constexpr int NLOAD = F::loads;
+    constexpr int W_LOADS0 = (NLOAD + 1) / 2, W_LOADS1 = NLOAD - W_LOADS0;   // packed-weight loads issued by wavefront 0 / 1
+    constexpr int A_LOADS = 2;                             // one 16-byte load per lane and slab
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 31, kh = lane >> 5;
+    const int c16 = c & 15, half = c >> 4;
+    const int t_of_lane = c16 >> 3, fc = (c16 >> 2) & 1, q = c16 & 3;
+    const uint32_t half_shift = 16 * half;
+
+    // workgroup i runs on XCD i % 8: every XCD gets a contiguous range of blocks, so that the column groups of a slice
+    // (which all read the slice's A) share one L2
+    uint32_t idx = blockIdx.x;
+    if ((gridDim.x & 7u) == 0) idx = (idx & 7u) * (gridDim.x >> 3) + (idx >> 3);
+    const uint32_t tm = idx % p.tiles_m; idx /= p.tiles_m;
+    const uint32_t tn = idx % p.tiles_n;                                 // 64-column group
+    const uint32_t bb = idx / p.tiles_n;
+    const uint32_t m0 = tm * BM;
+    const uint32_t nt0 = tn * 2;                                         // < nt
+    const uint32_t n_valid = min(2u, p.nt - nt0);
+
+    // ---- direct-to-LDS loads of this wavefront ---------------------------------------------------------------
+    uint32_t chunk_of[NLOAD], src_off[NLOAD];
+    stage_chunks<W>(lane, chunk_of);
+    const uint32_t chunks_valid = n_valid * F::chunks;
+#pragma unroll
+    for (int l = 0; l < NLOAD; ++l) src_off[l] = min(chunk_of[l], chunks_valid - 1) * 16;
+    const uint8_t *wptr = p.b + ((uint64_t)(p.b_batch == 1 ? 0 : bb) * p.kt * p.nt + nt0) * F::tile_bytes;
+    const uint64_t w_step = (uint64_t)p.nt * F::tile_bytes;
+    // A: a wavefront is the only reader of its 32 rows, so they go straight into registers in the layout of the MFMA's A
+    // operand: lane (c, kh) holds, for slab s, the 16 bytes of row wave*32 + c at k chunk 2s + kh (in TILE layout the 64
+    // lanes of such a load cover two whole faces)
+    uint32_t a_off[A_LOADS];
+    const uint8_t *a_base;
+    uint32_t a_step;
+    {
+        const uint32_t row = min(m0 + wave * 32 + c, p.m - 1);           // rows past M repeat the last row, never stored
+#pragma unroll
+        for (int sl = 0; sl < A_LOADS; ++sl) {
+            const uint32_t kq = 2 * sl + kh;
+            if (p.a_tiled) a_off[sl] = (row >> 5) * p.kt * 2048 + (((row >> 4) & 1) * 2 + (kq >> 1)) * 512 + (row & 15) * 32 + (kq & 1) * 16;
+            else a_off[sl] = (row * p.k + kq * 8) * 2;
+        }
+    }
+    if (p.a_tiled) { a_base = p.a + (uint64_t)bb * ((p.m + 31) / 32) * p.kt * 2048; a_step = 2048; }
+    else { a_base = p.a + (uint64_t)bb * p.m * p.k * 2; a_step = 64; }
+    bf16x8 a_ring[D][A_LOADS];
+
+    // requests of one k step: slot = step % D names both the registers for A and the ring stage for the packed weights
+    auto fetch = [&](auto slot_c) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_c)::value;
+        uint8_t *base = lds + SLOT * STAGE_BYTES;
+#pragma unroll
+        for (int sl = 0; sl < A_LOADS; ++sl) a_ring[SLOT][sl] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(a_base + a_off[sl]));
+        if (wave == 0) {
+#pragma unroll
+            for (int l = 0; l < W_LOADS0; ++l)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[l]),
+                                                 (__attribute__((address_space(3))) void *)(base + l * 1024), 16, 0, 0);
+        } else if (wave == 1) {
+#pragma unroll
+            for (int l = W_LOADS0; l < NLOAD; ++l)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[l]),
+                                                 (__attribute__((address_space(3))) void *)(base + l * 1024), 16, 0, 0);
+        }
+        a_base += a_step;
+        wptr += w_step;
+    };
+
+    // wavefront e = 0..7 expands a quarter of slab e / 4 (faces h = e / 4): of the 8 k rows 8kh .. that a lane holds of the
+    // slab, rows 2pr and 2pr + 1 (pr = e % 4), i.e. one 32-bit word of each of the slab's two operands
+    const int es = (wave >> 2) & 1, pr = wave & 3;
+    const uint32_t exp_off = F::exp_base + t_of_lane * 64 + fc * 16 + kh * 8 + es * 32 + 2 * pr;
+    const uint32_t mant_off = (es * 4 + t_of_lane * 2 + fc) * F::face_stride + (kh * 8 + 2 * pr) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);
+    const uint32_t ops_write_off = OPS_BASE + (es * 2) * 1024 + lane * 16 + pr * 4;     // + parity * OPS_BYTES, + operand * 1024
+    const uint32_t ops_read_off = OPS_BASE + lane * 16;                             // + parity * OPS_BYTES, + (slab * 2 + operand) * 1024
+    f32x16 acc[1][2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[0][cb][r] = 0.f;
+
+    const uint32_t total = p.kt;
+    uint32_t requested = 0, step = 0;
+    using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>; using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>; using S4 = std::integral_constant<int, 4>; using S5 = std::integral_constant<int, 5>;
+    static_assert(D == 6, "the request and iteration sequences below are written out for six slots");
+    if (requested < total) { fetch(S0{}); ++requested; }
+    if (requested < total) { fetch(S1{}); ++requested; }
+    if (requested < total) { fetch(S2{}); ++requested; }
+    if (requested < total) { fetch(S3{}); ++requested; }
+    if (requested < total) { fetch(S4{}); ++requested; }
+    if (requested < total) { fetch(S5{}); ++requested; }
+
+    // vector-memory operations complete in order and every wavefront issues the same number per step (its two A loads
+    // and its share of the weight loads), so "step `which` has landed" is a bound on the operations still in flight
+    auto wait_for_step = [&](uint32_t which) __attribute__((always_inline)) {
+        const uint32_t ahead = which < requested ? requested - which - 1 : 0;   // steps requested after `which`: 0 .. D - 1
+        auto ladder = [&](auto vm_c) __attribute__((always_inline)) {
+            constexpr int VM = decltype(vm_c)::value;
+            if (ahead >= 5) wait_vmcnt<5 * VM>(); else if (ahead == 4) wait_vmcnt<4 * VM>(); else if (ahead == 3) wait_vmcnt<3 * VM>();
+            else if (ahead == 2) wait_vmcnt<2 * VM>(); else if (ahead == 1) wait_vmcnt<VM>(); else wait_vmcnt<0>();
+        };
+        if (wave == 0) ladder(std::integral_constant<int, A_LOADS + W_LOADS0>{});
+        else if (wave == 1) ladder(std::integral_constant<int, A_LOADS + W_LOADS1>{});
+        else ladder(std::integral_constant<int, A_LOADS>{});
+    };
+    // wavefronts 0..7: expand their two rows of the step in `from_stage` into operand buffer `parity`; the arithmetic is
+    // that of weights_operand8 for one pair of rows
+    auto expand = [&](int from_stage, uint32_t parity) __attribute__((always_inline)) {
+        const uint8_t *stage_at = lds + from_stage * STAGE_BYTES;
+        const float scale0 = __uint_as_float((uint32_t)stage_at[exp_off] << 23), scale1 = __uint_as_float((uint32_t)stage_at[exp_off + 1] << 23);
+        uint32_t word[2] = {*reinterpret_cast<const uint32_t *>(stage_at + mant_off), *reinterpret_cast<const uint32_t *>(stage_at + mant_off + F::row_bytes)};
+        uint32_t mag[2];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            if (W == 7) {
+                word[r] >>= half_shift;
+                mag[r] = word[r] & 0x7f7fu;
+            } else {                                         // four 4-bit codes -> one code per byte, sign to bit 7 of its byte
+                uint32_t v = (word[r] >> (16 * (q & 1))) & 0xffffu;
+                v = (v | (v << 8)) & 0x00ff00ffu;
+                v = ((v | (v << 4)) & 0x0f0f0f0fu) >> half_shift;
+                word[r] = v << 4;
+                mag[r] = v & 0x0707u;
+            }
+        }
+        const uint32_t both0 = __builtin_amdgcn_perm(__float_as_uint(byte_to_float<0>(mag[1]) * scale1),
+                                                     __float_as_uint(byte_to_float<0>(mag[0]) * scale0), 0x07060302u);
+        const uint32_t both1 = __builtin_amdgcn_perm(__float_as_uint(byte_to_float<1>(mag[1]) * scale1), __float_as_uint(byte_to_float<1>(mag[0]) * scale0), 0x07060302u);
+        const uint32_t signs0 = __builtin_amdgcn_perm(word[1], word[0], (4u << 24) | (0x0cu << 16) | (0u << 8) | 0x0cu);
+        const uint32_t signs1 = __builtin_amdgcn_perm(word[1], word[0], (5u << 24) | (0x0cu << 16) | (1u << 8) | 0x0cu);
+        *reinterpret_cast<uint32_t *>(lds + parity * OPS_BYTES + ops_write_off) = (signs0 & 0x80008000u) | both0;
+        *reinterpret_cast<uint32_t *>(lds + parity * OPS_BYTES + ops_write_off + 1024) = (signs1 & 0x80008000u) | both1;
+    };
+
+    // prologue: the operands of step 0
+    wait_for_step(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    if (wave < 8) expand(0, 0);
+
+    // one k step; SLOT = step % D
+    auto iteration = [&](auto slot_c) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_c)::value, NEXT = (SLOT + 1) % D;
+        const bool more = step + 1 < total;
+        const uint32_t parity = step & 1;
+        if (more) wait_for_step(step + 1);
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // our LDS reads and operand writes of the previous step are done
+        __builtin_amdgcn_s_barrier();
+        bf16x8 b[2][2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb)
+                b[s][cb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + parity * OPS_BYTES + ops_read_off + (s * 2 + cb) * 1024));
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SLOT][0], b[0][0], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SLOT][0], b[0][1], acc[0][1], 0, 0, 0);
+        if (more && wave < 8) expand(NEXT, parity ^ 1);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SLOT][1], b[1][0], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SLOT][1], b[1][1], acc[0][1], 0, 0, 0);
+        // this step's registers and ring stage are free (the stage was read before the barrier above): request step + D
+        if (requested < total) { fetch(slot_c); ++requested; }
+        ++step;
+    };
+#pragma unroll 1
+    for (;;) {
+        iteration(S0{}); if (step == total) break;
+        iteration(S1{}); if (step == total) break;
+        iteration(S2{}); if (step == total) break;
+        iteration(S3{}); if (step == total) break;
+        iteration(S4{}); if (step == total) break;
+        iteration(S5{}); if (step == total) break;
+    }
+
+    // ---- epilogue: acc[0][cb][i] is row wave*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the group's 64;
+    // ring and operand buffers are idle now and become the staging of store_wave_part (4 KB per wavefront)
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    StoreTarget o;
+    o.c = p.c; o.bias = p.bias; o.m = p.m; o.n = p.n; o.nt = p.nt; o.slice = bb;
+    o.row0 = m0 + wave * 32; o.nt0 = nt0;
+    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32;
+    static_assert(LDS_BYTES >= NW * 4096, "staging of the epilogue does not fit into LDS");
+    store_wave_part<ACT>(acc, o, lds + wave * 4096, lane);
+}
+
+template <int W, int NW>
+static void launch_tall_act(const TileDev &p, int activation, uint32_t blocks, hipStream_t st) {
+    switch (activation) {
+        case TTMI_ACT_RELU: hipLaunchKernelGGL((matmul_tall_kernel<W, TTMI_ACT_RELU, NW>), dim3(blocks), dim3(64 * NW), 0, st, p); break;
+        case TTMI_ACT_GELU: hipLaunchKernelGGL((matmul_tall_kernel<W, TTMI_ACT_GELU, NW>), dim3(blocks), dim3(64 * NW), 0, st, p); break;
+        case TTMI_ACT_SILU: hipLaunchKernelGGL((matmul_tall_kernel<W, TTMI_ACT_SILU, NW>), dim3(blocks), dim3(64 * NW), 0, st, p); break;
+        default: hipLaunchKernelGGL((matmul_tall_kernel<W, TTMI_ACT_NONE, NW>), dim3(blocks), dim3(64 * NW), 0, st, p); break;
+    }
+}
+
 template <int W, int MB>
 static void launch_tile8_act(const TileDev &p, int activation, uint32_t blocks, hipStream_t st) {
     switch (activation) {
@@ -490,10 +712,27 @@ int matmul_bfp_tiled(const MatmulArgs &x, hipStream_t st) {
     p.kt = x.k / 32; p.nt = x.n / 32;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE; p.c_f32 = x.c_dtype == TTMI_FLOAT32;
     // 256-row blocks when they fill the chip, 128-row blocks otherwise (fewer idle CUs, half the accumulators).
-    // TTMI_MATMUL_BM forces a form: "256", "128" (eight wavefronts) or "4" (128 rows, four wavefronts).
+    // TTMI_MATMUL_BM forces a form: "256", "128" (eight wavefronts), "4" (128 rows, four wavefronts) or "384" (384 x 64).
     const uint32_t tiles_n = (x.n + TILE_COLS - 1) / TILE_COLS;
     const uint64_t big = (uint64_t)x.batch * ((x.m + 255) / 256) * tiles_n;
     const char *force_bm = getenv("TTMI_MATMUL_BM");
+    // 384-row x 64-column blocks (every weight expanded once per slice) when the slices are whole multiples of 384 rows
+    // and 128-row blocks would leave CUs without a workgroup
+    constexpr int TALL_WAVES = 12;
+    const uint64_t blocks_128 = (uint64_t)x.batch * ((x.m + 127) / 128) * tiles_n;
+    const uint64_t blocks_tall = (uint64_t)x.batch * ((x.m + 32 * TALL_WAVES - 1) / (32 * TALL_WAVES)) * ((x.n + 63) / 64);
+    const bool use_tall = force_bm ? force_bm[0] == '3' : (x.m % (32 * TALL_WAVES) == 0 && blocks_128 < 256 && blocks_tall > blocks_128);
+    if (use_tall) {
+        p.tiles_m = (x.m + 32 * TALL_WAVES - 1) / (32 * TALL_WAVES); p.tiles_n = (x.n + 63) / 64;
+        if (blocks_tall > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
+        if ((uint64_t)x.m * x.k * 2 > 0xffffffffull || (uint64_t)((x.m + 31) / 32) * p.kt * 2048 > 0xffffffffull)
+            return fail(TTMI_ERR_UNSUPPORTED, "matmul: one batch slice of A exceeds 4 GiB");
+        if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
+            return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
+        if (x.b_fmt == TTMI_BFLOAT8_B) launch_tall_act<7, TALL_WAVES>(p, x.activation, (uint32_t)blocks_tall, st);
+        else launch_tall_act<3, TALL_WAVES>(p, x.activation, (uint32_t)blocks_tall, st);
+        return check_launch("matmul_tall_kernel");
+    }
     const bool use_256 = force_bm ? force_bm[0] == '2' : (x.m > 128 && big >= 256 && x.m % 256 == 0);
     // 128-row blocks: eight wavefronts (each 64 rows) measure 6 % better than four for short k ranges (batched bmm,
     // k = 1024: epilogue and start-up are spread over twice as many wavefronts), four 1-2 % better for k = 4096
