@@ -468,16 +468,17 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
 //   A     nobody but its wavefront reads a band of 32 rows, so A goes from memory straight into registers in the layout of
 //         the MFMA's A operand, six k steps ahead (a ring through LDS holds at most two to three steps of 24 KB in flight,
 //         and with 1.5 to 2 us of latency that, not any pipe, set the step time)
-//   LDS   ring of 6 stages [packed W of the group], then two operand buffers [slab][operand][lane] x 16 B (step parity)
-//   step  wait for the own loads of step i+1, barrier, operands of step i from LDS -> 4 MFMAs (32x32x16); wavefronts 0..7
-//         expand their part of step i+1 between the two slabs; request step i+6
+//   LDS   ring of 6 stages [packed W of the group], then two operand buffers [step in pair][slab][operand][lane] x 16 B
+//         (pair parity)
+//   pair  two k steps per barrier: wait for the own loads of the next pair, barrier, operands of this pair from LDS ->
+//         8 MFMAs (32x32x16); wavefronts 0..7 expand their parts of the next pair in between; request the steps 6 ahead
 template <int W, int ACT, int NW>
 __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p) {
     using F = Wfmt<W>;
     constexpr int BM = 32 * NW;
     constexpr int D = 6;                                   // k steps requested ahead (A into registers, packed W into the ring)
     constexpr int STAGE_BYTES = F::stage_bytes;
-    constexpr int OPS_BYTES = 2 * 2 * 64 * 16;             // one operand buffer
+    constexpr int OPS_BYTES = 2 * 2 * 2 * 64 * 16;         // one operand buffer: the two k steps of a pair
     constexpr int OPS_BASE = D * STAGE_BYTES;
     constexpr int LDS_BYTES = OPS_BASE + 2 * OPS_BYTES > NW * 4096 ? OPS_BASE + 2 * OPS_BYTES : NW * 4096;
     constexpr int NLOAD = F::loads;
@@ -556,8 +557,8 @@ __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p
     const int es = (wave >> 2) & 1, pr = wave & 3;
     const uint32_t exp_off = F::exp_base + t_of_lane * 64 + fc * 16 + kh * 8 + es * 32 + 2 * pr;
     const uint32_t mant_off = (es * 4 + t_of_lane * 2 + fc) * F::face_stride + (kh * 8 + 2 * pr) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);
-    const uint32_t ops_write_off = OPS_BASE + (es * 2) * 1024 + lane * 16 + pr * 4;     // + parity * OPS_BYTES, + operand * 1024
-    const uint32_t ops_read_off = OPS_BASE + lane * 16;                             // + parity * OPS_BYTES, + (slab * 2 + operand) * 1024
+    const uint32_t ops_write_off = OPS_BASE + (es * 2) * 1024 + lane * 16 + pr * 4;     // + parity * OPS_BYTES, + step in pair * 4096, + operand * 1024
+    const uint32_t ops_read_off = OPS_BASE + lane * 16;                             // + parity * OPS_BYTES, + step in pair * 4096, + (slab * 2 + operand) * 1024
     f32x16 acc[1][2];
 #pragma unroll
     for (int cb = 0; cb < 2; ++cb)
@@ -591,7 +592,7 @@ __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p
     };
     // wavefronts 0..7: expand their two rows of the step in `from_stage` into operand buffer `parity`; the arithmetic is
     // that of weights_operand8 for one pair of rows
-    auto expand = [&](int from_stage, uint32_t parity) __attribute__((always_inline)) {
+    auto expand = [&](int from_stage, uint32_t ops_at) __attribute__((always_inline)) {
         const uint8_t *stage_at = lds + from_stage * STAGE_BYTES;
         const float scale0 = __uint_as_float((uint32_t)stage_at[exp_off] << 23), scale1 = __uint_as_float((uint32_t)stage_at[exp_off + 1] << 23);
         uint32_t word[2] = {*reinterpret_cast<const uint32_t *>(stage_at + mant_off), *reinterpret_cast<const uint32_t *>(stage_at + mant_off + F::row_bytes)};
@@ -614,47 +615,61 @@ __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p
         const uint32_t both1 = __builtin_amdgcn_perm(__float_as_uint(byte_to_float<1>(mag[1]) * scale1), __float_as_uint(byte_to_float<1>(mag[0]) * scale0), 0x07060302u);
         const uint32_t signs0 = __builtin_amdgcn_perm(word[1], word[0], (4u << 24) | (0x0cu << 16) | (0u << 8) | 0x0cu);
         const uint32_t signs1 = __builtin_amdgcn_perm(word[1], word[0], (5u << 24) | (0x0cu << 16) | (1u << 8) | 0x0cu);
-        *reinterpret_cast<uint32_t *>(lds + parity * OPS_BYTES + ops_write_off) = (signs0 & 0x80008000u) | both0;
-        *reinterpret_cast<uint32_t *>(lds + parity * OPS_BYTES + ops_write_off + 1024) = (signs1 & 0x80008000u) | both1;
+        *reinterpret_cast<uint32_t *>(lds + ops_at + ops_write_off) = (signs0 & 0x80008000u) | both0;
+        *reinterpret_cast<uint32_t *>(lds + ops_at + ops_write_off + 1024) = (signs1 & 0x80008000u) | both1;
     };
 
-    // prologue: the operands of step 0
-    wait_for_step(0);
+    // prologue: the operands of the first pair of steps
+    wait_for_step(total > 1 ? 1 : 0);
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __builtin_amdgcn_s_barrier();
-    if (wave < 8) expand(0, 0);
+    if (wave < 8) {
+        expand(0, 0);
+        if (total > 1) expand(1, 4096);
+    }
 
-    // one k step; SLOT = step % D
-    auto iteration = [&](auto slot_c) __attribute__((always_inline)) {
-        constexpr int SLOT = decltype(slot_c)::value, NEXT = (SLOT + 1) % D;
-        const bool more = step + 1 < total;
-        const uint32_t parity = step & 1;
-        if (more) wait_for_step(step + 1);
-        __builtin_amdgcn_s_waitcnt(0xC07F);   // our LDS reads and operand writes of the previous step are done
+    // Two k steps per barrier (a step alone is 4 MFMAs per wavefront, too little for what a barrier and the loop around
+    // it cost).  PAIR = (step / 2) % 3 names the slots 2 PAIR and 2 PAIR + 1; the second step of the last pair may not exist.
+    auto iteration = [&](auto pair_c) __attribute__((always_inline)) {
+        constexpr int FIRST = 2 * decltype(pair_c)::value, SECOND = FIRST + 1, NEXT0 = (FIRST + 2) % D, NEXT1 = (FIRST + 3) % D;
+        const bool have1 = step + 1 < total, more0 = step + 2 < total, more1 = step + 3 < total;
+        const uint32_t ops_now = ((step >> 1) & 1) * OPS_BYTES, ops_next = OPS_BYTES - ops_now;
+        if (more0) wait_for_step(more1 ? step + 3 : step + 2);
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // our LDS reads and operand writes of the previous pair are done
         __builtin_amdgcn_s_barrier();
-        bf16x8 b[2][2];
+        bf16x8 b[2][2][2];                    // [step in pair][slab][operand]
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int cb = 0; cb < 2; ++cb)
-                b[s][cb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + parity * OPS_BYTES + ops_read_off + (s * 2 + cb) * 1024));
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SLOT][0], b[0][0], acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SLOT][0], b[0][1], acc[0][1], 0, 0, 0);
-        if (more && wave < 8) expand(NEXT, parity ^ 1);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SLOT][1], b[1][0], acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SLOT][1], b[1][1], acc[0][1], 0, 0, 0);
-        // this step's registers and ring stage are free (the stage was read before the barrier above): request step + D
-        if (requested < total) { fetch(slot_c); ++requested; }
-        ++step;
+            for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb)
+                    b[h][sb][cb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + ops_now + ops_read_off + h * 4096 + (sb * 2 + cb) * 1024));
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[FIRST][0], b[0][0][0], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[FIRST][0], b[0][0][1], acc[0][1], 0, 0, 0);
+        if (more0 && wave < 8) expand(NEXT0, ops_next);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[FIRST][1], b[0][1][0], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[FIRST][1], b[0][1][1], acc[0][1], 0, 0, 0);
+        if (have1) {
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SECOND][0], b[1][0][0], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SECOND][0], b[1][0][1], acc[0][1], 0, 0, 0);
+        }
+        if (more1 && wave < 8) expand(NEXT1, ops_next + 4096);
+        if (have1) {
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SECOND][1], b[1][1][0], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SECOND][1], b[1][1][1], acc[0][1], 0, 0, 0);
+        }
+        // the pair's registers and ring stages are free (the stages were read before the barrier above): request the
+        // steps D ahead
+        if (requested < total) { fetch(std::integral_constant<int, FIRST>{}); ++requested; }
+        if (requested < total) { fetch(std::integral_constant<int, SECOND>{}); ++requested; }
+        step += 2;
     };
 #pragma unroll 1
     for (;;) {
-        iteration(S0{}); if (step == total) break;
-        iteration(S1{}); if (step == total) break;
-        iteration(S2{}); if (step == total) break;
-        iteration(S3{}); if (step == total) break;
-        iteration(S4{}); if (step == total) break;
-        iteration(S5{}); if (step == total) break;
+        iteration(S0{}); if (step >= total) break;
+        iteration(S1{}); if (step >= total) break;
+        iteration(S2{}); if (step >= total) break;
     }
 
     // ---- epilogue: acc[0][cb][i] is row wave*32 + (i/4)*8 + kh*4 + i%4, column 4*c16 + 2*half + cb of the group's 64;
