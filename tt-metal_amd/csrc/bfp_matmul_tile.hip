@@ -529,14 +529,24 @@ __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p
     }
     if (p.a_tiled) { a_base = p.a + (uint64_t)bb * ((p.m + 31) / 32) * p.kt * 2048; a_step = 2048; }
     else { a_base = p.a + (uint64_t)bb * p.m * p.k * 2; a_step = 64; }
-    bf16x8 a_ring[D][A_LOADS];
+    // The loads of A and the waits for them are inline assembly: with direct-to-LDS loads pending, the compiler's own
+    // wait before the first use of a loaded register is for ALL vector-memory operations (seen here once per trip of the
+    // loop, which emptied the six-step pipeline every six steps).  The ring registers are read-write operands of the
+    // loads, so each entry stays in one physical register from request to use; vector-memory operations complete in
+    // order, so wait_for_step() covers them.
+    u32x4 a_ring[D][A_LOADS];
+#pragma unroll
+    for (int u = 0; u < D; ++u)
+#pragma unroll
+        for (int sl = 0; sl < A_LOADS; ++sl) a_ring[u][sl] = u32x4{0u, 0u, 0u, 0u};
 
     // requests of one k step: slot = step % D names both the registers for A and the ring stage for the packed weights
     auto fetch = [&](auto slot_c) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
         uint8_t *base = lds + SLOT * STAGE_BYTES;
 #pragma unroll
-        for (int sl = 0; sl < A_LOADS; ++sl) a_ring[SLOT][sl] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(a_base + a_off[sl]));
+        for (int sl = 0; sl < A_LOADS; ++sl)
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "+v"(a_ring[SLOT][sl]) : "v"(a_off[sl]), "s"(a_base) : "memory");
         if (wave == 0) {
 #pragma unroll
             for (int l = 0; l < W_LOADS0; ++l)
@@ -634,7 +644,8 @@ __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p
         constexpr int FIRST = 2 * decltype(pair_c)::value, SECOND = FIRST + 1, NEXT0 = (FIRST + 2) % D, NEXT1 = (FIRST + 3) % D;
         const bool have1 = step + 1 < total, more0 = step + 2 < total, more1 = step + 3 < total;
         const uint32_t ops_now = ((step >> 1) & 1) * OPS_BYTES, ops_next = OPS_BYTES - ops_now;
-        if (more0) wait_for_step(more1 ? step + 3 : step + 2);
+        wait_for_step(more1 ? step + 3 : more0 ? step + 2 : have1 ? step + 1 : step);   // the next pair's weights; at the end at least this pair's A
+        asm volatile("" : "+v"(a_ring[FIRST][0]), "+v"(a_ring[FIRST][1]), "+v"(a_ring[SECOND][0]), "+v"(a_ring[SECOND][1]) :: "memory");   // uses stay behind the wait
         __builtin_amdgcn_s_waitcnt(0xC07F);   // our LDS reads and operand writes of the previous pair are done
         __builtin_amdgcn_s_barrier();
         bf16x8 b[2][2][2];                    // [step in pair][slab][operand]
@@ -645,19 +656,19 @@ __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p
 #pragma unroll
                 for (int cb = 0; cb < 2; ++cb)
                     b[h][sb][cb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(lds + ops_now + ops_read_off + h * 4096 + (sb * 2 + cb) * 1024));
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[FIRST][0], b[0][0][0], acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[FIRST][0], b[0][0][1], acc[0][1], 0, 0, 0);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_ring[FIRST][0]), b[0][0][0], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_ring[FIRST][0]), b[0][0][1], acc[0][1], 0, 0, 0);
         if (more0 && wave < 8) expand(NEXT0, ops_next);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[FIRST][1], b[0][1][0], acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[FIRST][1], b[0][1][1], acc[0][1], 0, 0, 0);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_ring[FIRST][1]), b[0][1][0], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_ring[FIRST][1]), b[0][1][1], acc[0][1], 0, 0, 0);
         if (have1) {
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SECOND][0], b[1][0][0], acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SECOND][0], b[1][0][1], acc[0][1], 0, 0, 0);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_ring[SECOND][0]), b[1][0][0], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_ring[SECOND][0]), b[1][0][1], acc[0][1], 0, 0, 0);
         }
         if (more1 && wave < 8) expand(NEXT1, ops_next + 4096);
         if (have1) {
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SECOND][1], b[1][1][0], acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_ring[SECOND][1], b[1][1][1], acc[0][1], 0, 0, 0);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_ring[SECOND][1]), b[1][1][0], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_ring[SECOND][1]), b[1][1][1], acc[0][1], 0, 0, 0);
         }
         // the pair's registers and ring stages are free (the stages were read before the barrier above): request the
         // steps D ahead
