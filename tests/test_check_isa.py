@@ -99,3 +99,44 @@ def test_inline_lds_reads_are_in_flight_until_lgkmcnt_zero(tmp_path, capsys):
     # the compiler's own combined wait releases them as well
     also_good = ring + asm("ds_read_b64 v[40:41], v5 offset:32") + "\ts_waitcnt vmcnt(0) lgkmcnt(0)\n\tv_add_u32_e32 v42, v40, v41\n"
     assert run(tmp_path, also_good) == 0
+
+
+# ---- the 384-row GEMM: ring registers are read by the MFMAs directly, behind the kernel's own partial wait -------------
+TALL_HEAD = "_ZN4ttmi18matmul_tall_kernelILi7ELi0ELi12EEEvNS_7TileDevE:\n"
+
+
+def run_tall(tmp_path, body):
+    f = tmp_path / "t.s"
+    f.write_text(TALL_HEAD + body + TAIL)
+    return check_isa.check_ring_operands(str(f))
+
+
+TALL_OK = (
+    "\tv_mov_b32_e32 v34, 0\n\tv_mov_b32_e32 v35, v34\n"                    # zero initialisation before the first load
+    + asm("global_load_dwordx4 v[34:37], v116, s[4:5]")
+    + ".LBB0_1:\n"
+    + "\ts_waitcnt vmcnt(2)\n\ts_barrier\n"
+    + "\tv_mfma_f32_32x32x16_bf16 v[2:17], v[34:37], v[82:85], v[2:17]\n"
+    + "\tv_mfma_f32_32x32x16_bf16 v[18:33], v[34:37], v[86:89], v[18:33]\n"
+    + asm("global_load_dwordx4 v[34:37], v116, s[4:5]")
+    + "\ts_cbranch_scc1 .LBB0_1\n"
+    + "\ts_waitcnt vmcnt(0)\n"
+)
+
+
+def test_tall_kernel_ring_read_only_by_mfma_passes(tmp_path):
+    assert run_tall(tmp_path, TALL_OK) == 0
+
+
+def test_tall_kernel_copy_of_a_ring_register_in_flight_is_rejected(tmp_path):
+    bad = TALL_OK.replace("\ts_cbranch_scc1 .LBB0_1\n", "\tv_mov_b32_e32 v90, v35\n\ts_cbranch_scc1 .LBB0_1\n")
+    assert run_tall(tmp_path, bad) > 0
+
+
+def test_tall_kernel_mfma_writing_a_ring_register_in_flight_is_rejected(tmp_path):
+    bad = TALL_OK.replace("\ts_waitcnt vmcnt(2)\n", "\tv_mfma_f32_32x32x16_bf16 v[34:49], v[50:53], v[82:85], v[34:49]\n\ts_waitcnt vmcnt(2)\n")
+    assert run_tall(tmp_path, bad) > 0
+
+
+def test_tall_kernel_without_inline_loads_is_reported(tmp_path):
+    assert run_tall(tmp_path, "\tv_mfma_f32_32x32x16_bf16 v[2:17], v[34:37], v[82:85], v[2:17]\n") > 0

@@ -18,6 +18,9 @@ and fails the build if any compiler-generated instruction mentions a register wh
 still in flight when the kernel ends.
 
     python tt-metal_amd/check_isa.py file.s
+
+A second, simpler check (check_ring_operands, `--ring-operands file.s`) covers the 384-row kernel of bfp_matmul_tile.hip,
+whose inline loads of A land in registers that the MFMAs read directly; it is described at the function.
 """
 from __future__ import annotations
 
@@ -92,7 +95,7 @@ def _blocks(body):
     return blocks
 
 
-def _check_kernel(name, body, problems):
+def _check_kernel(name, body, problems, release_on_mfma=False):
     blocks = _blocks(body)
     index = {b["label"]: i for i, b in enumerate(blocks) if b["label"] is not None}
     succs = []
@@ -132,6 +135,13 @@ def _check_kernel(name, body, problems):
             if text.startswith("s_waitcnt") and "vmcnt(0)" in text:      # every vector-memory operation has landed
                 ring.clear()
                 slot.clear()
+                continue
+            if release_on_mfma and text.startswith("v_mfma"):
+                operands = text.split(None, 1)[1].split(",")
+                written = _regs(operands[0]) & ring
+                if written and report is not None:
+                    report.append(f"{name}: an MFMA writes registers {sorted(written)} while a hand-scheduled load into them is in flight: {text}")
+                ring -= _regs(",".join(operands[1:]))
                 continue
             if report is not None:
                 hit = _regs(text) & (ring | slot | lds)
@@ -181,5 +191,25 @@ def check(path: str, kernel_substrings=("matmul_stream_kernel", "matmul_wide_ker
     return len(problems)
 
 
+def check_ring_operands(path: str, kernel_substrings=("matmul_tall_kernel",)) -> int:
+    """The 384-row GEMM of bfp_matmul_tile.hip loads its A operands with inline `global_load_dwordx4 vDST, vOFF, s[..]` into
+    a ring of registers that the MFMAs read directly, behind the kernel's own partial waits.  Here a register is in flight
+    from its inline load until the first compiler-generated v_mfma that reads it (the kernel puts that behind its wait);
+    any other compiler-generated instruction naming it meanwhile (a copy, a spill, a reuse) fails the build, as does an
+    MFMA that writes it."""
+    problems, checked = [], 0
+    with open(path) as f:
+        lines = f.read().split("\n")
+    for name, body in _kernels(lines):
+        if any(k in name for k in kernel_substrings):
+            checked += 1
+            _check_kernel(name, body, problems, release_on_mfma=True)
+    if not checked:
+        problems.append(f"no kernel matching {kernel_substrings} in {path}")
+    for p in problems[:40]:
+        print("check_isa:", p, file=sys.stderr)
+    return len(problems)
+
+
 if __name__ == "__main__":
-    sys.exit(1 if check(sys.argv[1]) else 0)
+    sys.exit(1 if (check_ring_operands(sys.argv[2]) if sys.argv[1] == "--ring-operands" else check(sys.argv[1])) else 0)
