@@ -41,6 +41,12 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("" ::: "memory");
 }
 
+// Scale of a face row from its shared exponent byte: the byte moved into the exponent field of a float, 2^(E - 127) —
+// 2^(bias_exp - 127) times too large for every row alike (whoever stores the sums takes that power of two out again,
+// exactly).  E = 0 is read as E = 1, the IEEE convention for a zero exponent field, which is also what the hidden-one
+// form of the streaming kernels gives: every GEMM kernel treats such rows (fp32 subnormal sources) alike.
+__device__ __forceinline__ float row_scale(uint32_t e) { return __uint_as_float(max(e, 1u) << 23); }
+
 template <int ACT> __device__ __forceinline__ float apply_activation(float x) {
     if (ACT == TTMI_ACT_RELU) return x > 0.f ? x : 0.f;
     if (ACT == TTMI_ACT_GELU) return 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
@@ -88,38 +94,6 @@ __device__ __forceinline__ bf16x8 weights_operand8(const uint32_t (&words)[8], c
     return __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
 }
 
-// BFLOAT4_B, four operands from 8 mantissa words of 8 k rows (lane uses the half of each word that q selects): a code is
-// sign + a 3-bit integer, which fp8 (e4m3) holds exactly, and gfx950 converts two fp8 bytes to two bf16 times a power of two
-// in one instruction (v_cvt_scalef32_pk_bf16_fp8: the scale is the exponent of a float, i.e. exactly the row scale used
-// here; checked on the hardware for every code and exponent).  Per row: spread the nibbles, look the magnitudes up in a
-// byte table (v_perm_b32), put the signs on top, two conversions; per pair of rows four v_perm_b32 bring (row, row + 1) of a
-// column together.  About 3 instructions per weight instead of 5.5 for convert-and-scale; the values are the same except in
-// rows with E = 0, which contribute their mantissa times 2^-129 instead of nothing.
-__device__ __forceinline__ void bfp4_operands(const uint32_t (&words)[8], int q, const float (&scale)[8], bf16x8 (&bop)[4]) {
-    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-    uint32_t lo[8], hi[8];         // (columns 0, 1) and (columns 2, 3) of row jj as bf16 pairs
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) {
-        uint32_t v = (words[jj] >> (16 * (q & 1))) & 0xffffu;
-        v = (v | (v << 8)) & 0x00ff00ffu;
-        v = (v | (v << 4)) & 0x0f0f0f0fu;                                   // one code per byte
-        // e4m3 bytes of 0..7: 00 38 40 44 48 4A 4C 4E
-        const uint32_t fp8 = ((v << 4) & 0x80808080u) | __builtin_amdgcn_perm(0x4E4C4A48u, 0x44403800u, v & 0x07070707u);
-        lo[jj] = __builtin_bit_cast(uint32_t, (bf16x2_t)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(fp8, scale[jj], false));
-        hi[jj] = __builtin_bit_cast(uint32_t, (bf16x2_t)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(fp8, scale[jj], true));
-    }
-    uint32_t packed[4][4];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        packed[0][p] = __builtin_amdgcn_perm(lo[2 * p + 1], lo[2 * p], 0x05040100u);
-        packed[1][p] = __builtin_amdgcn_perm(lo[2 * p + 1], lo[2 * p], 0x07060302u);
-        packed[2][p] = __builtin_amdgcn_perm(hi[2 * p + 1], hi[2 * p], 0x05040100u);
-        packed[3][p] = __builtin_amdgcn_perm(hi[2 * p + 1], hi[2 * p], 0x07060302u);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) bop[j] = __builtin_bit_cast(bf16x8, make_uint4(packed[j][0], packed[j][1], packed[j][2], packed[j][3]));
-}
-
 // Fills `chunk_of[l]` with the global chunk (16 bytes, counted from the start of a 2-tile run) that lands in this
 // lane's slot of direct-to-LDS load l, for the stage layout described at Wfmt.
 template <int W> __device__ __forceinline__ void stage_chunks(int lane, uint32_t (&chunk_of)[Wfmt<W>::loads]) {
@@ -142,58 +116,15 @@ template <int W> __device__ __forceinline__ void stage_chunks(int lane, uint32_t
     }
 }
 
-// The four bf16 B operands (columns 4c+0..3 of a 64-column group, k rows 8g..8g+7) of lane (c = lane % 16,
-// g = lane / 16) from a staged pair of packed tiles.  exp_at / mant_at: this lane's LDS byte addresses of the
-// exponents and mantissa words in stage 0 (see Wfmt); q = c % 4.  `after_lds_reads` runs once every LDS read has
-// returned (the stage may be refilled).
-// LDS reads are written as inline assembly: the compiler orders every LDS read it knows of behind ALL outstanding
-// direct-to-LDS loads (it cannot tell that they write other stages), which would drain the prefetch pipeline at
-// every unit.  STAGE_OFF is a compile-time byte offset added to both addresses; the s_waitcnt carries the results
-// as operands so that nothing that uses them can be scheduled in front of it.
-template <int W, int STAGE_OFF, typename AfterReads>
-__device__ __forceinline__ void staged_operands(uint32_t exp_at, uint32_t mant_at, int q, AfterReads after_lds_reads, bf16x8 (&bop)[4]) {
-    using F = Wfmt<W>;
-    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-    uint32_t e[8], words[8], mags[8];
-    u32x2 e01, w01, w23, w45, w67;
-    const uint32_t mant_stage = mant_at + STAGE_OFF;
-    constexpr int R = F::row_bytes / 4;      // dwords between consecutive k rows
-    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(e01) : "v"(exp_at), "n"(STAGE_OFF));
-    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(w01) : "v"(mant_stage), "n"(0 * R), "n"(1 * R));
-    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(w23) : "v"(mant_stage), "n"(2 * R), "n"(3 * R));
-    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(w45) : "v"(mant_stage), "n"(4 * R), "n"(5 * R));
-    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(w67) : "v"(mant_stage), "n"(6 * R), "n"(7 * R));
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e01), "+v"(w01), "+v"(w23), "+v"(w45), "+v"(w67)::"memory");
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) e[jj] = (e01[jj >> 2] >> (8 * (jj & 3))) & 0xffu;
-    words[0] = w01[0]; words[1] = w01[1]; words[2] = w23[0]; words[3] = w23[1];
-    words[4] = w45[0]; words[5] = w45[1]; words[6] = w67[0]; words[7] = w67[1];
-    after_lds_reads();
-    // The scale of row jj is its exponent byte moved into the exponent field of a float: 2^(E - 127), that is
-    // 2^(bias_exp - 127) times too large for every row alike; whoever stores the sums takes that power of two out
-    // again (exactly, see Wfmt::unscale).  Rows with E = 0 (all zeros, or fp32 subnormals below 2^-126) get scale 0.
-    float scale[8];
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(e[jj] << 23);
-    if constexpr (W == 3) {
-        bfp4_operands(words, q, scale, bop);
-    } else {
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) mags[jj] = words[jj] & 0x7f7f7f7fu;
-        bop[0] = weights_operand8<0>(words, mags, scale);
-        bop[1] = weights_operand8<1>(words, mags, scale);
-        bop[2] = weights_operand8<2>(words, mags, scale);
-        bop[3] = weights_operand8<3>(words, mags, scale);
-    }
-}
-
-// The same in two steps, for kernels that read several slabs before they wait: what one lane reads from LDS for 8 k rows
-// of one face (8 exponent bytes, 8 mantissa words) ...
+// What one lane reads from LDS for 8 k rows of one face of a staged pair of packed tiles (8 exponent bytes, 8 mantissa
+// words; exp_at / mant_at: this lane's LDS byte addresses in stage 0, see Wfmt).  LDS reads are written as inline
+// assembly: the compiler orders every LDS read it knows of behind ALL outstanding direct-to-LDS loads (it cannot tell
+// that they write other stages), which would drain the prefetch pipeline at every unit.
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 struct SlabRaw { u32x2 e01, w01, w23, w45, w67; };
 
-// ... requested here (inline assembly for the reason given at staged_operands; EXP_OFF / MANT_OFF are compile-time byte
-// offsets; the caller waits with wait_slabs before it touches the result) ...
+// requested here (EXP_OFF / MANT_OFF are compile-time byte offsets; the caller waits with wait_slab / wait_slabs, which
+// carry the results as operands so that nothing that uses them can be scheduled in front of the wait)
 template <int W, int EXP_OFF, int MANT_OFF> __device__ __forceinline__ void slab_read(uint32_t exp_at, uint32_t mant_at, SlabRaw &r) {
     constexpr int R = Wfmt<W>::row_bytes / 4;
     const uint32_t mant = mant_at + MANT_OFF;
@@ -203,26 +134,69 @@ template <int W, int EXP_OFF, int MANT_OFF> __device__ __forceinline__ void slab
     asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w45) : "v"(mant), "n"(4 * R), "n"(5 * R));
     asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w67) : "v"(mant), "n"(6 * R), "n"(7 * R));
 }
+__device__ __forceinline__ void wait_slab(SlabRaw &a) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.e01), "+v"(a.w01), "+v"(a.w23), "+v"(a.w45), "+v"(a.w67)::"memory");
+}
 __device__ __forceinline__ void wait_slabs(SlabRaw &a, SlabRaw &b) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.e01), "+v"(a.w01), "+v"(a.w23), "+v"(a.w45), "+v"(a.w67),
                                           "+v"(b.e01), "+v"(b.w01), "+v"(b.w23), "+v"(b.w45), "+v"(b.w67)::"memory");
 }
-// ... and expanded into the four B operands (byte j of every word = operand j, as above; BFLOAT4_B through bfp4_operands).
-template <int W> __device__ __forceinline__ void slab_expand(const SlabRaw &r, int q, bf16x8 (&bop)[4]) {
+// Expansion without arithmetic ("hidden-one form"), for kernels that are bound by vector-ALU issue rather than by the
+// matrix pipe.  A code (sign s, mantissa m of W bits) under the shared exponent E of its face row is written into a bf16 as
+//      hi[15] = s, hi[14:7] = E, hi[6:7-W] = m          value  +-(1 + m / 2^W) * 2^(E - 127)
+// and a second operand carries sign and exponent alone
+//      lo[15] = s, lo[14:7] = E                          value  +-2^(E - 127)
+// so that hi - lo = +-m * 2^(E - 127 - W), half of the weight m * 2^(E - 127 - (W - 1)) the reference unpacker produces
+// (bfloat8.hpp:229-249, bfloat4.hpp:113-146): A.W = hidden_unscale * (A.hi - A.lo), exactly (both operands and every
+// product are exact; only the fp32 additions see other intermediate sums than a product with the expanded weight would).
+// Nothing is converted, multiplied or normalised: per pair of k rows one v_perm_b32 brings the two codes of a column
+// together and two v_and_or_b32 assemble hi and lo; the exponent field of a pair of rows is prepared once for the four
+// operands.  Edge rows: E = 0 makes hi a bf16 subnormal and lo a zero, and the matrix cores keep subnormals, so such a row
+// is read with the scale of E = 1 (the IEEE convention for a zero exponent field; all-zero rows give exactly 0);
+// E = 255 (Inf / NaN sources) makes the sums of the 16 columns that share the exponent non-finite; every other exponent,
+// 254 included, is exact.
+constexpr float hidden_unscale = 2.0f;
+
+// exponent field of k rows (2p, 2p + 1), one in each half of a word
+__device__ __forceinline__ uint32_t hidden_pair_field(const u32x2 e01, int p) {
+    const uint32_t ew = e01[p >> 1];
+    const uint32_t spread = (p & 1) ? __builtin_amdgcn_perm(0u, ew, 0x0c030c02u) : __builtin_amdgcn_perm(0u, ew, 0x0c010c00u);   // [E(2p), 0, E(2p+1), 0]
+    return spread << 7;
+}
+
+template <int W> __device__ __forceinline__ void slab_expand_hidden(const SlabRaw &r, int q, bf16x8 (&hi)[4], bf16x8 (&lo)[4]) {
     const uint32_t words[8] = {r.w01[0], r.w01[1], r.w23[0], r.w23[1], r.w45[0], r.w45[1], r.w67[0], r.w67[1]};
-    float scale[8];
+    uint32_t hi_w[4][4], lo_w[4][4];     // [operand j][row pair p]
 #pragma unroll
-    for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(((r.e01[jj >> 2] >> (8 * (jj & 3))) & 0xffu) << 23);
-    if constexpr (W == 3) {
-        bfp4_operands(words, q, scale, bop);
-    } else {
-        uint32_t mags[8];
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t field = hidden_pair_field(r.e01, p);
+        if constexpr (W == 7) {
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) mags[jj] = words[jj] & 0x7f7f7f7fu;
-        bop[0] = weights_operand8<0>(words, mags, scale);
-        bop[1] = weights_operand8<1>(words, mags, scale);
-        bop[2] = weights_operand8<2>(words, mags, scale);
-        bop[3] = weights_operand8<3>(words, mags, scale);
+            for (int j = 0; j < 4; ++j) {
+                // both codes of column j, each in both bytes of its half
+                const uint32_t sel = ((4u + j) << 24) | ((4u + j) << 16) | ((uint32_t)j << 8) | (uint32_t)j;
+                const uint32_t both = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], sel);
+                hi_w[j][p] = (both & 0x807f807fu) | field;
+                lo_w[j][p] = (both & 0x80008000u) | field;
+            }
+        } else {
+            // this lane's four codes of each row: the 16-bit half (q & 1) of the row's word, row 2p in the low half
+            const uint32_t both = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], (q & 1) ? 0x07060302u : 0x05040100u);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // code j sits at bits 4j..4j+3 of each half: its sign goes to bit 15, its mantissa to bits 6..4 (bits that a
+                // shift carries over from the other half never reach the masked positions)
+                const uint32_t s_at = j == 3 ? both : both << (12 - 4 * j);
+                const uint32_t m_at = j == 0 ? both << 4 : j == 1 ? both : both >> (4 * j - 4);
+                lo_w[j][p] = (s_at & 0x80008000u) | field;
+                hi_w[j][p] = (m_at & 0x00700070u) | lo_w[j][p];
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        hi[j] = __builtin_bit_cast(bf16x8, make_uint4(hi_w[j][0], hi_w[j][1], hi_w[j][2], hi_w[j][3]));
+        lo[j] = __builtin_bit_cast(bf16x8, make_uint4(lo_w[j][0], lo_w[j][1], lo_w[j][2], lo_w[j][3]));
     }
 }
 

@@ -44,8 +44,7 @@ struct MatmulDev {
     uint32_t groups;         // batch * mt * ngroups
     uint32_t workgroups;     // P
     uint32_t units;          // U = batch * mt * ngroups * kt
-    uint32_t share, extra;   // U = P * share + extra: the first `extra` workgroups take share + 1 units
-    uint32_t split;          // k ranges per output group, or 0 for stream-K
+    uint32_t split;          // k ranges per output group (>= 1)
     int a_tiled, c_tiled, c_f32;
 };
 
@@ -84,22 +83,15 @@ __device__ __forceinline__ u32x4 slot_load_issue(const float4 *from) {
 }
 __device__ __forceinline__ uint32_t not_empty(uint32_t bits) { return bits == SLOT_EMPTY ? 0xfffffffeu : bits; }
 
-// Which units a workgroup takes.
-//   split > 0   every output group is cut into `split` nearly equal k ranges, one per workgroup (P = groups * split):
-//               one output per workgroup, at most `split` partial sums to add
-//   split == 0  "stream-K": the U units are dealt out contiguously, the first `extra` workgroups take share + 1 units,
-//               the rest `share`; a range may end one output and begin the next (the host does not choose this)
+// Which units a workgroup takes: every output group is cut into `split` nearly equal k ranges, one per workgroup
+// (P = groups * split): one output per workgroup, at most `split` partial sums to add.  Units are numbered with the
+// k-tile fastest.
 __device__ __forceinline__ uint32_t range_start(const MatmulDev &p, uint32_t i) {
-    if (p.split) return (i / p.split) * p.kt + ((i % p.split) * p.kt) / p.split;
-    return i * p.share + min(i, p.extra);
+    return (i / p.split) * p.kt + ((i % p.split) * p.kt) / p.split;
 }
 __device__ __forceinline__ uint32_t workgroup_of(const MatmulDev &p, uint32_t unit) {
-    if (p.split) {
-        const uint32_t og = unit / p.kt, within = unit - og * p.kt;
-        return og * p.split + ((within + 1) * p.split - 1) / p.kt;     // largest part j with (j * kt) / split <= within
-    }
-    const uint32_t fat = p.extra * (p.share + 1);
-    return unit < fat ? unit / (p.share + 1) : p.extra + (unit - fat) / p.share;
+    const uint32_t og = unit / p.kt, within = unit - og * p.kt;
+    return og * p.split + ((within + 1) * p.split - 1) / p.kt;     // largest part j with (j * kt) / split <= within
 }
 
 // Work decomposition: units are numbered with the k-tile fastest; a workgroup takes a contiguous range of them (see
@@ -199,13 +191,24 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
                 asm volatile("v_mov_b32 %0, %1" : "=v"(moved) : "v"(a_ring[S][h][e]));
                 a_now[h][e] = moved;
             }
-        const bf16x8 a_lo = __builtin_bit_cast(bf16x8, a_now[0]), a_hi = __builtin_bit_cast(bf16x8, a_now[1]);
-        bf16x8 bop[4];
-        staged_operands<W, S * F::stage_bytes>(lds_base + exp_off, lds_base + mant_off, q, [&]() __attribute__((always_inline)) { if (refill) fetch(stage_tag); }, bop);
+        // weights in hidden-one form (bfp_dequant.h): A.W = 2 (A.hi - A.lo), the subtraction as an MFMA with the negated activations
+        u32x4 a_neg[2];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bop[j], acc[0][j], 0, 0, 0);
-            acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bop[j], acc[1][j], 0, 0, 0);
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a_neg[h][e] = a_now[h][e] ^ 0x80008000u;
+        SlabRaw raw;
+        slab_read<W, S * F::stage_bytes, S * F::stage_bytes>(lds_base + exp_off, lds_base + mant_off, raw);
+        wait_slab(raw);
+        if (refill) fetch(stage_tag);
+        bf16x8 hi[4], lo[4];
+        slab_expand_hidden<W>(raw, q, hi, lo);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_now[h]), hi[j], acc[h][j], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_neg[h]), lo[j], acc[h][j], 0, 0, 0);
         }
     };
 
@@ -388,7 +391,7 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
                 float v[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    float x = mine[r][j] * F::unscale;
+                    float x = mine[r][j] * hidden_unscale;
                     if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
                     v[j] = apply_activation<ACT>(x);
                 }
@@ -433,6 +436,7 @@ constexpr int WIDE_COLS = WIDE_TILES * 32;
 #ifndef TTMI_WIDE_STAGES
 #define TTMI_WIDE_STAGES 2      // measured: 2 beats 3 by 1.5 us on the Falcon h_to_4h shape (less code, fewer registers), 4 leaves one workgroup per CU
 #endif
+constexpr int WEIGHTS_ONCE = 2;     // cache policy of the weight loads: nt (read once, not to displace the activations in L2); measured 0.4 us per launch
 constexpr int WIDE_WGS_PER_CU = TTMI_WIDE_WGS_PER_CU;
 constexpr int WIDE_STAGES = TTMI_WIDE_STAGES;
 constexpr int WIDE_REDUCE_BYTES = WAVES * 32 * 64 * 4;     // every wavefront lays out half of its 64 accumulator registers
@@ -522,7 +526,7 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
             for (int l = 0; l < NLOAD; ++l)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[pr][l]),
                                                  (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * UNIT_BYTES + pr * PAIR_STRIDE + l * 1024),
-                                                 16, 0, 0);
+                                                 16, 0, WEIGHTS_ONCE);
         wptr += w_step;
         asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][0]) : "v"(aptr) : "memory");
         asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][1]) : "v"(aptr + a_second) : "memory");
@@ -547,13 +551,23 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         slab_read<W, S * UNIT_BYTES + 32, S * UNIT_BYTES + 4 * F::face_stride>(exp_at, mant_at, raw1);
         wait_slabs(raw0, raw1);
         if (refill) fetch(stage_tag);
-        bf16x8 bop[4];
-        slab_expand<W>(raw0, q, bop);
+        // hidden-one form (bfp_dequant.h): A.W = 2 (A.hi - A.lo); the subtraction is an MFMA with the negated activations
+        bf16x8 hi[4], lo[4];
+        u32x4 a_neg[2];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[0]), bop[j], acc[j], 0, 0, 0);
-        slab_expand<W>(raw1, q, bop);
+        for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[1]), bop[j], acc[j], 0, 0, 0);
+            for (int e = 0; e < 4; ++e) a_neg[s][e] = a_now[s][e] ^ 0x80008000u;
+        slab_expand_hidden<W>(raw0, q, hi, lo);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[0]), hi[j], acc[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[0]), lo[j], acc[j], 0, 0, 0);
+        slab_expand_hidden<W>(raw1, q, hi, lo);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[1]), hi[j], acc[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[1]), lo[j], acc[j], 0, 0, 0);
     };
 
     // This wavefront's units: k_begin + wave, + WAVES, ...; unit i lives in stage i % STAGES and is requested STAGES
@@ -625,7 +639,7 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         float v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            float x = sums[j] * F::unscale;
+            float x = sums[j] * hidden_unscale;
             if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
             v[j] = apply_activation<ACT>(x);
         }
@@ -749,9 +763,7 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     d.units = d.groups * d.kt;
     // Workgroups to aim for, every output's k range being cut into as many parts as get there (every wavefront keeping
     // >= 2 k-tiles).  64-column kernel: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone nearly get
-    // there, x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot reset; the kernel
-    // can also deal the units out evenly across output boundaries, split == 0, but a workgroup that is consumer of one
-    // output and producer of the next would then make its successor wait: not offered).  128-column kernel: two
+    // there, x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot reset).  128-column kernel: two
     // workgroups per CU (all it can hold, the collecting workgroups included) when that takes few parts per output, one
     // per CU when the outputs are few (measured: many short k ranges cost more than the second workgroup gains).
     const bool few = d.groups < 100;
@@ -802,12 +814,12 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
     p.mt = d.mt; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.groups = (uint32_t)d.groups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
-    p.share = p.units / p.workgroups; p.extra = p.units % p.workgroups; p.split = d.split;
+    p.split = d.split;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE;
     p.c_f32 = x.c_dtype == TTMI_FLOAT32;
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
-    if (d.units > 0x7fffffffull || d.groups * (d.split ? d.split : 1) > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
+    if (d.units > 0x7fffffffull || d.groups * d.split > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
     const size_t need = slot_bytes_needed(d, wide);
     void *slots = nullptr;
     if (need == 0) {

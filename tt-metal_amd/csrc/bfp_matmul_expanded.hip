@@ -66,9 +66,8 @@ __global__ __launch_bounds__(256) void expand_kernel(const uint8_t *__restrict__
         for (int jj = 0; jj < 8; ++jj) e[jj] = lds[exp_off + jj];
 #pragma unroll
         for (int jj = 0; jj < 8; ++jj) words[jj] = *reinterpret_cast<const uint32_t *>(lds + mant_off + jj * F::row_bytes);
-        // row scale = exponent byte in the exponent field of a float (see staged_operands in bfp_dequant.h)
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(e[jj] << 23);
+        for (int jj = 0; jj < 8; ++jj) scale[jj] = row_scale(e[jj]);
 #pragma unroll
         for (int jj = 0; jj < 8; ++jj) {
             if (W == 7) {

@@ -58,10 +58,10 @@ template <int W> __device__ __forceinline__ void read_slab(const uint8_t *lds, u
 // Row scales and mantissa-only words of a slab; `half_shift` = 16 * (c / 16) brings this lane's two columns to bytes 0, 1.
 // The scale of a row is its exponent byte moved into the exponent field of a float: 2^(E - 127), i.e. 2^(bias_exp - 127)
 // times too large for every row alike; the epilogue takes that power of two out of the sums again (exactly).  Rows with
-// E = 0 (all zeros or fp32 subnormals, magnitudes below 2^-126) get scale 0.
+// E = 0 are read as E = 1 (row_scale in bfp_dequant.h).
 template <int W> __device__ __forceinline__ void prepare_slab(Slab &s, int q, uint32_t half_shift, float (&scale)[8], uint32_t (&mags)[8]) {
 #pragma unroll
-    for (int jj = 0; jj < 8; ++jj) scale[jj] = __uint_as_float(s.e[jj] << 23);
+    for (int jj = 0; jj < 8; ++jj) scale[jj] = row_scale(s.e[jj]);
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) {
         if (W == 7) {
@@ -604,7 +604,7 @@ __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p
     // that of weights_operand8 for one pair of rows
     auto expand = [&](int from_stage, uint32_t ops_at) __attribute__((always_inline)) {
         const uint8_t *stage_at = lds + from_stage * STAGE_BYTES;
-        const float scale0 = __uint_as_float((uint32_t)stage_at[exp_off] << 23), scale1 = __uint_as_float((uint32_t)stage_at[exp_off + 1] << 23);
+        const float scale0 = row_scale(stage_at[exp_off]), scale1 = row_scale(stage_at[exp_off + 1]);
         uint32_t word[2] = {*reinterpret_cast<const uint32_t *>(stage_at + mant_off), *reinterpret_cast<const uint32_t *>(stage_at + mant_off + F::row_bytes)};
         uint32_t mag[2];
 #pragma unroll
