@@ -96,6 +96,26 @@ TTMI_API int ttmi_tilize(const void *src, uint32_t elem_size, uint32_t batch, ui
 TTMI_API int ttmi_untilize(const void *src, uint32_t elem_size, uint32_t batch, uint32_t h, uint32_t w, void *dst,
                   void *stream);
 
+/* Tensor::pad and Tensor::unpad on 4-D row-major data (tt_eager/tensor/tensor.cpp:204-260 -> tt_eager/tensor/tensor_impl.hpp:508-578
+ * pad<T>, :609-660 unpad<T>), and for block-float tensors pad_bfloat8_b / unpad_bfloat8_b / pad_bfloat4_b / unpad_bfloat4_b
+ * (tt_eager/tensor/tensor_impl.cpp:200-283: unpack the sequential 1024-element chunks, pad or unpad as fp32, pack again),
+ * in one pass:  dst[i0,i1,i2,i3] = src[i0-o0, i1-o1, i2-o2, i3-o3] where that index lies inside src, `fill` elsewhere.
+ *   pad    offset = input_tensor_start, dst_shape = output_tensor_shape, fill = pad_value
+ *   unpad  offset = -output_tensor_start, dst_shape = output_tensor_end - output_tensor_start + 1
+ * dtype: TTMI_FLOAT32 | TTMI_UINT32 | TTMI_BFLOAT16 | TTMI_UINT16 (dense elements; fill is converted as static_cast<T>
+ * does in the reference: a bfloat16 keeps the upper 16 bits of the float), or TTMI_BFLOAT8_B | TTMI_BFLOAT4_B (src and dst
+ * are packed words of tensors declared ROW_MAJOR; both volumes must be multiples of 1024, both pointers 16-byte aligned). */
+TTMI_API int ttmi_copy_window(int dtype, const void *src, const uint32_t src_shape[4], void *dst, const uint32_t dst_shape[4],
+                     const int32_t offset[4], float fill, void *stream);
+
+/* tt::tt_metal::unpad on a device tensor in TILE layout (tt_eager/tt_dnn/op_library/unpad/unpad_op.hpp:14-40, the op behind
+ * ttnn.Tensor.__getitem__, ttnn/ttnn/operations/core.py:99-108): start and end are tile-aligned there
+ * (unpad_op.cpp validate), so whole tiles move and a block-float tensor keeps its codes.
+ * src: tiles of a tensor whose tile grid is src_tiles = [N, C, H/32, W/32] (tile (n, c, r, q) at ((n*C + c)*Ht + r)*Wt + q);
+ * dst: the dst_tiles grid that starts at start_tile.  dtype gives the tile size. */
+TTMI_API int ttmi_unpad_tiles(int dtype, const void *src, const uint32_t src_tiles[4], void *dst, const uint32_t start_tile[4],
+                     const uint32_t dst_tiles[4], void *stream);
+
 /* Bytes of scratch ttmi_matmul_bfp wants for these sizes (0 when none).  No reference counterpart: the
  * reference's op allocates its circular buffers inside the program factory
  * (tt_eager/tt_dnn/op_library/bmm/multi_core_reuse_mcast_1d_optimized/bmm_op_multi_core_reuse_mcast_1d_optimized.cpp:48-52). */

@@ -17,7 +17,8 @@
  * test_bfp4_conversion.cpp, an independent floating-point formulation of
  * the quantiser, brute force over every (exponent, shared exponent) pair and
  * every code x exponent for the unpackers, and the tilize permutation closed
- * form.  The matmul gold loop is pinned against numpy float64.
+ * form.  The matmul gold loop is pinned against numpy float64; pad / unpad
+ * against numpy.pad and numpy slicing of the unpacked values.
  */
 #include <stdint.h>
 #include <stddef.h>
@@ -318,6 +319,103 @@ ORACLE_API int oracle_to_torch_bfp_tiles(int fmt, const uint32_t *words, uint32_
         rc = 0;
     }
     free(faces); free(rows); free(again);
+    return rc;
+}
+
+/* tt_eager/tensor/tensor_impl.hpp:508-578 pad<T> on a 4-D row-major tensor: the output is written front to back, runs of
+ * pad_value in front of and behind the input along every dimension, the input rows in between.  elem = bytes per
+ * element (2 or 4); pad = the pad value already converted to the element type.  Returns -1 when the input does not fit
+ * (the reference's TT_ASSERTs, :522-525). */
+ORACLE_API int oracle_pad_rowmajor(const void *src, uint32_t elem, const uint32_t in_shape[4], const uint32_t out_shape[4],
+                                   const uint32_t start[4], const void *pad, void *dst) {
+    for (int d = 0; d < 4; ++d)
+        if ((uint64_t)in_shape[d] + start[d] > out_shape[d]) return -1;
+    uint32_t pad_size[4][2];
+    for (int d = 0; d < 4; ++d) { pad_size[d][0] = start[d]; pad_size[d][1] = out_shape[d] - in_shape[d] - start[d]; }
+    const size_t out_strides[4] = {(size_t)out_shape[1] * out_shape[2] * out_shape[3], (size_t)out_shape[2] * out_shape[3], out_shape[3], 1};
+    const size_t in_strides[4] = {(size_t)in_shape[1] * in_shape[2] * in_shape[3], (size_t)in_shape[2] * in_shape[3], in_shape[3], 1};
+    uint8_t *out = (uint8_t *)dst;
+    const uint8_t *in = (const uint8_t *)src;
+    size_t o = 0;
+#define ORACLE_FILL(count) for (size_t i_ = 0; i_ < (count); ++i_) memcpy(out + (o++) * elem, pad, elem)
+    ORACLE_FILL(pad_size[0][0] * out_strides[0]);
+    for (uint32_t d0 = 0; d0 < in_shape[0]; ++d0) {
+        ORACLE_FILL(pad_size[1][0] * out_strides[1]);
+        for (uint32_t d1 = 0; d1 < in_shape[1]; ++d1) {
+            ORACLE_FILL(pad_size[2][0] * out_strides[2]);
+            for (uint32_t d2 = 0; d2 < in_shape[2]; ++d2) {
+                ORACLE_FILL(pad_size[3][0] * out_strides[3]);
+                for (uint32_t d3 = 0; d3 < in_shape[3]; ++d3) {
+                    const size_t i = d3 + in_strides[2] * d2 + in_strides[1] * d1 + in_strides[0] * d0;
+                    memcpy(out + (o++) * elem, in + i * elem, elem);
+                }
+                ORACLE_FILL(pad_size[3][1] * out_strides[3]);
+            }
+            ORACLE_FILL(pad_size[2][1] * out_strides[2]);
+        }
+        ORACLE_FILL(pad_size[1][1] * out_strides[1]);
+    }
+    ORACLE_FILL(pad_size[0][1] * out_strides[0]);
+#undef ORACLE_FILL
+    return 0;
+}
+
+/* tensor_impl.hpp:609-660 unpad<T>: the elements start..end (inclusive, every dimension) in row-major order. */
+ORACLE_API int oracle_unpad_rowmajor(const void *src, uint32_t elem, const uint32_t in_shape[4], const uint32_t start[4],
+                                     const uint32_t end[4], void *dst) {
+    for (int d = 0; d < 4; ++d)
+        if (start[d] >= in_shape[d] || end[d] >= in_shape[d] || start[d] > end[d]) return -1;
+    const size_t in_strides[4] = {(size_t)in_shape[1] * in_shape[2] * in_shape[3], (size_t)in_shape[2] * in_shape[3], in_shape[3], 1};
+    uint8_t *out = (uint8_t *)dst;
+    const uint8_t *in = (const uint8_t *)src;
+    size_t o = 0;
+    for (uint32_t d0 = start[0]; d0 <= end[0]; ++d0)
+        for (uint32_t d1 = start[1]; d1 <= end[1]; ++d1)
+            for (uint32_t d2 = start[2]; d2 <= end[2]; ++d2)
+                for (uint32_t d3 = start[3]; d3 <= end[3]; ++d3) {
+                    const size_t i = d3 + in_strides[2] * d2 + in_strides[1] * d1 + in_strides[0] * d0;
+                    memcpy(out + (o++) * elem, in + i * elem, elem);
+                }
+    return 0;
+}
+
+/* tt_eager/tensor/tensor_impl.cpp:200-215 pad_bfloat8_b (and :248-263 pad_bfloat4_b): unpack the sequential 1024-element
+ * chunks to fp32, pad as a row-major fp32 tensor, pack sequentially again.  Both volumes must be whole chunks.
+ * words_out: out volume / 1024 tiles.  Returns -1 on a shape error or when memory runs out. */
+ORACLE_API int oracle_pad_bfp(int fmt, const uint32_t *words, const uint32_t in_shape[4], const uint32_t out_shape[4],
+                              const uint32_t start[4], float pad_value, uint32_t *words_out) {
+    const size_t in_vol = (size_t)in_shape[0] * in_shape[1] * in_shape[2] * in_shape[3];
+    const size_t out_vol = (size_t)out_shape[0] * out_shape[1] * out_shape[2] * out_shape[3];
+    if (in_vol % 1024 || out_vol % 1024) return -1;
+    float *in_f = (float *)malloc(in_vol * 4 + 4), *out_f = (float *)malloc(out_vol * 4 + 4);
+    int rc = -1;
+    if (in_f && out_f) {
+        oracle_unpack_bfp_tiles_into_float_vec(fmt, words, in_vol / 1024, 0, in_f);
+        rc = oracle_pad_rowmajor(in_f, 4, in_shape, out_shape, start, &pad_value, out_f);
+        if (rc == 0) oracle_pack_fp32_vec_as_bfp_tiles(fmt, out_f, out_vol / 1024, 0, words_out);
+    }
+    free(in_f); free(out_f);
+    return rc;
+}
+
+/* tensor_impl.cpp:217-230 unpad_bfloat8_b (and :265-280 unpad_bfloat4_b): the same with unpad in the middle. */
+ORACLE_API int oracle_unpad_bfp(int fmt, const uint32_t *words, const uint32_t in_shape[4], const uint32_t start[4],
+                                const uint32_t end[4], uint32_t *words_out) {
+    const size_t in_vol = (size_t)in_shape[0] * in_shape[1] * in_shape[2] * in_shape[3];
+    size_t out_vol = 1;
+    for (int d = 0; d < 4; ++d) {
+        if (start[d] >= in_shape[d] || end[d] >= in_shape[d] || start[d] > end[d]) return -1;
+        out_vol *= (size_t)end[d] - start[d] + 1;
+    }
+    if (in_vol % 1024 || out_vol % 1024) return -1;
+    float *in_f = (float *)malloc(in_vol * 4 + 4), *out_f = (float *)malloc(out_vol * 4 + 4);
+    int rc = -1;
+    if (in_f && out_f) {
+        oracle_unpack_bfp_tiles_into_float_vec(fmt, words, in_vol / 1024, 0, in_f);
+        rc = oracle_unpad_rowmajor(in_f, 4, in_shape, start, end, out_f);
+        if (rc == 0) oracle_pack_fp32_vec_as_bfp_tiles(fmt, out_f, out_vol / 1024, 0, words_out);
+    }
+    free(in_f); free(out_f);
     return rc;
 }
 

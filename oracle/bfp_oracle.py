@@ -59,6 +59,14 @@ def lib() -> ctypes.CDLL:
         for name in ("oracle_from_torch_bfp_tiles", "oracle_to_torch_bfp_tiles"):
             getattr(L, name).restype = i32
             getattr(L, name).argtypes = [i32, vp, u32, u32, u32, vp]
+        L.oracle_pad_rowmajor.restype = i32
+        L.oracle_pad_rowmajor.argtypes = [vp, u32, vp, vp, vp, vp, vp]
+        L.oracle_unpad_rowmajor.restype = i32
+        L.oracle_unpad_rowmajor.argtypes = [vp, u32, vp, vp, vp, vp]
+        L.oracle_pad_bfp.restype = i32
+        L.oracle_pad_bfp.argtypes = [i32, vp, vp, vp, vp, ctypes.c_float, vp]
+        L.oracle_unpad_bfp.restype = i32
+        L.oracle_unpad_bfp.argtypes = [i32, vp, vp, vp, vp, vp]
         L.oracle_bf16_truncate.restype = ctypes.c_uint16
         L.oracle_bf16_truncate.argtypes = [ctypes.c_float]
         L.oracle_gold_bmm.restype = None
@@ -167,6 +175,54 @@ def to_torch_bfp_tiles(fmt: int, words, shape) -> np.ndarray:
     out = np.empty(shape, dtype=np.float32)
     if lib().oracle_to_torch_bfp_tiles(fmt, _ptr(wds), batch, h, w, _ptr(out)) != 0:
         raise MemoryError
+    return out
+
+
+def _shape4(shape) -> np.ndarray:
+    shape = tuple(int(x) for x in shape)
+    assert len(shape) == 4, "pad / unpad work on 4-D shapes (tt_eager/tensor/tensor_impl.hpp:508-660)"
+    return np.array(shape, dtype=np.uint32)
+
+
+def pad_rowmajor(x: np.ndarray, output_shape, input_start, pad_value) -> np.ndarray:
+    """Tensor::pad of a 4-D row-major array with 2- or 4-byte elements; pad_value is converted by numpy to x's dtype."""
+    x = np.ascontiguousarray(x)
+    out = np.empty(tuple(int(v) for v in output_shape), dtype=x.dtype)
+    pad = np.array([pad_value], dtype=x.dtype)
+    in_s, out_s, at = _shape4(x.shape), _shape4(output_shape), _shape4(input_start)      # kept alive across the call
+    if lib().oracle_pad_rowmajor(_ptr(x), x.dtype.itemsize, _ptr(in_s), _ptr(out_s), _ptr(at), _ptr(pad), _ptr(out)) != 0:
+        raise RuntimeError("pad: the input does not fit into the output at that position")
+    return out
+
+
+def unpad_rowmajor(x: np.ndarray, start, end) -> np.ndarray:
+    """Tensor::unpad: elements start..end (inclusive) of a 4-D row-major array."""
+    x = np.ascontiguousarray(x)
+    out = np.empty(tuple(int(e) - int(s) + 1 for s, e in zip(start, end)), dtype=x.dtype)
+    in_s, lo, hi = _shape4(x.shape), _shape4(start), _shape4(end)
+    if lib().oracle_unpad_rowmajor(_ptr(x), x.dtype.itemsize, _ptr(in_s), _ptr(lo), _ptr(hi), _ptr(out)) != 0:
+        raise RuntimeError("unpad: start / end outside the tensor")
+    return out
+
+
+def pad_bfp(fmt: int, words, input_shape, output_shape, input_start, pad_value: float) -> np.ndarray:
+    """pad_bfloat8_b / pad_bfloat4_b: words of a block-float tensor declared ROW_MAJOR (sequential 1024-chunks)."""
+    w = _c(words, np.uint32).reshape(-1)
+    out_vol = int(np.prod(_shape4(output_shape), dtype=np.int64))
+    out = np.empty(out_vol // 1024 * TILE_WORDS[fmt], dtype=np.uint32)
+    in_s, out_s, at = _shape4(input_shape), _shape4(output_shape), _shape4(input_start)
+    if lib().oracle_pad_bfp(fmt, _ptr(w), _ptr(in_s), _ptr(out_s), _ptr(at), float(pad_value), _ptr(out)) != 0:
+        raise RuntimeError("pad: shapes must hold whole 1024-element chunks and the input must fit")
+    return out
+
+
+def unpad_bfp(fmt: int, words, input_shape, start, end) -> np.ndarray:
+    w = _c(words, np.uint32).reshape(-1)
+    out_vol = int(np.prod([int(e) - int(s) + 1 for s, e in zip(start, end)], dtype=np.int64))
+    out = np.empty(max(out_vol // 1024, 0) * TILE_WORDS[fmt], dtype=np.uint32)
+    in_s, lo, hi = _shape4(input_shape), _shape4(start), _shape4(end)
+    if lib().oracle_unpad_bfp(fmt, _ptr(w), _ptr(in_s), _ptr(lo), _ptr(hi), _ptr(out)) != 0:
+        raise RuntimeError("unpad: shapes must hold whole 1024-element chunks and start / end must lie inside the tensor")
     return out
 
 

@@ -131,62 +131,63 @@ def test_as_tensor_with_cache(tmp_path, device):
 
 
 # ---- MLP blocks -------------------------------------------------------------------------------------------------------
-def falcon_reference(x, w1, w2):
-    h = bf16_round(torch.nn.functional.gelu(x @ w1))
-    return h @ w2
+# The decode MLPs of the two models, issued op by op on the mirrored API; what is checked against is the torch functional
+# model of tests/ttnn/integration_tests/falcon7b/test_falcon_mlp.py:17-44 (and its Mistral counterpart), evaluated in fp64.
+def weight_on_device(ttnn, device, linear_weight, dtype, cache_file_name=None):
+    """torch.nn.Linear weight [out, in] -> [1, 1, in, out] block-float tiles on the device (through a weight cache file when named)."""
+    return ttnn.as_tensor(linear_weight.t().contiguous()[None, None], dtype=dtype, layout=ttnn.TILE_LAYOUT, device=device,
+                          cache_file_name=cache_file_name)
+
+
+def falcon_mlp_on_device(tt_lib, x, w_up, w_down):
+    gelu = [tt_lib.tensor.FusibleActivation.GELU, True]
+    return tt_lib.tensor.falcon_dense_4h_to_h_matmul(tt_lib.tensor.falcon_dense_h_to_4h_matmul(x, w_up, fused_activation=gelu), w_down)
+
+
+def mistral_mlp_on_device(ttnn, x, w_gate, w_up, w_down):
+    return ttnn.linear(ttnn.mul(ttnn.linear(x, w_gate, activation="silu"), ttnn.linear(x, w_up)), w_down)
 
 
 @pytest.mark.parametrize("seq,hidden", [(32, 128), (128, 256), (32, 4544)])
 def test_falcon_mlp_block(oracle, device, tmp_path, seq, hidden):
     import tt_lib
     import ttnn
-    from blocks import TtFalconMLP, falcon_mlp_model_config
 
     torch.manual_seed(0)
-    state = {"transformer.h.0.mlp.dense_h_to_4h.weight": torch.randn(4 * hidden, hidden) * 0.02,
-             "transformer.h.0.mlp.dense_4h_to_h.weight": torch.randn(hidden, 4 * hidden) * 0.02}
+    up, down = torch.randn(4 * hidden, hidden) * 0.02, torch.randn(hidden, 4 * hidden) * 0.02
     x = ((torch.rand(1, 1, seq, hidden) * 2) - 1).to(torch.bfloat16)
     cache = tmp_path if hidden <= 256 else None
-    block = TtFalconMLP([device], state, "transformer.h", 0, hidden, falcon_mlp_model_config(), tt_cache_path=cache)
-    assert block.dense_h_to_4h_weights[0].dtype == tt_lib.tensor.DataType.BFLOAT8_B
-    tx = ttnn.from_torch(x, dtype=ttnn.bfloat16, layout=ttnn.TILE_LAYOUT, device=device)
-    out = block([tx])[0]
+    w_up = weight_on_device(ttnn, device, up, ttnn.bfloat8_b, cache and cache / "up")
+    w_down = weight_on_device(ttnn, device, down, ttnn.bfloat8_b, cache and cache / "down")
+    assert w_up.dtype == tt_lib.tensor.DataType.BFLOAT8_B
+    out = falcon_mlp_on_device(tt_lib, ttnn.from_torch(x, dtype=ttnn.bfloat16, layout=ttnn.TILE_LAYOUT, device=device), w_up, w_down)
     assert tuple(out.shape) == (1, 1, seq, hidden) and out.dtype == ttnn.bfloat16
     got = ttnn.to_torch(out)[0, 0]
-    w1 = state["transformer.h.0.mlp.dense_h_to_4h.weight"].t()
-    w2 = state["transformer.h.0.mlp.dense_4h_to_h.weight"].t()
-    want_q = falcon_reference(x[0, 0].double(), quantised(oracle, ttnn.bfloat8_b, w1), quantised(oracle, ttnn.bfloat8_b, w2))
-    assert pcc(got, want_q) >= 0.9999
-    want = torch.nn.functional.gelu(x[0, 0].float() @ w1) @ w2         # torch_functional_falcon_mlp with unquantised weights
-    assert pcc(got, want) >= 0.99
-    if cache is not None:                                              # a second block reads the cached tensor files
-        again = TtFalconMLP([device], {k: torch.zeros_like(v) for k, v in state.items()}, "transformer.h", 0, hidden,
-                            falcon_mlp_model_config(), tt_cache_path=cache)
-        assert torch.equal(again.dense_4h_to_h_weights[0]._buf, block.dense_4h_to_h_weights[0]._buf)
+    hidden_act = bf16_round(torch.nn.functional.gelu(x[0, 0].double() @ quantised(oracle, ttnn.bfloat8_b, up.t())))
+    assert pcc(got, hidden_act @ quantised(oracle, ttnn.bfloat8_b, down.t())) >= 0.9999
+    assert pcc(got, torch.nn.functional.gelu(x[0, 0].float() @ up.t()) @ down.t()) >= 0.99      # unquantised weights
+    if cache is not None:                                              # a second conversion reads the cached tensor file
+        again = weight_on_device(ttnn, device, torch.zeros_like(down), ttnn.bfloat8_b, cache / "down")
+        assert torch.equal(again._buf, w_down._buf)
 
 
 @pytest.mark.parametrize("seq,dim,hidden_dim,name", [(32, 128, 352, "bfloat8_b"), (64, 256, 704, "bfloat4_b"), (32, 4096, 14336, "bfloat4_b")])
 def test_mistral_mlp_block(oracle, device, seq, dim, hidden_dim, name):
     import ttnn
-    from blocks import TtMistralMLP, mistral_mlp_model_config
 
     dtype = getattr(ttnn, name)
     torch.manual_seed(1)
-    state = {"layers.0.feed_forward.w1.weight": torch.randn(hidden_dim, dim) * 0.02,
-             "layers.0.feed_forward.w2.weight": torch.randn(dim, hidden_dim) * 0.02,
-             "layers.0.feed_forward.w3.weight": torch.randn(hidden_dim, dim) * 0.02}
+    gate, up, down = torch.randn(hidden_dim, dim) * 0.02, torch.randn(hidden_dim, dim) * 0.02, torch.randn(dim, hidden_dim) * 0.02
     x = torch.randn(1, 1, seq, dim).to(torch.bfloat16)
-    block = TtMistralMLP(device, None, state, None, 0, dtype, mistral_mlp_model_config())
-    out = block(ttnn.from_torch(x, dtype=ttnn.bfloat16, layout=ttnn.TILE_LAYOUT, device=device))
+    out = mistral_mlp_on_device(ttnn, ttnn.from_torch(x, dtype=ttnn.bfloat16, layout=ttnn.TILE_LAYOUT, device=device),
+                                *(weight_on_device(ttnn, device, w, dtype) for w in (gate, up, down)))
     assert tuple(out.shape) == (1, 1, seq, dim)
     got = ttnn.to_torch(out)[0, 0]
-    w1, w2, w3 = (state[f"layers.0.feed_forward.{n}.weight"].t() for n in ("w1", "w2", "w3"))
     xd = x[0, 0].double()
-    gate = bf16_round(torch.nn.functional.silu(xd @ quantised(oracle, dtype, w1)))
-    up = bf16_round(xd @ quantised(oracle, dtype, w3))
-    want_q = bf16_round(gate * up) @ quantised(oracle, dtype, w2)
+    gated = bf16_round(torch.nn.functional.silu(xd @ quantised(oracle, dtype, gate.t())))
+    want_q = bf16_round(gated * bf16_round(xd @ quantised(oracle, dtype, up.t()))) @ quantised(oracle, dtype, down.t())
     assert pcc(got, want_q) >= 0.9999
-    want = (torch.nn.functional.silu(x[0, 0].float() @ w1) * (x[0, 0].float() @ w3)) @ w2
+    want = (torch.nn.functional.silu(x[0, 0].float() @ gate.t()) * (x[0, 0].float() @ up.t())) @ down.t()
     assert pcc(got, want) >= (0.99 if name == "bfloat8_b" else 0.95)   # 3-bit mantissas: the quantisation itself costs that much
 
 

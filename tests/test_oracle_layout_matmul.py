@@ -92,3 +92,48 @@ def test_gold_bmm_exact_on_small_integers_and_close_to_float64(oracle):
     bound = k * 2.0 ** -24 * np.matmul(np.abs(a).astype(np.float64), np.abs(b).astype(np.float64))
     assert np.all(np.abs(f - exact) <= bound + 1e-30)
     assert np.array_equal(oracle.matmul_reference(a[0], b[0]), exact[0].astype(np.float32))
+
+
+# ---- pad / unpad (tt_eager/tensor/tensor_impl.hpp:508-660, tensor_impl.cpp:200-283) -------------------------------------
+@pytest.mark.parametrize("dtype", [np.float32, np.uint16, np.uint32])
+def test_pad_and_unpad_rowmajor_are_numpy_pad_and_slicing(oracle, dtype):
+    """The reference writes the output front to back with runs of the pad value; numpy.pad and basic slicing state the same
+    result without any of its index arithmetic (a wrong stride, a swapped front / back pad or an off-by-one end fails here)."""
+    rng = np.random.default_rng(5)
+    x = rng.integers(1, 60000, size=(2, 3, 5, 7)).astype(dtype)
+    out_shape, start = (4, 5, 9, 16), (1, 2, 3, 4)
+    want = np.pad(x, [(s, o - s - i) for s, o, i in zip(start, out_shape, x.shape)], constant_values=dtype(9))
+    assert np.array_equal(oracle.pad_rowmajor(x, out_shape, start, 9), want)
+    assert np.array_equal(oracle.pad_rowmajor(x, x.shape, (0, 0, 0, 0), 9), x)
+    lo, hi = (1, 0, 2, 3), (1, 2, 4, 6)
+    assert np.array_equal(oracle.unpad_rowmajor(x, lo, hi), x[1:2, 0:3, 2:5, 3:7])
+    assert np.array_equal(oracle.unpad_rowmajor(want, start, tuple(s + i - 1 for s, i in zip(start, x.shape))), x)   # unpad inverts pad
+    with pytest.raises(RuntimeError):
+        oracle.pad_rowmajor(x, (2, 3, 5, 7), (0, 0, 0, 1), 0)
+    with pytest.raises(RuntimeError):
+        oracle.unpad_rowmajor(x, (0, 0, 0, 0), (1, 2, 4, 7))
+
+
+@pytest.mark.parametrize("fmt", [3, 4])
+def test_pad_and_unpad_block_float_requantise_the_moved_values(oracle, fmt):
+    """pad_bfloat8_b / unpad_bfloat8_b: unpack -> fp32 pad / unpad -> pack.  Checked against numpy.pad / slicing of the
+    unpacked values followed by one sequential pack; and, where the window keeps every 16-element run intact, against the
+    source's own codes (nothing is re-quantised when a run moves as a whole)."""
+    rng = np.random.default_rng(6)
+    shape = (1, 2, 32, 64)
+    x = (rng.standard_normal(shape) * np.exp2(rng.integers(-6, 6, size=shape))).astype(np.float32)
+    words = oracle.pack_fp32_vec_as_bfp_tiles(fmt, x.reshape(-1), False)
+    values = oracle.unpack_bfp_tiles_into_float_vec(fmt, words, False).reshape(shape)
+    out_shape, start = (2, 2, 64, 96), (1, 0, 16, 16)
+    padded = np.pad(values, [(s, o - s - i) for s, o, i in zip(start, out_shape, shape)], constant_values=np.float32(0.5))
+    got = oracle.pad_bfp(fmt, words, shape, out_shape, start, 0.5)
+    assert np.array_equal(got, oracle.pack_fp32_vec_as_bfp_tiles(fmt, padded.reshape(-1), False))
+    # every run of 16 stays whole here (offsets are multiples of 16), so unpacking gives back exactly the padded values
+    assert np.array_equal(oracle.unpack_bfp_tiles_into_float_vec(fmt, got, False).reshape(out_shape), padded)
+    lo, hi = (0, 1, 3, 5), (0, 1, 18, 36)                                   # 16 x 32 values = half a chunk: rejected
+    with pytest.raises(RuntimeError):
+        oracle.unpad_bfp(fmt, words, shape, lo, hi)
+    lo, hi = (0, 0, 3, 5), (0, 1, 18, 36)                                   # 2 x 16 x 32 = one chunk, runs cut at column 5
+    cut = oracle.unpad_bfp(fmt, words, shape, lo, hi)
+    assert np.array_equal(cut, oracle.pack_fp32_vec_as_bfp_tiles(fmt, values[0:1, 0:2, 3:19, 5:37].reshape(-1), False))
+    assert cut.size == oracle.TILE_WORDS[fmt]

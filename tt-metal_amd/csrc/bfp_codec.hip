@@ -14,6 +14,7 @@
 //   packed tiles are assembled in LDS and leave (or enter) the block as one contiguous run of 16-byte accesses.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <string.h>
 
 #include "ttmi_internal.h"
 
@@ -403,8 +404,141 @@ __global__ __launch_bounds__(256) void relayout_kernel(const uint8_t *__restrict
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// pad / unpad of 4-D row-major data: dst[i] = src[i - offset] where that lies inside src, a fill value elsewhere
+// (tt_eager/tensor/tensor_impl.hpp:508-578 pad, :609-660 unpad: offset = input_tensor_start, or minus output_tensor_start).
+// ---------------------------------------------------------------------------------------------------------
+struct WindowDev { uint32_t src[4], dst[4]; int32_t off[4]; };
+
+// flat source index of flat destination index `o`, or -1 outside the source
+__device__ __forceinline__ int64_t window_source(const WindowDev &w, uint64_t o) {
+    int64_t at = 0;
+    uint64_t stride = 1;
+    bool inside = true;
+#pragma unroll
+    for (int d = 3; d >= 0; --d) {
+        const int64_t c = (int64_t)(o % w.dst[d]) - w.off[d];
+        o /= w.dst[d];
+        inside = inside && c >= 0 && c < (int64_t)w.src[d];
+        at += c * (int64_t)stride;
+        stride *= w.src[d];
+    }
+    return inside ? at : -1;
+}
+
+// an element is `inner` consecutive values of T (1 for scalars; the 32-bit words of a tile when whole tiles are moved)
+template <typename T>
+__global__ __launch_bounds__(256) void window_copy_kernel(const T *__restrict__ src, T *__restrict__ dst, const WindowDev w, T fill, uint32_t inner,
+                                                          uint64_t total) {
+    for (uint64_t o = (uint64_t)blockIdx.x * 256 + threadIdx.x; o < total; o += (uint64_t)gridDim.x * 256) {
+        const uint64_t elem = inner == 1 ? o : o / inner;
+        const int64_t i = window_source(w, elem);
+        dst[o] = i >= 0 ? src[(uint64_t)i * inner + (o - elem * inner)] : fill;
+    }
+}
+
+// The same for block-float tensors declared ROW_MAJOR (consecutive 1024-element chunks of the row-major data, packed in
+// sequence: tt_eager/tt_lib/csrc/tt_lib_bindings_tensor_pytensor.cpp:145-151), as tensor_impl.cpp:200-283 does it — unpack
+// to fp32, pad / unpad, pack again — in one pass: a thread owns one run of 16 output elements (one shared exponent),
+// decodes the source codes under it and encodes the run.
+template <int W>
+__global__ __launch_bounds__(256) void window_copy_bfp_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, const WindowDev w,
+                                                              uint32_t fill_bits, uint64_t runs) {
+    using F = Fmt<W>;
+    for (uint64_t r = (uint64_t)blockIdx.x * 256 + threadIdx.x; r < runs; r += (uint64_t)gridDim.x * 256) {
+        uint32_t bits[16], shared = 0;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int64_t i = window_source(w, r * 16 + e);
+            uint32_t v = fill_bits;
+            if (i >= 0) {
+                const uint8_t *tile = src + (uint64_t)(i >> 10) * F::tile_bytes;
+                const uint32_t at = (uint32_t)i & 1023u;
+                const uint32_t code = W == 7 ? tile[64 + at] : (tile[64 + (at >> 1)] >> (4 * (at & 1))) & 0xfu;
+                v = from_code<W>(code, tile[at >> 4]);
+            }
+            bits[e] = v;
+            shared = max(shared, (v >> 23) & 0xffu);
+        }
+        uint8_t *tile = dst + (r >> 6) * F::tile_bytes;
+        const uint32_t k = (uint32_t)r & 63u;
+        tile[k] = (uint8_t)shared;
+        uint32_t out[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t code = to_code<W>(bits[e], shared);
+            if (W == 7) out[e >> 2] |= code << (8 * (e & 3));
+            else out[e >> 3] |= code << (4 * (e & 7));
+        }
+        if (W == 7) *reinterpret_cast<uint4 *>(tile + 64 + k * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+        else *reinterpret_cast<uint2 *>(tile + 64 + k * 8) = make_uint2(out[0], out[1]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // host launchers
 // ---------------------------------------------------------------------------------------------------------
+int codec_copy_window(int dtype, const void *src, const uint32_t src_shape[4], void *dst, const uint32_t dst_shape[4],
+                      const int32_t offset[4], float fill, hipStream_t st) {
+    WindowDev w{};
+    uint64_t total = 1, src_total = 1;
+    for (int d = 0; d < 4; ++d) {
+        w.src[d] = src_shape[d]; w.dst[d] = dst_shape[d]; w.off[d] = offset[d];
+        total *= dst_shape[d]; src_total *= src_shape[d];
+    }
+    if (total == 0) return TTMI_OK;
+    if (total >> 40 || src_total >> 40) return fail(TTMI_ERR_INVALID_ARGUMENT, "pad / unpad: tensor too large");
+    uint32_t fill_bits;
+    memcpy(&fill_bits, &fill, 4);
+    const bool bfp = dtype == TTMI_BFLOAT8_B || dtype == TTMI_BFLOAT4_B;
+    const uint64_t items = bfp ? total / 16 : total;
+    const uint32_t blocks = (uint32_t)((items + 255) / 256 < 256 * 32 ? (items + 255) / 256 : 256 * 32);
+    switch (dtype) {
+        case TTMI_BFLOAT8_B: case TTMI_BFLOAT4_B:
+            // whole chunks on both sides (the reference's packers assert it: tt_metal/common/bfloat8.hpp:107)
+            if (total % 1024 || src_total % 1024)
+                return fail(TTMI_ERR_INVALID_ARGUMENT, "pad / unpad: a block-float tensor holds whole 1024-element chunks (%llu -> %llu elements)",
+                            (unsigned long long)src_total, (unsigned long long)total);
+            if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u)
+                return fail(TTMI_ERR_INVALID_ARGUMENT, "pad / unpad: src and dst must be 16-byte aligned");
+            if (dtype == TTMI_BFLOAT8_B) hipLaunchKernelGGL((window_copy_bfp_kernel<7>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, w, fill_bits, items);
+            else hipLaunchKernelGGL((window_copy_bfp_kernel<3>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, w, fill_bits, items);
+            break;
+        case TTMI_FLOAT32:
+            hipLaunchKernelGGL((window_copy_kernel<uint32_t>), dim3(blocks), dim3(256), 0, st, (const uint32_t *)src, (uint32_t *)dst, w, fill_bits, 1u, items);
+            break;
+        case TTMI_UINT32:
+            hipLaunchKernelGGL((window_copy_kernel<uint32_t>), dim3(blocks), dim3(256), 0, st, (const uint32_t *)src, (uint32_t *)dst, w, (uint32_t)fill, 1u, items);
+            break;
+        case TTMI_BFLOAT16:      // static_cast<bfloat16>(float) keeps the upper 16 bits (tt_metal/common/bfloat16.hpp:28-38)
+            hipLaunchKernelGGL((window_copy_kernel<uint16_t>), dim3(blocks), dim3(256), 0, st, (const uint16_t *)src, (uint16_t *)dst, w, (uint16_t)(fill_bits >> 16), 1u, items);
+            break;
+        case TTMI_UINT16:
+            hipLaunchKernelGGL((window_copy_kernel<uint16_t>), dim3(blocks), dim3(256), 0, st, (const uint16_t *)src, (uint16_t *)dst, w, (uint16_t)fill, 1u, items);
+            break;
+        default: return fail(TTMI_ERR_INVALID_ARGUMENT, "pad / unpad: unknown dtype %d", dtype);
+    }
+    return check_launch("window_copy_kernel");
+}
+
+// unpad of a TILE-layout tensor at tile granularity: whole tiles are moved, nothing is decoded
+int codec_unpad_tiles(uint32_t tile_bytes, const void *src, const uint32_t src_tiles[4], void *dst, const uint32_t start[4],
+                      const uint32_t dst_tiles[4], hipStream_t st) {
+    WindowDev w{};
+    uint64_t total = 1;
+    for (int d = 0; d < 4; ++d) {
+        if ((uint64_t)start[d] + dst_tiles[d] > src_tiles[d]) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpad: the range leaves the tensor in dimension %d", d);
+        w.src[d] = src_tiles[d]; w.dst[d] = dst_tiles[d]; w.off[d] = -(int32_t)start[d];
+        total *= dst_tiles[d];
+    }
+    if (total == 0) return TTMI_OK;
+    const uint32_t inner = tile_bytes / 4;
+    const uint64_t items = total * inner;
+    if (items >> 40) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpad: tensor too large");
+    const uint32_t blocks = (uint32_t)((items + 255) / 256 < 256 * 32 ? (items + 255) / 256 : 256 * 32);
+    hipLaunchKernelGGL((window_copy_kernel<uint32_t>), dim3(blocks), dim3(256), 0, st, (const uint32_t *)src, (uint32_t *)dst, w, 0u, inner, items);
+    return check_launch("window_copy_kernel");
+}
+
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <int W, int ELEM, int MODE>

@@ -97,6 +97,24 @@ int ttmi_untilize(const void *src, uint32_t elem_size, uint32_t batch, uint32_t 
     return codec_relayout(false, src, elem_size, batch, h, w, dst, (hipStream_t)stream);
 }
 
+int ttmi_copy_window(int dtype, const void *src, const uint32_t src_shape[4], void *dst, const uint32_t dst_shape[4],
+                     const int32_t offset[4], float fill, void *stream) {
+    if (!src_shape || !dst_shape || !offset) return fail(TTMI_ERR_INVALID_ARGUMENT, "pad / unpad: null shape");
+    uint64_t total = 1, src_total = 1;
+    for (int d = 0; d < 4; ++d) { total *= dst_shape[d]; src_total *= src_shape[d]; }
+    if (total && (!dst || (src_total && !src))) return fail(TTMI_ERR_INVALID_ARGUMENT, "pad / unpad: null pointer");
+    return codec_copy_window(dtype, src, src_shape, dst, dst_shape, offset, fill, (hipStream_t)stream);
+}
+
+int ttmi_unpad_tiles(int dtype, const void *src, const uint32_t src_tiles[4], void *dst, const uint32_t start_tile[4],
+                     const uint32_t dst_tiles[4], void *stream) {
+    const uint32_t tile_bytes = ttmi_tile_size(dtype);
+    if (!tile_bytes) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpad: unknown dtype %d", dtype);
+    if (!src_tiles || !start_tile || !dst_tiles) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpad: null shape");
+    if (!src || !dst) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpad: null pointer");
+    return codec_unpad_tiles(tile_bytes, src, src_tiles, dst, start_tile, dst_tiles, (hipStream_t)stream);
+}
+
 size_t ttmi_matmul_bfp_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt) {
     return matmul_workspace_bytes(batch, m, k, n, b_fmt);
 }

@@ -23,6 +23,12 @@ int codec_unpack_tensor(int fmt, const uint32_t *words, uint32_t batch, uint32_t
 int codec_relayout(bool to_tiles, const void *src, uint32_t elem, uint32_t batch, uint32_t h, uint32_t w, void *dst,
                    hipStream_t st);
 
+int codec_copy_window(int dtype, const void *src, const uint32_t src_shape[4], void *dst, const uint32_t dst_shape[4],
+                      const int32_t offset[4], float fill, hipStream_t st);
+
+int codec_unpad_tiles(uint32_t tile_bytes, const void *src, const uint32_t src_tiles[4], void *dst, const uint32_t start[4],
+                      const uint32_t dst_tiles[4], hipStream_t st);
+
 int eltwise_bf16(int op, const void *a, const void *b, float scalar, void *c, size_t count, hipStream_t st);
 
 struct MatmulArgs {

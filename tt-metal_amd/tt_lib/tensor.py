@@ -251,6 +251,72 @@ class Tensor:
             raise RuntimeError("reshape of a TILE tensor must keep the last two padded dimensions")
         return self._like(buf, shape=logical, padded=padded)
 
+    # ---- pad / unpad on the host (tt_eager/tensor/tensor.cpp:204-260) ----------------------------------------
+    def _window(self, dst_shape, offset, fill, what):
+        """dst[i] = self[i - offset] inside self, `fill` elsewhere: pad<T> / unpad<T> (tensor_impl.hpp:508-660), and for
+        block-float tensors unpack -> fp32 pad / unpad -> pack (tensor_impl.cpp:200-283) in one kernel."""
+        if self._device is not None:
+            raise RuntimeError("TT_THROW: Device storage isn't supported")          # tensor_impl.hpp:590, 675
+        if self._layout != Layout.ROW_MAJOR:
+            raise RuntimeError(f"TT_ASSERT: Tensor layout must be ROW_MAJOR for {what}")
+        if len(self._padded) != 4 or len(dst_shape) != 4:
+            raise RuntimeError(f"{what}: shapes must have rank 4")
+        dst_shape = tuple(int(x) for x in dst_shape)
+        code = int(self._dtype)
+        if self._dtype in _BFP:
+            volume = dst_shape[0] * dst_shape[1] * dst_shape[2] * dst_shape[3]
+            if volume % 1024:
+                raise RuntimeError("TT_ASSERT: fp32_vec.size() % num_float_in_tile == 0 (block-float tensors hold whole tiles)")
+            src = self._buf
+        else:
+            src = self._buf.view(self._padded)
+        return _run_on_gpu(src, lambda d: capi.copy_window(code, d, self._padded, dst_shape, offset, fill))
+
+    def pad(self, output_tensor_shape, input_tensor_start, pad_value: float):
+        """tensor.cpp:204-224: the tensor placed at input_tensor_start inside a tensor of output_tensor_shape filled with pad_value."""
+        out_shape = tuple(int(x) for x in output_tensor_shape)
+        start = tuple(int(x) for x in input_tensor_start)
+        if len(out_shape) != 4 or len(start) != 4 or len(self._padded) != 4:
+            raise RuntimeError("pad: shapes must have rank 4")
+        for i in range(4):
+            if self._padded[i] + start[i] > out_shape[i]:      # tensor_impl.hpp:522-525
+                raise RuntimeError(f"TT_ASSERT: input_tensor_shape[{i}] + input_tensor_start[{i}] <= output_tensor_shape[{i}]")
+        buf = self._window(out_shape, start, float(pad_value), "padding")
+        return self._like(buf, shape=tuple(self._padded), padded=out_shape)
+
+    def unpad(self, output_tensor_start, output_tensor_end):
+        """tensor.cpp:226-230: the elements output_tensor_start..output_tensor_end (inclusive in every dimension)."""
+        start = tuple(int(x) for x in output_tensor_start)
+        end = tuple(int(x) for x in output_tensor_end)
+        if len(start) != 4 or len(end) != 4 or len(self._padded) != 4:
+            raise RuntimeError("unpad: shapes must have rank 4")
+        for i in range(4):                                      # tensor_impl.hpp:614-627
+            if start[i] >= self._padded[i] or end[i] >= self._padded[i] or start[i] > end[i]:
+                raise RuntimeError(f"TT_ASSERT: output_tensor_start[{i}] <= output_tensor_end[{i}] < input_tensor_shape[{i}]")
+        out_shape = tuple(e - b + 1 for b, e in zip(start, end))
+        buf = self._window(out_shape, tuple(-b for b in start), 0.0, "unpadding")
+        return self._like(buf, shape=out_shape, padded=out_shape)
+
+    def pad_to_tile(self, pad_value: float):
+        """tensor.cpp:232-246: height and width rounded up to 32, the tensor in the top left corner."""
+        if len(self._padded) != 4:
+            raise RuntimeError("pad_to_tile: the tensor must have rank 4")
+        n, c, h, w = self._padded
+        return self.pad((n, c, _pad32(h), _pad32(w)), (0, 0, 0, 0), pad_value)
+
+    def unpad_from_tile(self, output_tensor_shape):
+        """tensor.cpp:248-260: the inverse of pad_to_tile for a given logical shape."""
+        out = tuple(int(x) for x in output_tensor_shape)
+        if len(out) != 4 or len(self._padded) != 4:
+            raise RuntimeError("unpad_from_tile: shapes must have rank 4")
+        if self._padded[0] != out[0] or self._padded[1] != out[1]:
+            raise RuntimeError("TT_ASSERT: Input shape must match output shape apart from last 2 dims")
+        if self._padded[2] % 32 or self._padded[3] % 32:
+            raise RuntimeError("TT_ASSERT: Last 2 dims of input shape must be multiples of 32")
+        if not (self._padded[2] - 32 < out[2] <= self._padded[2] and self._padded[3] - 32 < out[3] <= self._padded[3]):
+            raise RuntimeError("TT_ASSERT: Last 2 dims of output must be within range to have been padded to input")
+        return self.unpad((0, 0, 0, 0), tuple(x - 1 for x in out))
+
     def to_torch(self):
         """pytensor.cpp:354-412: block-float comes back as float32 (sequential unpack), others in their own dtype."""
         if self._device is not None:
@@ -347,6 +413,93 @@ def bmm(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConf
         untilize_out: bool = False) -> Tensor:
     """tt_lib.tensor.bmm: [B, C, M, K] x [B, C, K, N] (tt_lib_bindings_tensor_custom_bmm_ops.cpp:66-81, bmm_op.hpp:425)."""
     return _matmul(input_a, input_b, bcast_batch=False, op="bmm")
+
+
+def unpad(input_tensor: Tensor, output_tensor_start, output_tensor_end, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:
+    """tt_lib.tensor.unpad on a device tensor (tt_eager/tt_dnn/op_library/unpad/unpad_op.cpp:95-125): in TILE layout start and
+    extent are whole tiles, so tiles are moved as they are and a block-float tensor keeps its codes."""
+    if input_tensor.storage_type() != StorageType.DEVICE:
+        raise RuntimeError("TT_FATAL: Operands to unpad need to be on device!")
+    padded = tuple(input_tensor._padded)
+    start, end = tuple(int(x) for x in output_tensor_start), tuple(int(x) for x in output_tensor_end)
+    if len(padded) != 4 or len(start) != 4 or len(end) != 4:
+        raise RuntimeError("unpad: shapes must have rank 4")
+    for i in range(4):
+        if start[i] >= padded[i] or end[i] >= padded[i] or start[i] > end[i]:
+            raise RuntimeError(f"TT_FATAL: output_tensor_start[{i}] <= output_tensor_end[{i}] < input shape[{i}]")
+    out_shape = tuple(e - b + 1 for b, e in zip(start, end))
+    with torch.cuda.device(input_tensor._device.torch_device):
+        if input_tensor.layout == Layout.TILE:
+            if out_shape[-2] % 32 or start[-2] % 32 or out_shape[-1] % 32 or start[-1] % 32:
+                raise RuntimeError("TT_FATAL: Can only unpad tilized tensor with full tiles")
+            grid = lambda sh: (sh[0], sh[1], sh[2] // 32, sh[3] // 32)
+            buf = capi.unpad_tiles(int(input_tensor.dtype), input_tensor._buf, grid(padded), grid(start), grid(out_shape))
+        else:
+            if input_tensor.dtype in _BFP:
+                raise RuntimeError("TT_FATAL: block-float tensors on device are in TILE layout")
+            elem = input_tensor._buf.element_size()
+            if (out_shape[-1] * elem) % 4 or (start[-1] * elem) % 4:
+                raise RuntimeError("TT_FATAL: RM unpadding requires output X size to be packable")
+            buf = capi.copy_window(int(input_tensor.dtype), input_tensor._buf.view(padded), padded, out_shape, tuple(-b for b in start))
+    return input_tensor._like(buf, shape=out_shape, padded=out_shape)
+
+
+# ---- the BERT-Large matmuls (bmm_op.cpp:631-742): fixed shapes, otherwise primary::matmul ----------------------------
+def _expect_shape(t: Tensor, shape) -> None:
+    if tuple(t._padded) != tuple(shape):
+        raise RuntimeError(f"TT_FATAL: Unsupported input shape (expected {list(shape)}, got {list(t._padded)})")
+
+
+def bert_large_fused_qkv_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None,
+                                output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:634-651: [B, 1, 384, 1024] x [1, 1, 1024, 3072]."""
+    _expect_shape(input_a, (input_a._padded[0], 1, 384, 1024))
+    _expect_shape(input_b, (1, 1, 1024, 3072))
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, output_dtype=output_dtype, op="bert_large_fused_qkv_matmul")
+
+
+def bert_large_ff1_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None, fused_activation=None,
+                          output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:653-672: [B, 1, 384, 1024] x [1, 1, 1024, 4096], optional fused activation (the L1 / DRAM rule of :656 is
+    about Tensix buffers and has nothing to check here)."""
+    _expect_shape(input_a, (input_a._padded[0], 1, 384, 1024))
+    _expect_shape(input_b, (1, 1, 1024, 4096))
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, activation=_fused_activation_code(fused_activation),
+                   output_dtype=output_dtype, op="bert_large_ff1_matmul")
+
+
+def bert_large_ff2_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None,
+                          output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:674-691: [B, 1, 384, 4096] x [1, 1, 4096, 1024]."""
+    _expect_shape(input_a, (input_a._padded[0], 1, 384, 4096))
+    _expect_shape(input_b, (1, 1, 4096, 1024))
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, output_dtype=output_dtype, op="bert_large_ff2_matmul")
+
+
+def bert_large_selfout_matmul(input_a: Tensor, input_b: Tensor, bias: Optional[Tensor] = None,
+                              output_mem_config: Optional[MemoryConfig] = None, output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:693-710: [B, 1, 384, 1024] x [1, 1, 1024, 1024]."""
+    _expect_shape(input_a, (input_a._padded[0], 1, 384, 1024))
+    _expect_shape(input_b, (1, 1, 1024, 1024))
+    return _matmul(input_a, input_b, bcast_batch=True, bias=bias, output_dtype=output_dtype, op="bert_large_selfout_matmul")
+
+
+def bert_large_pre_softmax_bmm(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None,
+                               output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:712-726: [B, 16, 384, 64] x [B, 16, 64, 384], every slice with its own right operand."""
+    b = input_a._padded[0]
+    _expect_shape(input_a, (b, 16, 384, 64))
+    _expect_shape(input_b, (b, 16, 64, 384))
+    return _matmul(input_a, input_b, bcast_batch=False, output_dtype=output_dtype, op="bert_large_pre_softmax_bmm")
+
+
+def bert_large_post_softmax_bmm(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None,
+                                output_dtype: Optional[DataType] = None) -> Tensor:
+    """bmm_op.cpp:728-742: [B, 16, 384, 384] x [B, 16, 384, 64]."""
+    b = input_a._padded[0]
+    _expect_shape(input_a, (b, 16, 384, 384))
+    _expect_shape(input_b, (b, 16, 384, 64))
+    return _matmul(input_a, input_b, bcast_batch=False, output_dtype=output_dtype, op="bert_large_post_softmax_bmm")
 
 
 # ---- fused activations and the Falcon matmuls (bmm_op.cpp:747-807) -------------------------------------------------

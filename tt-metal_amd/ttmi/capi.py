@@ -23,7 +23,7 @@ SYMBOLS = (
     "ttmi_pack_fp32_vec_as_bfp_tiles", "ttmi_unpack_bfp_tiles_into_float_vec",
     "ttmi_pack_rowmajor_as_bfp_tiles", "ttmi_unpack_bfp_tiles_as_rowmajor",
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
-    "ttmi_eltwise_bf16",
+    "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles",
 )
 
 _lib = None
@@ -62,6 +62,10 @@ def lib() -> ctypes.CDLL:
         L.ttmi_matmul_bfp_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
         L.ttmi_matmul_bfp.restype = i32
         L.ttmi_matmul_bfp.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, sz, vp]
+        L.ttmi_copy_window.restype = i32
+        L.ttmi_copy_window.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(ctypes.c_int32), ctypes.c_float, vp]
+        L.ttmi_unpad_tiles.restype = i32
+        L.ttmi_unpad_tiles.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(u32), vp]
         L.ttmi_eltwise_bf16.restype = i32
         L.ttmi_eltwise_bf16.argtypes = [i32, vp, vp, ctypes.c_float, vp, sz, vp]
         _lib = L
@@ -205,4 +209,38 @@ def eltwise(op: int, a, b=None, scalar: float = 0.0):
     b = b.contiguous() if b is not None else None
     out = torch.empty_like(a)
     check(lib().ttmi_eltwise_bf16(op, _dev(a), _dev(b) if b is not None else None, float(scalar), _dev(out), a.numel(), _stream()))
+    return out
+
+
+def copy_window(dtype: int, src, src_shape, dst_shape, offset, fill: float = 0.0):
+    """Tensor::pad / unpad on a cuda buffer: dst[i] = src[i - offset] inside src, `fill` elsewhere (4-D shapes).
+    Dense dtypes return a tensor of dst_shape; block-float dtypes take and return flat packed words."""
+    import torch
+
+    src_shape = tuple(int(x) for x in src_shape)
+    dst_shape = tuple(int(x) for x in dst_shape)
+    volume = 1
+    for x in dst_shape:
+        volume *= x
+    if dtype in (BFLOAT8_B, BFLOAT4_B):
+        out = torch.empty(volume // 1024 * (TILE_BYTES[dtype] // 4), dtype=src.dtype, device=src.device)
+    else:
+        out = torch.empty(dst_shape, dtype=src.dtype, device=src.device)
+    check(lib().ttmi_copy_window(dtype, _dev(src.contiguous()), (ctypes.c_uint32 * 4)(*src_shape), _dev(out), (ctypes.c_uint32 * 4)(*dst_shape),
+                                 (ctypes.c_int32 * 4)(*[int(x) for x in offset]), float(fill), _stream()))
+    return out
+
+
+def unpad_tiles(dtype: int, tiles, src_tiles, start_tile, dst_tiles):
+    """Whole tiles [start_tile, start_tile + dst_tiles) of a TILE-layout cuda buffer with tile grid src_tiles (4-D)."""
+    import torch
+
+    count = 1
+    for x in dst_tiles:
+        count *= int(x)
+    per_tile = TILE_BYTES[dtype] // tiles.element_size()
+    out = torch.empty(count * per_tile, dtype=tiles.dtype, device=tiles.device)
+    u4 = ctypes.c_uint32 * 4
+    check(lib().ttmi_unpad_tiles(dtype, _dev(tiles.contiguous()), u4(*[int(x) for x in src_tiles]), _dev(out), u4(*[int(x) for x in start_tile]),
+                                 u4(*[int(x) for x in dst_tiles]), _stream()))
     return out
