@@ -50,6 +50,13 @@ enum { TTMI_OP_ADD = 0, TTMI_OP_SUB = 1, TTMI_OP_MUL = 2, TTMI_OP_RELU = 17, TTM
 TTMI_API const char *ttmi_last_error(void);
 TTMI_API const char *ttmi_version(void);
 
+/* What kernels on the current device have reported since the last query: TTMI_OK, or TTMI_ERR_HIP (message in
+ * ttmi_last_error()) when a matmul kernel gave up waiting for another workgroup's partial sums — its output is invalid.
+ * Reads a word of pinned host memory, no synchronisation; the report becomes visible once the kernel has run, and
+ * ttmi_matmul_bfp makes the same check on entry.  The reference learns of a stuck kernel from its watcher thread
+ * (tt_metal/impl/debug/watcher_server.cpp) or never; there is no call of this kind in it. */
+TTMI_API int ttmi_device_status(void);
+
 /* tt_metal/common/tt_backend_api_types.hpp:109-132 tile_size(DataFormat): bytes of one 32x32 tile
  * (1088 bfloat8_b, 576 bfloat4_b, 2048 bfloat16/uint16, 4096 float32/uint32); 0 for an unknown dtype. */
 TTMI_API uint32_t ttmi_tile_size(int dtype);

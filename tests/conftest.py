@@ -19,3 +19,31 @@ def oracle():
 
     bfp_oracle.build()
     return bfp_oracle
+
+
+# knobs of libttmi's test entry point (tt-metal_amd/csrc/ttmi_internal.h: TTMI_KNOB_*)
+KNOB = {"kernel": 0, "workgroups": 1, "block": 2, "spin_limit": 3, "drop_partial_sums": 4}
+KERNEL_CODE = {"stream": 1, "wide": 2, "tile": 3, "expanded": 4}
+
+
+@pytest.fixture
+def knobs():
+    """knobs(name, value) on the library's test entry point (name: kernel = stream | wide | tile | expanded, workgroups,
+    block = 256 | 128 | 4 | 384, spin_limit, drop_partial_sums); everything set is cleared again after the test."""
+    import ctypes
+
+    from ttmi import capi
+
+    L = capi.lib()
+    L.ttmi_test_set_knob.restype = ctypes.c_int
+    L.ttmi_test_set_knob.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_int]
+    touched = []
+
+    def set_knob(name, value):
+        which = KNOB[name]
+        capi.check(L.ttmi_test_set_knob(which, KERNEL_CODE[value] if name == "kernel" else int(value), 1))
+        touched.append(which)
+
+    yield set_knob
+    for which in touched:
+        L.ttmi_test_set_knob(which, 0, 0)

@@ -39,7 +39,7 @@ def test_size_helpers_need_no_gpu():
     assert L.ttmi_tiled_size_bytes(3, 6, 7, 3) == 6 * 1088
 
 
-def test_matmul_workspace_sizes_follow_the_decomposition(monkeypatch):
+def test_matmul_workspace_sizes_follow_the_decomposition():
     """What a caller has to bring for a GEMM of its own stream: 16 KB of partial-sum slots per computing workgroup of the
     128-column kernel (one band of rows), nothing when every output has a workgroup of its own, the expanded weights
     (2 bytes each) from 512 rows on."""
@@ -47,8 +47,6 @@ def test_matmul_workspace_sizes_follow_the_decomposition(monkeypatch):
 
     if not os.path.exists(capi.LIB_PATH):
         pytest.skip("libttmi.so not built")
-    for name in ("TTMI_MATMUL_KERNEL", "TTMI_MATMUL_WGS", "TTMI_MATMUL_BM"):
-        monkeypatch.delenv(name, raising=False)
     ws = capi.lib().ttmi_matmul_bfp_workspace_bytes
     assert ws(1, 32, 4544, 18176, 3) == 142 * 3 * 16384        # 142 groups of 128 columns, 512 // 143 = 3 k ranges each
     assert ws(1, 32, 18176, 4544, 3) == 36 * 7 * 16384         # 36 groups (the last one half empty), 256 // 36 = 7
@@ -85,3 +83,92 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(capi, "LIB_PATH", "/nonexistent/libttmi.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         capi.lib()
+
+
+# ---- host bookkeeping of the streaming GEMM kernels (no GPU) -------------------------------------------------------------
+def _test_entries():
+    from ttmi import capi
+
+    if not os.path.exists(capi.LIB_PATH):
+        pytest.skip("libttmi.so not built")
+    L = capi.lib()
+    u32 = ctypes.c_uint32
+    L.ttmi_test_stream_decomposition.restype = None
+    L.ttmi_test_stream_decomposition.argtypes = [u32, u32, u32, u32, ctypes.c_int, ctypes.POINTER(u32)]
+    L.ttmi_test_range_start.restype = u32
+    L.ttmi_test_range_start.argtypes = [u32, u32, u32]
+    L.ttmi_test_workgroup_of.restype = u32
+    L.ttmi_test_workgroup_of.argtypes = [u32, u32, u32]
+    L.ttmi_test_scratch_grown_size.restype = ctypes.c_size_t
+    L.ttmi_test_scratch_grown_size.argtypes = [ctypes.c_size_t, ctypes.c_size_t]
+    return L
+
+
+SHAPES = [(1, 32, 4544, 18176), (1, 32, 18176, 4544), (1, 32, 4096, 6144), (1, 32, 4096, 4096), (1, 32, 14336, 4096),
+          (1, 32, 4096, 14336), (3, 24, 768, 160), (2, 40, 1024, 288), (1, 8, 32, 32), (1, 32, 64, 4096), (5, 100, 96, 2080)]
+
+
+@pytest.mark.parametrize("wide", [0, 1])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_every_unit_has_exactly_one_workgroup_and_collectors_come_last(shape, wide):
+    """The two functions the kernels cut the work with, on the decompositions the host chooses: the k ranges of an output
+    tile it without gap or overlap, workgroup_of inverts range_start, and whoever collects an output has a higher index
+    than every workgroup that contributes to it — the collectors wait for lower indices only.  (That lower indices are
+    dispatched first and therefore finish without waiting for anybody is an assumption about the hardware's dispatcher,
+    not a guarantee of the programming model; the bounded wait and the error word cover the case that it fails.)"""
+    L = _test_entries()
+    out = (ctypes.c_uint32 * 4)()
+    L.ttmi_test_stream_decomposition(*shape, wide, out)
+    groups, kt, split, workgroups = (int(x) for x in out)
+    batch, m, k, n = shape
+    assert kt == k // 32 and groups == batch * -(-m // 32) * -(-(n // 32) // (4 if wide else 2))
+    assert split >= 1 and workgroups == groups * split
+    assert split == 1 or kt // split >= 2                     # every wavefront of a shared output keeps work to do
+    starts = [L.ttmi_test_range_start(kt, split, i) for i in range(min(workgroups, 600) + 1)]
+    for i in range(len(starts) - 1):
+        og, part = divmod(i, split)
+        assert og * kt <= starts[i] < starts[i + 1] <= (og + 1) * kt          # non-empty, inside its own output
+        if part == 0:
+            assert starts[i] == og * kt                                         # the first range starts the output
+        for unit in {starts[i], starts[i + 1] - 1, (starts[i] + starts[i + 1]) // 2}:
+            assert L.ttmi_test_workgroup_of(kt, split, unit) == i
+    if split > 1:
+        # wide kernel: the `split` workgroups of output g + 1 (after the last output: `split` extra workgroups) collect
+        # output g; 64-column kernel: the contributor with the highest index collects
+        for g in range(min(groups, 50)):
+            contributors = range(g * split, (g + 1) * split)
+            collectors = range((g + 1) * split, (g + 2) * split) if wide else [contributors[-1]]
+            assert min(collectors) >= max(contributors) and (not wide or min(collectors) > max(contributors))
+
+
+def test_library_scratch_grows_geometrically_and_is_never_shrunk():
+    """A buffer that is too small is replaced by one of at least twice its size (the old one is retired, not freed: a
+    kernel of another host thread may still be about to use it), so the retired buffers of a stream add up to less than
+    the live one; sizes are multiples of 256 bytes."""
+    L = _test_entries()
+    grown = L.ttmi_test_scratch_grown_size
+    assert grown(0, 1) == 256 and grown(0, 16384) == 16384 and grown(4096, 100) == 4096
+    assert grown(16384, 16385) == 32768 and grown(16384, 100000) == 100096
+    have, retired = 0, 0
+    for need in (1000, 5000, 5001, 70000, 70001, 300000):
+        new = grown(have, need)
+        assert new >= need and new % 256 == 0
+        if new != have:
+            retired += have
+            assert have == 0 or new >= 2 * have
+            have = new
+    assert retired < have
+
+
+def test_test_knobs_are_validated_and_cleared(knobs):
+    from ttmi import capi
+
+    L = _test_entries()
+    ws = L.ttmi_matmul_bfp_workspace_bytes
+    assert ws(1, 32, 4544, 18176, 3) == 142 * 3 * 16384
+    knobs("workgroups", 256)
+    assert ws(1, 32, 4544, 18176, 3) == 0                       # 256 // 143 = 1 k range per output: nothing is shared
+    knobs("kernel", "expanded")
+    assert ws(1, 32, 64, 64, 3) == 2 * 1 * 4096                 # forced onto the expanding kernel: one 64-column group, two k tiles
+    L.ttmi_test_set_knob.restype = ctypes.c_int
+    assert L.ttmi_test_set_knob(99, 0, 1) == 1 and b"unknown test knob" in L.ttmi_last_error()

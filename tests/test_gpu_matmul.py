@@ -134,12 +134,12 @@ def test_linear_bias_and_activation(oracle, activation):
 
 @pytest.mark.parametrize("m", [40, 24])      # two bands (64-column streaming kernel), one band (128-column kernel)
 @pytest.mark.parametrize("workgroups", ["1", "3", "7", "64", "512", "4096"])
-def test_any_number_of_workgroups_gives_the_same_bits(oracle, workgroups, m, monkeypatch):
+def test_any_number_of_workgroups_gives_the_same_bits(oracle, workgroups, m, knobs):
     """The k range of an output may be shared between workgroups in any way; partial sums are added in a fixed order."""
     k, n = 1024, 288
     a_bits = workloads.activations_bf16(m, k, seed=71)
     words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=72), BFP8)
-    monkeypatch.setenv("TTMI_MATMUL_WGS", workgroups)
+    knobs("workgroups", workgroups)
     c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
     again = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
     assert torch.equal(c.view(torch.int16), again.view(torch.int16))
@@ -165,17 +165,17 @@ def test_caller_workspace(oracle):
 @pytest.mark.parametrize("batch,b_batch,m,k,n", [(1, 1, 256, 128, 256), (1, 1, 300, 96, 288), (2, 1, 130, 160, 96), (1, 1, 288, 224, 96),
                                                  (2, 2, 512, 64, 544), (1, 1, 40, 32, 2080),
                                                  (2, 2, 32, 1024, 224), (3, 1, 24, 768, 160)])
-def test_every_kernel_on_every_shape(oracle, kernel, fmt, batch, b_batch, m, k, n, monkeypatch):
+def test_every_kernel_on_every_shape(oracle, kernel, fmt, batch, b_batch, m, k, n, knobs):
     """Each GEMM kernel forced onto shapes it would not be chosen for: ragged row blocks, odd tile counts, one k step,
     more than eight 256-column blocks, shared and per-slice weights, k ranges long enough for the streaming kernels to
     share outputs between workgroups (with batches and ragged column groups); TILE layout in and out, bias and activation."""
-    monkeypatch.setenv("TTMI_MATMUL_KERNEL", kernel[:4])
+    knobs("kernel", "tile" if kernel.startswith("tile") else kernel)
     if kernel == "tile256":
-        monkeypatch.setenv("TTMI_MATMUL_BM", "256")
+        knobs("block", 256)
     if kernel == "tile4waves":
-        monkeypatch.setenv("TTMI_MATMUL_BM", "4")
+        knobs("block", 4)
     if kernel == "tile384":                                  # 384-row x 64-column blocks, twelve wavefronts
-        monkeypatch.setenv("TTMI_MATMUL_BM", "384")
+        knobs("block", 384)
     a_bits = workloads.activations_bf16(m, k, seed=75, batch=batch)
     w = workloads.weights_f32(k, n, seed=76, batch=b_batch)
     words, w_unpacked = pack_weights(oracle, w, fmt)
@@ -198,8 +198,8 @@ def test_every_kernel_on_every_shape(oracle, kernel, fmt, batch, b_batch, m, k, 
     assert torch.allclose(g, want, rtol=1e-5, atol=1e-5)
 
 
-def test_expanded_weights_in_a_caller_workspace(oracle, monkeypatch):
-    monkeypatch.setenv("TTMI_MATMUL_KERNEL", "expanded")
+def test_expanded_weights_in_a_caller_workspace(oracle, knobs):
+    knobs("kernel", "expanded")
     m, k, n = 512, 128, 160
     a_bits = workloads.activations_bf16(m, k, seed=78)
     words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=79), BFP8)
@@ -251,10 +251,10 @@ def test_decode_gemm_in_a_hip_graph(oracle):
 
 @pytest.mark.parametrize("kernel", ["stream", "wide"])
 @pytest.mark.parametrize("fmt", [BFP8, BFP4])
-def test_row_exponents_over_the_whole_range(oracle, kernel, fmt, monkeypatch):
+def test_row_exponents_over_the_whole_range(oracle, kernel, fmt, knobs):
     """Weight rows scaled by 2^s, s in [-100, 100], against activation columns scaled by 2^-s: every shared exponent from
     about 20 to 230 occurs, the products stay of order one, and the result must not care (scales are exact powers of two)."""
-    monkeypatch.setenv("TTMI_MATMUL_KERNEL", kernel)
+    knobs("kernel", kernel)
     rng = np.random.default_rng(97)
     m, k, n = 32, 512, 256
     shift = rng.integers(-100, 101, size=k)
@@ -358,3 +358,54 @@ def test_bert_like_bmm_full_size(oracle):
     a = workloads.bf16_bits_to_f32(a_bits)
     for b in (0, 5, 11):
         check_against_reference(c[b].float().cpu().numpy(), a[b], w_unpacked[b], k)
+
+
+@pytest.mark.parametrize("kernel,m", [("wide", 32), ("stream", 64)])
+def test_a_wait_that_gives_up_is_reported_and_leaves_later_calls_correct(oracle, kernel, m, knobs):
+    """Forced from the host: producers keep their partial sums to themselves and the bounded wait is cut to a few polls,
+    so every collector gives up (every kernel still runs to its end).  The launch raises the device's error word, the
+    next call reports TTMI_ERR_HIP, and the call after that — on slots that the library refills — is correct again."""
+    k, n = 2048, 256
+    a_bits = workloads.activations_bf16(m, k, seed=120)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=121), BFP8)
+    a = bf16_dev(a_bits)
+    knobs("kernel", kernel)
+    good = capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    torch.cuda.synchronize()
+    capi.device_status()                                                # nothing to report
+    knobs("drop_partial_sums", 1)
+    knobs("spin_limit", 3)
+    capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)     # outputs shared between workgroups: the waits give up
+    torch.cuda.synchronize()
+    knobs("drop_partial_sums", 0)
+    knobs("spin_limit", 1 << 20)
+    with pytest.raises(RuntimeError, match="gave up waiting"):
+        capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    capi.device_status()                                                # reported once, then clear
+    again = capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    torch.cuda.synchronize()
+    capi.device_status()
+    assert torch.equal(again.view(torch.int16), good.view(torch.int16))
+    check_against_reference(again.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+
+
+def test_library_scratch_is_per_stream(oracle):
+    """Without a caller workspace every stream gets slots of its own, so decode GEMMs issued on two streams at once do not
+    share partial sums (the same two calls on one stream share a buffer and run in order)."""
+    m, k, n = 32, 4096, 512
+    a_bits = workloads.activations_bf16(m, k, seed=122)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=123), BFP8)
+    a = bf16_dev(a_bits)
+    want = capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n).clone()
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    results = [[], []]
+    for rep in range(20):
+        for s, stream in enumerate(streams):
+            with torch.cuda.stream(stream):
+                results[s].append(capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n))
+    torch.cuda.synchronize()
+    capi.device_status()
+    for per_stream in results:
+        for c in per_stream:
+            assert torch.equal(c.view(torch.int16), want.view(torch.int16))

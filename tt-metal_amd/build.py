@@ -16,7 +16,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libttmi.so")
-SOURCES = ["ttmi_capi.hip", "bfp_codec.hip", "bfp_matmul.hip", "bfp_matmul_tile.hip", "bfp_matmul_expanded.hip", "eltwise.hip"]
+SOURCES = ["ttmi_capi.hip", "host_state.hip", "bfp_codec.hip", "bfp_matmul.hip", "bfp_matmul_tile.hip", "bfp_matmul_expanded.hip", "eltwise.hip"]
 # files whose device assembly is inspected before the object is built, and the check of check_isa.py that applies
 ISA_CHECKED = {"bfp_matmul.hip": "check", "bfp_matmul_tile.hip": "check_ring_operands"}
 HEADERS = [os.path.join(CSRC, "ttmi_internal.h"), os.path.join(CSRC, "bfp_dequant.h"), os.path.join(ROOT, "include", "ttmi.h")]

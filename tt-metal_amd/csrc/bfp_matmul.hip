@@ -21,10 +21,6 @@
 //              workgroup that owns the last part (see the kernel).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include <stdlib.h>
-
-#include <mutex>
-
 #include <type_traits>
 #include <utility>
 
@@ -39,6 +35,9 @@ struct MatmulDev {
     const uint16_t *bias;    // bf16 [n] or null
     uint8_t *c;              // output (bf16 or fp32)
     float *slots;            // 2 slots of 32x64 fp32 per workgroup, for outputs shared between workgroups (see SLOT_EMPTY)
+    uint32_t *error;         // the device's error word (host memory): raised when a wait for partial sums gives up
+    uint32_t spin_limit;     // polls before such a wait gives up
+    int drop_partial_sums;   // test only: producers keep their sums to themselves, so that the wait must give up
     uint32_t batch, b_batch, m, k, n;
     uint32_t mt, kt, nt, ngroups;
     uint32_t groups;         // batch * mt * ngroups
@@ -70,6 +69,13 @@ constexpr size_t SLOT_BYTES = 32 * GROUP_COLS * sizeof(float);
 // that bit pattern), and the consumer simply re-reads until no word is SLOT_EMPTY, then puts SLOT_EMPTY back.
 constexpr uint32_t SLOT_EMPTY = 0xffffffffu;         // a NaN that arithmetic on bf16-derived inputs does not produce
 constexpr uint32_t SLOT_SPIN_LIMIT = 1u << 20;       // bounded wait: a lost producer must not hang the GPU
+constexpr uint32_t ERROR_SLOT_TIMEOUT = 1;           // what the error word is set to
+
+// A wait that gave up: tell the host (one plain store into the error word, which lives in host memory) and carry on,
+// so that the grid still drains.  The output of this launch is invalid and the call that follows reports it.
+__device__ __forceinline__ void report_timeout(const MatmulDev &p) {
+    if ((threadIdx.x & 63) == 0) __builtin_nontemporal_store(ERROR_SLOT_TIMEOUT, p.error);
+}
 
 __device__ __forceinline__ void slot_store(float4 *to, const u32x4 v) {
     // A store of more than 8 bytes reads its data registers for two more cycles after it has issued; the compiler
@@ -86,13 +92,15 @@ __device__ __forceinline__ uint32_t not_empty(uint32_t bits) { return bits == SL
 // Which units a workgroup takes: every output group is cut into `split` nearly equal k ranges, one per workgroup
 // (P = groups * split): one output per workgroup, at most `split` partial sums to add.  Units are numbered with the
 // k-tile fastest.
-__device__ __forceinline__ uint32_t range_start(const MatmulDev &p, uint32_t i) {
-    return (i / p.split) * p.kt + ((i % p.split) * p.kt) / p.split;
+__host__ __device__ __forceinline__ uint32_t range_start(uint32_t kt, uint32_t split, uint32_t i) {
+    return (i / split) * kt + ((i % split) * kt) / split;
 }
-__device__ __forceinline__ uint32_t workgroup_of(const MatmulDev &p, uint32_t unit) {
-    const uint32_t og = unit / p.kt, within = unit - og * p.kt;
-    return og * p.split + ((within + 1) * p.split - 1) / p.kt;     // largest part j with (j * kt) / split <= within
+__host__ __device__ __forceinline__ uint32_t workgroup_of(uint32_t kt, uint32_t split, uint32_t unit) {
+    const uint32_t og = unit / kt, within = unit - og * kt;
+    return og * split + ((within + 1) * split - 1) / kt;     // largest part j with (j * kt) / split <= within
 }
+__device__ __forceinline__ uint32_t range_start(const MatmulDev &p, uint32_t i) { return range_start(p.kt, p.split, i); }
+__device__ __forceinline__ uint32_t workgroup_of(const MatmulDev &p, uint32_t unit) { return workgroup_of(p.kt, p.split, unit); }
 
 // Work decomposition: units are numbered with the k-tile fastest; a workgroup takes a contiguous range of them (see
 // range_start).  A workgroup whose range covers all k-tiles of an output group stores that output directly.
@@ -325,7 +333,7 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
                     u32x4 v;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[r][j]));
-                    slot_store(slot + r * 64, v);
+                    if (!p.drop_partial_sums) slot_store(slot + r * 64, v);
                 }
                 store_now = false;
             } else {
@@ -360,8 +368,10 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
                             for (int r = 0; r < 2; ++r)
 #pragma unroll
                                 for (int j = 0; j < 4; ++j) missing |= part[u][r][j] == SLOT_EMPTY;
-                        waiting = __ballot(missing) != 0 && ++spins < SLOT_SPIN_LIMIT;
+                        const bool any_missing = __ballot(missing) != 0;
+                        waiting = any_missing && ++spins < p.spin_limit;
                         if (waiting) __builtin_amdgcn_s_sleep(4);
+                        else if (any_missing) report_timeout(p);
                     } while (waiting);
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
@@ -679,7 +689,7 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
             u32x4 v;
 #pragma unroll
             for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[r][j]));
-            slot_store(slot + r * 64, v);
+            if (!p.drop_partial_sums) slot_store(slot + r * 64, v);
         }
     }
     if (og == 0) return;
@@ -697,7 +707,7 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
             u32x4 probe = slot_load_issue(at + (uint64_t)(p.split - 1) * 1024);
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(probe)::"memory");
             const bool missing = active && (probe[0] == SLOT_EMPTY || probe[1] == SLOT_EMPTY || probe[2] == SLOT_EMPTY || probe[3] == SLOT_EMPTY);
-            waiting = __ballot(missing) != 0 && ++spins < SLOT_SPIN_LIMIT;
+            waiting = __ballot(missing) != 0 && ++spins < p.spin_limit;
             if (waiting) __builtin_amdgcn_s_sleep(8);
         } while (waiting);
         float sums[4] = {0.f, 0.f, 0.f, 0.f};
@@ -716,8 +726,10 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
                 for (int u = 0; u < N; ++u)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) missing |= got[u][j] == SLOT_EMPTY;
-                waiting = __ballot(missing && active) != 0 && ++spins < SLOT_SPIN_LIMIT;
+                const bool any_missing = __ballot(missing && active) != 0;
+                waiting = any_missing && ++spins < p.spin_limit;
                 if (waiting) __builtin_amdgcn_s_sleep(4);
+                else if (any_missing) report_timeout(p);
             } while (waiting);
 #pragma unroll
             for (int u = 0; u < N; ++u) {
@@ -745,13 +757,6 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
 // ---------------------------------------------------------------------------------------------------------
 // host side: decomposition, workspace, launch
 // ---------------------------------------------------------------------------------------------------------
-static uint32_t env_u32(const char *name, uint32_t fallback) {
-    const char *v = getenv(name);
-    if (!v || !*v) return fallback;
-    const long x = strtol(v, nullptr, 10);
-    return x > 0 ? (uint32_t)x : fallback;
-}
-
 struct Decomposition { uint32_t mt, kt, nt, ngroups, workgroups, split; uint64_t groups, units; };
 
 static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, bool wide) {
@@ -767,7 +772,7 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     // workgroups per CU (all it can hold, the collecting workgroups included) when that takes few parts per output, one
     // per CU when the outputs are few (measured: many short k ranges cost more than the second workgroup gains).
     const bool few = d.groups < 100;
-    const uint64_t resident = env_u32("TTMI_MATMUL_WGS", wide ? (few ? 256 : 256 * WIDE_WGS_PER_CU) : d.groups >= 256 ? 768 : 512);
+    const uint64_t resident = knob_or(TTMI_KNOB_MATMUL_WORKGROUPS, wide ? (few ? 256 : 256 * WIDE_WGS_PER_CU) : d.groups >= 256 ? 768 : 512);
     uint64_t parts = d.groups >= resident ? 1 : wide && !few ? resident / (d.groups + 1) : resident / d.groups;
     if (parts == 0) parts = 1;
     const uint64_t most = d.kt / (2 * WAVES) ? d.kt / (2 * WAVES) : 1;
@@ -775,32 +780,6 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     d.split = (uint32_t)parts;
     d.workgroups = (uint32_t)(d.groups * parts);
     return d;
-}
-
-// The library's own partial-sum slots, per device, grown on demand and kept until the process ends.  Every word is
-// SLOT_EMPTY when allocated, and every launch leaves it that way.
-struct Scratch { void *ptr = nullptr; size_t bytes = 0; };
-static Scratch g_slots[64];
-
-static int own_slots(size_t bytes, void **slots) {
-    static std::mutex guard;                     // host threads may call in at the same time
-    std::lock_guard<std::mutex> lock(guard);
-    int dev = 0;
-    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
-    if (dev < 0 || dev >= 64) return fail(TTMI_ERR_UNSUPPORTED, "device index %d out of range", dev);
-    Scratch &s = g_slots[dev];
-    if (s.bytes < bytes) {
-        if (s.ptr) {
-            if (int rc = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize")) return rc;
-            if (int rc = check_hip(hipFree(s.ptr), "hipFree")) return rc;
-            s.ptr = nullptr; s.bytes = 0;
-        }
-        if (int rc = check_hip(hipMalloc(&s.ptr, bytes), "hipMalloc(matmul slots)")) return rc;
-        if (int rc = check_hip(hipMemset(s.ptr, 0xff, bytes), "hipMemset(matmul slots)")) return rc;
-        s.bytes = bytes;
-    }
-    *slots = s.ptr;
-    return TTMI_OK;
 }
 
 static size_t slot_bytes_needed(const Decomposition &d, bool wide) {
@@ -822,20 +801,29 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     if (d.units > 0x7fffffffull || d.groups * d.split > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
     const size_t need = slot_bytes_needed(d, wide);
     void *slots = nullptr;
+    bool fill = false;
     if (need == 0) {
     } else if (x.workspace) {
         if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
         if (reinterpret_cast<uintptr_t>(x.workspace) & 255u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 256-byte aligned");
-        // a caller's buffer may hold anything: mark every slot of this launch empty (with a kernel, not a memset node:
-        // the caller may be capturing the stream into a graph)
-        const uint32_t chunks = (uint32_t)(need / 16);
-        hipLaunchKernelGGL(fill_slots_kernel, dim3((chunks + 255) / 256 < 2048 ? (chunks + 255) / 256 : 2048), dim3(256), 0, st, (u32x4 *)x.workspace, chunks);
-        if (int rc = check_launch("fill_slots_kernel")) return rc;
         slots = x.workspace;
-    } else if (int rc = own_slots(need, &slots)) {
+        fill = true;                                // a caller's buffer may hold anything
+    } else if (int rc = scratch_get(SCRATCH_SLOTS, st, need, &slots, &fill)) {
+        // the library's own slots, one buffer per stream: every word is SLOT_EMPTY once filled, and every launch that
+        // completes leaves it that way
         return rc;
     }
+    if (fill) {
+        // every slot of this launch becomes empty (with a kernel, not a memset node: the caller may be capturing the
+        // stream into a graph)
+        const uint32_t chunks = (uint32_t)(need / 16);
+        hipLaunchKernelGGL(fill_slots_kernel, dim3((chunks + 255) / 256 < 2048 ? (chunks + 255) / 256 : 2048), dim3(256), 0, st, (u32x4 *)slots, chunks);
+        if (int rc = check_launch("fill_slots_kernel")) return rc;
+    }
     p.slots = (float *)slots;
+    if (int rc = error_word(&p.error, nullptr)) return rc;
+    p.spin_limit = knob_or(TTMI_KNOB_SPIN_LIMIT, SLOT_SPIN_LIMIT);
+    p.drop_partial_sums = (int)knob_or(TTMI_KNOB_DROP_PARTIAL_SUMS, 0);
 #define TTMI_LAUNCH(W, ACT)                                                                                     \
     if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
     else hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
@@ -859,14 +847,11 @@ int matmul_bfp_wide(const MatmulArgs &x, hipStream_t st) { return launch_streami
 // 128-column units, several bands in 64-column units (measured: 43 against 46 us for 64 rows of the Falcon shape).
 // Taller activations are MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows on (two or more
 // 256-row blocks share every weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
-// TTMI_MATMUL_KERNEL=stream|wide|tile|expanded overrides the choice (for tests and measurements).
-enum class Kernel { Stream, Wide, Tile, Expanded };
+// The test entry point can force a kernel (TTMI_KNOB_MATMUL_KERNEL).
+enum class Kernel { Stream = 1, Wide = 2, Tile = 3, Expanded = 4 };
 static Kernel choose_kernel(uint32_t m) {
-    const char *force = getenv("TTMI_MATMUL_KERNEL");
-    if (force && force[0] == 's') return Kernel::Stream;
-    if (force && force[0] == 'w') return Kernel::Wide;
-    if (force && force[0] == 't') return Kernel::Tile;
-    if (force && force[0] == 'e') return Kernel::Expanded;
+    uint32_t forced;
+    if (knob(TTMI_KNOB_MATMUL_KERNEL, &forced) && forced >= 1 && forced <= 4) return (Kernel)forced;
     if (m >= 512) return Kernel::Expanded;
     if (m >= 128) return Kernel::Tile;
     return m <= 32 ? Kernel::Wide : Kernel::Stream;
@@ -885,6 +870,8 @@ size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n
 }
 
 int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
+    // what an earlier launch on this device has reported (a wait for partial sums that gave up) surfaces here
+    if (int rc = ttmi_device_status()) return rc;
     switch (choose_kernel(x.m)) {
         case Kernel::Expanded: return matmul_bfp_expanded(x, st);
         case Kernel::Tile: return matmul_bfp_tiled(x, st);
@@ -894,3 +881,15 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
 }
 
 }  // namespace ttmi
+
+// Test entry points (not declared in include/ttmi.h): the decomposition the host chooses for a shape, and the two index
+// functions the kernels cut the work with, so that their invariants can be checked without a GPU.
+extern "C" {
+__attribute__((visibility("default"))) void ttmi_test_stream_decomposition(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int wide,
+                                                                           uint32_t out[4]) {
+    const ttmi::Decomposition d = ttmi::decompose(batch, m, k, n, wide != 0);
+    out[0] = (uint32_t)d.groups; out[1] = d.kt; out[2] = d.split; out[3] = d.workgroups;
+}
+__attribute__((visibility("default"))) uint32_t ttmi_test_range_start(uint32_t kt, uint32_t split, uint32_t i) { return ttmi::range_start(kt, split, i); }
+__attribute__((visibility("default"))) uint32_t ttmi_test_workgroup_of(uint32_t kt, uint32_t split, uint32_t unit) { return ttmi::workgroup_of(kt, split, unit); }
+}

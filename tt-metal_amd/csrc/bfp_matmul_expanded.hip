@@ -240,30 +240,6 @@ size_t matmul_expanded_workspace_bytes(uint32_t b_batch, uint32_t k, uint32_t n)
     return (size_t)((uint64_t)b_batch * (k / 32) * groups * GROUP_BYTES);
 }
 
-// The library's own buffer of expanded weights, per device, grown on demand and kept until the process ends.
-struct Expanded { void *ptr = nullptr; size_t bytes = 0; };
-static Expanded g_expanded[64];
-
-static int own_expanded(size_t bytes, void **out) {
-    static std::mutex guard;                     // host threads may call in at the same time
-    std::lock_guard<std::mutex> lock(guard);
-    int dev = 0;
-    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
-    if (dev < 0 || dev >= 64) return fail(TTMI_ERR_UNSUPPORTED, "device index %d out of range", dev);
-    Expanded &s = g_expanded[dev];
-    if (s.bytes < bytes) {
-        if (s.ptr) {
-            if (int rc = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize")) return rc;
-            if (int rc = check_hip(hipFree(s.ptr), "hipFree")) return rc;
-            s.ptr = nullptr; s.bytes = 0;
-        }
-        if (int rc = check_hip(hipMalloc(&s.ptr, bytes), "hipMalloc(expanded weights)")) return rc;
-        s.bytes = bytes;
-    }
-    *out = s.ptr;
-    return TTMI_OK;
-}
-
 int matmul_bfp_expanded(const MatmulArgs &x, hipStream_t st) {
     ExpandedDev p{};
     p.a = (const uint8_t *)x.a; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
@@ -285,8 +261,10 @@ int matmul_bfp_expanded(const MatmulArgs &x, hipStream_t st) {
         if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
         if (reinterpret_cast<uintptr_t>(x.workspace) & 255u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 256-byte aligned");
         expanded = x.workspace;
-    } else if (int rc = own_expanded(need, &expanded)) {
-        return rc;
+    } else {
+        // the library's own buffer, one per stream (launches on one stream run in order, so they can share it)
+        bool fresh;
+        if (int rc = scratch_get(SCRATCH_EXPANDED, st, need, &expanded, &fresh)) return rc;
     }
     p.w = (const uint8_t *)expanded;
     const uint32_t expand_blocks = (uint32_t)((items + 3) / 4);

@@ -738,16 +738,17 @@ int matmul_bfp_tiled(const MatmulArgs &x, hipStream_t st) {
     p.kt = x.k / 32; p.nt = x.n / 32;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE; p.c_f32 = x.c_dtype == TTMI_FLOAT32;
     // 256-row blocks when they fill the chip, 128-row blocks otherwise (fewer idle CUs, half the accumulators).
-    // TTMI_MATMUL_BM forces a form: "256", "128" (eight wavefronts), "4" (128 rows, four wavefronts) or "384" (384 x 64).
+    // The test entry point can force a form (TTMI_KNOB_MATMUL_BLOCK): 256, 128 (eight wavefronts), 4 (128 rows, four wavefronts) or 384 (384 x 64).
     const uint32_t tiles_n = (x.n + TILE_COLS - 1) / TILE_COLS;
     const uint64_t big = (uint64_t)x.batch * ((x.m + 255) / 256) * tiles_n;
-    const char *force_bm = getenv("TTMI_MATMUL_BM");
+    uint32_t forced_form = 0;
+    const bool force_bm = knob(TTMI_KNOB_MATMUL_BLOCK, &forced_form);
     // 384-row x 64-column blocks (every weight expanded once per slice) when the slices are whole multiples of 384 rows
     // and 128-row blocks would leave CUs without a workgroup
     constexpr int TALL_WAVES = 12;
     const uint64_t blocks_128 = (uint64_t)x.batch * ((x.m + 127) / 128) * tiles_n;
     const uint64_t blocks_tall = (uint64_t)x.batch * ((x.m + 32 * TALL_WAVES - 1) / (32 * TALL_WAVES)) * ((x.n + 63) / 64);
-    const bool use_tall = force_bm ? force_bm[0] == '3' : (x.m % (32 * TALL_WAVES) == 0 && blocks_128 < 256 && blocks_tall > blocks_128);
+    const bool use_tall = force_bm ? forced_form == 384 : (x.m % (32 * TALL_WAVES) == 0 && blocks_128 < 256 && blocks_tall > blocks_128);
     if (use_tall) {
         p.tiles_m = (x.m + 32 * TALL_WAVES - 1) / (32 * TALL_WAVES); p.tiles_n = (x.n + 63) / 64;
         if (blocks_tall > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
@@ -759,10 +760,10 @@ int matmul_bfp_tiled(const MatmulArgs &x, hipStream_t st) {
         else launch_tall_act<3, TALL_WAVES>(p, x.activation, (uint32_t)blocks_tall, st);
         return check_launch("matmul_tall_kernel");
     }
-    const bool use_256 = force_bm ? force_bm[0] == '2' : (x.m > 128 && big >= 256 && x.m % 256 == 0);
+    const bool use_256 = force_bm ? forced_form == 256 : (x.m > 128 && big >= 256 && x.m % 256 == 0);
     // 128-row blocks: eight wavefronts (each 64 rows) measure 6 % better than four for short k ranges (batched bmm,
     // k = 1024: epilogue and start-up are spread over twice as many wavefronts), four 1-2 % better for k = 4096
-    const bool four_waves = force_bm ? force_bm[0] == '4' : x.k > 2048;
+    const bool four_waves = force_bm ? forced_form == 4 : x.k > 2048;
     const uint32_t bm = use_256 ? 256 : 128;
     p.tiles_m = (x.m + bm - 1) / bm; p.tiles_n = tiles_n;
     const uint64_t blocks = (uint64_t)x.batch * p.tiles_m * p.tiles_n;

@@ -14,6 +14,27 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int check_launch(const char *what);
 int check_hip(hipError_t e, const char *what);
 
+// ---- host state (host_state.hip) --------------------------------------------------------------------------------------
+enum { SCRATCH_SLOTS = 0, SCRATCH_EXPANDED = 1 };
+// The library's own device buffer of at least `bytes` for this purpose on the current device and this stream.  *fresh is
+// set when the contents are undefined (a new buffer, or one invalidated since): the caller initialises it on `stream`.
+int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fresh);
+void scratch_invalidate(int kind);
+size_t scratch_grown_size(size_t have, size_t need);
+// Device and host address of the current device's error word (either may be null).
+int error_word(uint32_t **device_ptr, volatile uint32_t **host_ptr);
+// Knobs of the test entry point ttmi_test_set_knob(which, value, set); product code never sets them.
+enum {
+    TTMI_KNOB_MATMUL_KERNEL = 0,      // 1 stream (64 columns), 2 wide (128 columns), 3 tiled, 4 expanded
+    TTMI_KNOB_MATMUL_WORKGROUPS = 1,  // workgroups the streaming kernels aim for
+    TTMI_KNOB_MATMUL_BLOCK = 2,       // block form of the tiled kernels: 256, 128 (eight wavefronts), 4 (128 rows, four wavefronts), 384
+    TTMI_KNOB_SPIN_LIMIT = 3,         // polls before a bounded wait gives up
+    TTMI_KNOB_DROP_PARTIAL_SUMS = 4,  // producers do not publish their partial sums (so that a wait must give up)
+    TTMI_KNOB_COUNT = 5
+};
+bool knob(int which, uint32_t *value);
+uint32_t knob_or(int which, uint32_t fallback);
+
 int codec_pack_chunks(int fmt, const float *src, size_t n_tiles, int row_major_input, uint32_t *dst, hipStream_t st);
 int codec_unpack_chunks(int fmt, const uint32_t *words, size_t n_tiles, int row_major_output, float *dst, hipStream_t st);
 int codec_pack_tensor(int fmt, const void *src, int elem, uint32_t batch, uint32_t h, uint32_t w, size_t row_stride,

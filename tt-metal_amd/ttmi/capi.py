@@ -23,7 +23,7 @@ SYMBOLS = (
     "ttmi_pack_fp32_vec_as_bfp_tiles", "ttmi_unpack_bfp_tiles_into_float_vec",
     "ttmi_pack_rowmajor_as_bfp_tiles", "ttmi_unpack_bfp_tiles_as_rowmajor",
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
-    "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles",
+    "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_device_status",
 )
 
 _lib = None
@@ -66,6 +66,8 @@ def lib() -> ctypes.CDLL:
         L.ttmi_copy_window.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(ctypes.c_int32), ctypes.c_float, vp]
         L.ttmi_unpad_tiles.restype = i32
         L.ttmi_unpad_tiles.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(u32), vp]
+        L.ttmi_device_status.restype = i32
+        L.ttmi_device_status.argtypes = []
         L.ttmi_eltwise_bf16.restype = i32
         L.ttmi_eltwise_bf16.argtypes = [i32, vp, vp, ctypes.c_float, vp, sz, vp]
         _lib = L
@@ -244,3 +246,8 @@ def unpad_tiles(dtype: int, tiles, src_tiles, start_tile, dst_tiles):
     check(lib().ttmi_unpad_tiles(dtype, _dev(tiles.contiguous()), u4(*[int(x) for x in src_tiles]), _dev(out), u4(*[int(x) for x in start_tile]),
                                  u4(*[int(x) for x in dst_tiles]), _stream()))
     return out
+
+
+def device_status() -> None:
+    """Raises what a kernel on the current device has reported since the last query (a wait that gave up)."""
+    check(lib().ttmi_device_status())
