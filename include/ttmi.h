@@ -148,6 +148,21 @@ TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
                     int c_dtype, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ttmi_matmul_bfp for callers that cannot allocate device memory: code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and results as
+ * ttmi_matmul_bfp without the workspace pair; the scratch of the kernels lies in a static device array of
+ * TTMI_STATIC_SCRATCH_BYTES (16 MiB) that every GPU the library runs on holds until the process ends, so the call
+ * allocates nothing (no hipMalloc, hipFree or hipHostMalloc).  Shapes whose scratch does not fit
+ * (ttmi_matmul_bfp_workspace_bytes() > TTMI_STATIC_SCRATCH_BYTES: in practice GEMMs of 512 rows and more, whose weights
+ * are expanded to 2 bytes each) are rejected with TTMI_ERR_UNSUPPORTED.  All calls on one GPU share the one array: calls
+ * that overlap in time on one GPU (two streams, two host threads) race and give wrong results — keep them on one
+ * stream.  A wait that gives up is reported through ttmi_device_status() only if the device's error word already exists
+ * (call ttmi_device_status() once beforehand, where allocating is allowed). */
+#define TTMI_STATIC_SCRATCH_BYTES (16u << 20)
+TTMI_API int ttmi_matmul_bfp_static(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch,
+                           uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
+                           int c_dtype, void *stream);
+
 /* c[i] = op(a[i], b[i]) on bf16 tensors of equal shape and layout (count elements, any layout: equal shapes have equal
  * element order), fp32 arithmetic, one rounding to bf16: tt::tt_metal::eltwise_binary
  * (tt_eager/tt_dnn/op_library/eltwise_binary/eltwise_binary_op.hpp:108-140) as reached from ttnn.mul / add / sub

@@ -21,6 +21,7 @@
 //              workgroup that owns the last part (see the kernel).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -821,7 +822,14 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
         if (int rc = check_launch("fill_slots_kernel")) return rc;
     }
     p.slots = (float *)slots;
-    if (int rc = error_word(&p.error, nullptr)) return rc;
+    if (x.no_alloc) {
+        // a report lands in the device's error word when one exists (any earlier ttmi_device_status() creates it),
+        // otherwise in the last bytes of the workspace, where nobody looks: the wait is bounded either way
+        if (!error_word_if_exists(&p.error, nullptr))
+            p.error = x.workspace ? reinterpret_cast<uint32_t *>((uint8_t *)x.workspace + x.workspace_bytes - 256) : nullptr;   // no workspace: nothing is shared, nobody waits
+    } else if (int rc = error_word(&p.error, nullptr)) {
+        return rc;
+    }
     p.spin_limit = knob_or(TTMI_KNOB_SPIN_LIMIT, SLOT_SPIN_LIMIT);
     p.drop_partial_sums = (int)knob_or(TTMI_KNOB_DROP_PARTIAL_SUMS, 0);
 #define TTMI_LAUNCH(W, ACT)                                                                                     \
@@ -871,7 +879,8 @@ size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n
 
 int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
     // what an earlier launch on this device has reported (a wait for partial sums that gave up) surfaces here
-    if (int rc = ttmi_device_status()) return rc;
+    if (!x.no_alloc || error_word_if_exists(nullptr, nullptr))
+        if (int rc = ttmi_device_status()) return rc;
     switch (choose_kernel(x.m)) {
         case Kernel::Expanded: return matmul_bfp_expanded(x, st);
         case Kernel::Tile: return matmul_bfp_tiled(x, st);
@@ -881,6 +890,46 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
 }
 
 }  // namespace ttmi
+
+// ---------------------------------------------------------------------------------------------------------
+// ttmi_matmul_bfp for callers that cannot allocate (a stream under graph capture, a serving loop that forbids hipMalloc):
+// the scratch of the kernels — partial-sum slots below 128 rows, expanded weights from 512 rows on — lies in a static
+// device array instead of a buffer that the library allocates on first use.  Every GPU that the library runs on holds its
+// own copy of the array, at its own address, until the process ends; all calls on one GPU share it.
+// ---------------------------------------------------------------------------------------------------------
+static __device__ __align__(256) uint8_t scratch[TTMI_STATIC_SCRATCH_BYTES + 256];      // + 256: stand-in for the error word
+static void *g_scratch_at[64];       // device address of `scratch` per device (the array's name is no device address on the host)
+static std::mutex g_scratch_guard;
+
+static int static_scratch(void **ptr) {
+    int dev = 0;
+    if (int rc = ttmi::check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (dev < 0 || dev >= 64) return ttmi::fail(TTMI_ERR_UNSUPPORTED, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_guard);
+    if (!g_scratch_at[dev]) {
+        void *at = nullptr;
+        if (int rc = ttmi::check_hip(hipGetSymbolAddress(&at, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+        g_scratch_at[dev] = at;
+    }
+    *ptr = g_scratch_at[dev];
+    return TTMI_OK;
+}
+
+extern "C" int ttmi_matmul_bfp_static(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch,
+                                      uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
+                                      int c_dtype, void *stream) {
+    if (int rc = ttmi::validate_matmul(a, a_layout, b, b_fmt, batch, b_batch, m, k, n, activation, c, c_layout, c_dtype)) return rc;
+    const size_t need = ttmi::matmul_workspace_bytes(batch, m, k, n, b_fmt);
+    if (need > TTMI_STATIC_SCRATCH_BYTES)
+        return ttmi::fail(TTMI_ERR_UNSUPPORTED, "matmul (static scratch): this shape needs %zu bytes of scratch, the static array holds %zu; "
+                          "use ttmi_matmul_bfp with a workspace", need, (size_t)TTMI_STATIC_SCRATCH_BYTES);
+    void *at = nullptr;
+    if (need)
+        if (int rc = static_scratch(&at)) return rc;
+    ttmi::MatmulArgs args{a, a_layout, b, b_fmt, batch, b_batch, m, k, n, bias, activation, c, c_layout, c_dtype, at, need ? (size_t)TTMI_STATIC_SCRATCH_BYTES + 256 : 0};
+    args.no_alloc = true;
+    return ttmi::matmul_bfp(args, (hipStream_t)stream);
+}
 
 // Test entry points (not declared in include/ttmi.h): the decomposition the host chooses for a shape, and the two index
 // functions the kernels cut the work with, so that their invariants can be checked without a GPU.

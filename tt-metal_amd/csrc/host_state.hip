@@ -94,6 +94,18 @@ int error_word(uint32_t **device_ptr, volatile uint32_t **host_ptr) {
     return TTMI_OK;
 }
 
+// The same without creating it: false when this device has no error word yet.
+bool error_word_if_exists(uint32_t **device_ptr, volatile uint32_t **host_ptr) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    std::lock_guard<std::mutex> lock(g_guard);
+    const ErrorWord &w = g_error_word[dev];
+    if (!w.host) return false;
+    if (device_ptr) *device_ptr = w.device;
+    if (host_ptr) *host_ptr = w.host;
+    return true;
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // Test knobs (ttmi_test_set_knob): which kernel, how many workgroups, which block form, the spin limit of the bounded
 // waits, and whether producers keep their partial sums to themselves.  Product code never sets them.

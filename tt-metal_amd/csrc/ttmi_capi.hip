@@ -25,6 +25,24 @@ int check_launch(const char *what) { return check_hip(hipGetLastError(), what); 
 
 static bool is_bfp(int fmt) { return fmt == TTMI_BFLOAT8_B || fmt == TTMI_BFLOAT4_B; }
 
+int validate_matmul(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch, uint32_t m, uint32_t k,
+                    uint32_t n, int activation, const void *c, int c_layout, int c_dtype) {
+    if (!is_bfp(b_fmt)) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: weight dtype must be BFLOAT8_B or BFLOAT4_B, got %d", b_fmt);
+    if (!a || !b || !c) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: null pointer");
+    if (batch == 0 || m == 0 || k == 0 || n == 0) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: empty dimension");
+    // tt_eager/tt_dnn/op_library/bmm/multi_core_reuse_mcast_1d_optimized/...cpp:1207-1210: tile-multiple shapes
+    if ((k & 31) || (n & 31)) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: K (%u) and N (%u) of the weights must be multiples of 32", k, n);
+    if ((a_layout == TTMI_TILE || c_layout == TTMI_TILE) && (m & 31))
+        return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: M (%u) must be a multiple of 32 for TILE layout", m);
+    if ((a_layout != TTMI_TILE && a_layout != TTMI_ROW_MAJOR) || (c_layout != TTMI_TILE && c_layout != TTMI_ROW_MAJOR))
+        return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: unknown layout");
+    if (b_batch != 1 && b_batch != batch)
+        return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: weight batch (%u) must be 1 or equal to the activation batch (%u)", b_batch, batch);
+    if (c_dtype != TTMI_BFLOAT16 && c_dtype != TTMI_FLOAT32) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: output dtype must be BFLOAT16 or FLOAT32");
+    if (activation < TTMI_ACT_NONE || activation > TTMI_ACT_SILU) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: unknown activation %d", activation);
+    return TTMI_OK;
+}
+
 }  // namespace ttmi
 
 using namespace ttmi;
@@ -122,19 +140,7 @@ size_t ttmi_matmul_bfp_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, u
 int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch,
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
                     int c_dtype, void *workspace, size_t workspace_bytes, void *stream) {
-    if (!is_bfp(b_fmt)) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: weight dtype must be BFLOAT8_B or BFLOAT4_B, got %d", b_fmt);
-    if (!a || !b || !c) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: null pointer");
-    if (batch == 0 || m == 0 || k == 0 || n == 0) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: empty dimension");
-    // tt_eager/tt_dnn/op_library/bmm/multi_core_reuse_mcast_1d_optimized/...cpp:1207-1210: tile-multiple shapes
-    if ((k & 31) || (n & 31)) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: K (%u) and N (%u) of the weights must be multiples of 32", k, n);
-    if ((a_layout == TTMI_TILE || c_layout == TTMI_TILE) && (m & 31))
-        return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: M (%u) must be a multiple of 32 for TILE layout", m);
-    if ((a_layout != TTMI_TILE && a_layout != TTMI_ROW_MAJOR) || (c_layout != TTMI_TILE && c_layout != TTMI_ROW_MAJOR))
-        return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: unknown layout");
-    if (b_batch != 1 && b_batch != batch)
-        return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: weight batch (%u) must be 1 or equal to the activation batch (%u)", b_batch, batch);
-    if (c_dtype != TTMI_BFLOAT16 && c_dtype != TTMI_FLOAT32) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: output dtype must be BFLOAT16 or FLOAT32");
-    if (activation < TTMI_ACT_NONE || activation > TTMI_ACT_SILU) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: unknown activation %d", activation);
+    if (int rc = validate_matmul(a, a_layout, b, b_fmt, batch, b_batch, m, k, n, activation, c, c_layout, c_dtype)) return rc;
     MatmulArgs args{a, a_layout, b, b_fmt, batch, b_batch, m, k, n, bias, activation, c, c_layout, c_dtype, workspace, workspace_bytes};
     return matmul_bfp(args, (hipStream_t)stream);
 }

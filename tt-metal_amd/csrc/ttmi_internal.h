@@ -23,6 +23,7 @@ void scratch_invalidate(int kind);
 size_t scratch_grown_size(size_t have, size_t need);
 // Device and host address of the current device's error word (either may be null).
 int error_word(uint32_t **device_ptr, volatile uint32_t **host_ptr);
+bool error_word_if_exists(uint32_t **device_ptr, volatile uint32_t **host_ptr);     // never allocates
 // Knobs of the test entry point ttmi_test_set_knob(which, value, set); product code never sets them.
 enum {
     TTMI_KNOB_MATMUL_KERNEL = 0,      // 1 stream (64 columns), 2 wide (128 columns), 3 tiled, 4 expanded
@@ -59,7 +60,12 @@ struct MatmulArgs {
     const void *bias; int activation;
     void *c; int c_layout, c_dtype;
     void *workspace; size_t workspace_bytes;
+    bool no_alloc = false;          // the call may not allocate: `workspace` is all the scratch there is, its last 256 bytes stand
+                                    // in for the error word when the device has none yet
 };
+// the argument checks of ttmi_matmul_bfp (everything but the workspace)
+int validate_matmul(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch, uint32_t m, uint32_t k,
+                    uint32_t n, int activation, const void *c, int c_layout, int c_dtype);
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
 int matmul_bfp(const MatmulArgs &args, hipStream_t st);         // streaming kernel (decode shapes) or the tiled one
 int matmul_bfp_stream(const MatmulArgs &args, hipStream_t st);

@@ -23,7 +23,7 @@ SYMBOLS = (
     "ttmi_pack_fp32_vec_as_bfp_tiles", "ttmi_unpack_bfp_tiles_into_float_vec",
     "ttmi_pack_rowmajor_as_bfp_tiles", "ttmi_unpack_bfp_tiles_as_rowmajor",
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
-    "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_device_status",
+    "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_device_status", "ttmi_matmul_bfp_static",
 )
 
 _lib = None
@@ -66,6 +66,8 @@ def lib() -> ctypes.CDLL:
         L.ttmi_copy_window.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(ctypes.c_int32), ctypes.c_float, vp]
         L.ttmi_unpad_tiles.restype = i32
         L.ttmi_unpad_tiles.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(u32), vp]
+        L.ttmi_matmul_bfp_static.restype = i32
+        L.ttmi_matmul_bfp_static.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp]
         L.ttmi_device_status.restype = i32
         L.ttmi_device_status.argtypes = []
         L.ttmi_eltwise_bf16.restype = i32
