@@ -71,19 +71,24 @@ template <int W> __device__ __forceinline__ uint32_t from_code(uint32_t code, ui
 }
 
 // Which (tile-in-block, face, row-in-face, lane-in-row) a lane handles at step `it`, and where its 16 source
-// bytes live.  ELEM = bytes per source element.
-template <int ELEM> struct Item {
+// bytes live.  ELEM = bytes per source element.  A block of 256 threads covers 32 rows x TPB tiles; TPB is 8 (fp32) or
+// 16 (bf16) halved SHRINK times: small tensors are cut into more, narrower blocks so that the grid still fills the chip.
+template <int ELEM, int SHRINK = 0> struct Item {
     static constexpr int LPR = ELEM;               // lanes per face row: 4 (fp32) or 2 (bf16)
     static constexpr int EPL = 16 / ELEM;          // elements per lane: 4 or 8
-    static constexpr int TPB = 32 / LPR;           // tiles per block: 8 or 16
+    static constexpr int TPB = (32 / LPR) >> SHRINK;   // tiles per block
+    static constexpr int ITS = 8 >> SHRINK;        // steps per wavefront, one KiB of source each
+    static constexpr int LANES_PER_ROW = TPB * 2 * LPR;            // 64, 32 or 16 lanes walk along one tensor row
+    static constexpr int ROWS_PER_STEP = 64 / LANES_PER_ROW;
     int t, face, i, q;
     __device__ __forceinline__ Item(int mode, int wave, int it, int lane) {
-        const int step = wave * 8 + it;            // 0..31: one KiB of source each
+        const int step = wave * ITS + it;
         q = lane % LPR;
-        if (mode == SRC_TENSOR) {                  // the wave walks along one tensor row
-            const int r = step;
-            t = lane / (2 * LPR);
-            face = (r >> 4) * 2 + ((lane / LPR) & 1);
+        if (mode == SRC_TENSOR) {                  // the wave walks along ROWS_PER_STEP tensor rows
+            const int r = step * ROWS_PER_STEP + lane / LANES_PER_ROW;
+            const int within = lane % LANES_PER_ROW;
+            t = within / (2 * LPR);
+            face = (r >> 4) * 2 + ((within / LPR) & 1);
             i = r & 15;
         } else {                                   // the wave walks through the block's contiguous chunks
             if (ELEM == 4) {                       // tile = 4 KiB = 4 steps
@@ -114,12 +119,12 @@ template <int ELEM> __device__ __forceinline__ void expand(const uint4 raw, uint
 // ---------------------------------------------------------------------------------------------------------
 // pack: MODE selects how the source is addressed; ALIGNED means every lane may use one 16-byte load.
 // ---------------------------------------------------------------------------------------------------------
-template <int W, int ELEM, int MODE, bool ALIGNED>
+template <int W, int ELEM, int MODE, bool ALIGNED, int SHRINK = 0>
 __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
                                                    const CodecShape s) {
     using F = Fmt<W>;
-    using I = Item<ELEM>;
-    constexpr int TPB = I::TPB, EPL = I::EPL, LPR = I::LPR;
+    using I = Item<ELEM, SHRINK>;
+    constexpr int TPB = I::TPB, EPL = I::EPL, LPR = I::LPR, ITS = I::ITS;
     __shared__ __attribute__((aligned(16))) uint8_t stage[TPB * F::tile_bytes];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -141,9 +146,9 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
         n_valid = (uint32_t)min((uint64_t)TPB, s.n_tiles - tile0);
     }
 
-    uint4 raw[8];
+    uint4 raw[ITS];
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
+    for (int it = 0; it < ITS; ++it) {
         const I at(MODE, wave, it, lane);
         raw[it] = make_uint4(0, 0, 0, 0);
         if (at.t >= (int)n_valid) continue;
@@ -179,10 +184,10 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
     // where the reference ORs a hidden one into subnormals and from_torch's double pass zeroes single-bit codes; Inf; NaN)
     // sends the wavefront through the integer recipe.  One ballot per wavefront: per-item ballots and the branches behind
     // them cost 2 to 4 us of 18 for a 4096 x 4096 tensor.
-    uint32_t shared_of[8];
+    uint32_t shared_of[ITS];
     bool odd = false;
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
+    for (int it = 0; it < ITS; ++it) {
         uint32_t bits[EPL];
         expand<ELEM>(raw[it], bits);
         uint32_t top = 0, nonzero = 0;
@@ -206,7 +211,7 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
     };
     if (ordinary) {
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
+        for (int it = 0; it < ITS; ++it) {
             const I at(MODE, wave, it, lane);
             uint32_t bits[EPL];
             expand<ELEM>(raw[it], bits);
@@ -225,7 +230,7 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
         }
     } else {
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
+        for (int it = 0; it < ITS; ++it) {
             const I at(MODE, wave, it, lane);
             uint32_t bits[EPL];
             expand<ELEM>(raw[it], bits);
@@ -255,12 +260,12 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
 // ---------------------------------------------------------------------------------------------------------
 // unpack: the inverse walk.  ELEM is the destination element size (4 = fp32, 2 = bf16).
 // ---------------------------------------------------------------------------------------------------------
-template <int W, int ELEM, int MODE, bool ALIGNED>
+template <int W, int ELEM, int MODE, bool ALIGNED, int SHRINK = 0>
 __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
                                                      const CodecShape s) {
     using F = Fmt<W>;
-    using I = Item<ELEM>;
-    constexpr int TPB = I::TPB, EPL = I::EPL;
+    using I = Item<ELEM, SHRINK>;
+    constexpr int TPB = I::TPB, EPL = I::EPL, ITS = I::ITS;
     __shared__ __attribute__((aligned(16))) uint8_t stage[TPB * F::tile_bytes];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -290,7 +295,7 @@ __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__
     __syncthreads();
 
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
+    for (int it = 0; it < ITS; ++it) {
         const I at(MODE, wave, it, lane);
         if (at.t >= (int)n_valid) continue;
         const uint8_t *tile = stage + at.t * F::tile_bytes;
@@ -541,23 +546,45 @@ int codec_unpad_tiles(uint32_t tile_bytes, const void *src, const uint32_t src_t
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <int W, int ELEM, int MODE>
+template <int W, int ELEM, int MODE, int SHRINK = 0>
 static void launch_pack(bool aligned, const void *src, void *dst, const CodecShape &s, uint32_t blocks, hipStream_t st) {
-    if (aligned) hipLaunchKernelGGL((pack_kernel<W, ELEM, MODE, true>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
-    else hipLaunchKernelGGL((pack_kernel<W, ELEM, MODE, false>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+    if (aligned) hipLaunchKernelGGL((pack_kernel<W, ELEM, MODE, true, SHRINK>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+    else hipLaunchKernelGGL((pack_kernel<W, ELEM, MODE, false, SHRINK>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
 }
-template <int W, int ELEM, int MODE>
+template <int W, int ELEM, int MODE, int SHRINK = 0>
 static void launch_unpack(bool aligned, const void *src, void *dst, const CodecShape &s, uint32_t blocks, hipStream_t st) {
-    if (aligned) hipLaunchKernelGGL((unpack_kernel<W, ELEM, MODE, true>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
-    else hipLaunchKernelGGL((unpack_kernel<W, ELEM, MODE, false>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+    if (aligned) hipLaunchKernelGGL((unpack_kernel<W, ELEM, MODE, true, SHRINK>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+    else hipLaunchKernelGGL((unpack_kernel<W, ELEM, MODE, false, SHRINK>), dim3(blocks), dim3(256), 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+}
+// the tensor forms, with the block width chosen for the tensor (tensor_shape)
+template <int W, int ELEM>
+static void launch_pack_tensor(int shrink, bool aligned, const void *src, void *dst, const CodecShape &s, uint32_t blocks, hipStream_t st) {
+    if (shrink == 2) launch_pack<W, ELEM, SRC_TENSOR, 2>(aligned, src, dst, s, blocks, st);
+    else if (shrink == 1) launch_pack<W, ELEM, SRC_TENSOR, 1>(aligned, src, dst, s, blocks, st);
+    else launch_pack<W, ELEM, SRC_TENSOR, 0>(aligned, src, dst, s, blocks, st);
+}
+template <int W, int ELEM>
+static void launch_unpack_tensor(int shrink, bool aligned, const void *src, void *dst, const CodecShape &s, uint32_t blocks, hipStream_t st) {
+    if (shrink == 2) launch_unpack<W, ELEM, SRC_TENSOR, 2>(aligned, src, dst, s, blocks, st);
+    else if (shrink == 1) launch_unpack<W, ELEM, SRC_TENSOR, 1>(aligned, src, dst, s, blocks, st);
+    else launch_unpack<W, ELEM, SRC_TENSOR, 0>(aligned, src, dst, s, blocks, st);
 }
 
+// Blocks of 32 rows x (32 / elem >> shrink) tiles.  Pack and unpack halve the block width (shrink 1, 2) while that is what it
+// takes to give the 256 CUs two blocks each: a 1024 x 1024 fp32 tensor is 128 blocks of 8 tiles, but 512 blocks of 2.
 static int tensor_shape(CodecShape &s, uint32_t batch, uint32_t h, uint32_t w, size_t row_stride, size_t batch_stride,
-                        int elem, uint64_t &blocks) {
+                        int elem, uint64_t &blocks, int *shrink = nullptr) {
     s.batch = batch; s.h = h; s.w = w;
     s.ht = (h + 31) / 32; s.wt = (w + 31) / 32;
-    const uint32_t tpb = 32 / elem;
+    uint32_t tpb = 32 / elem;
     s.col_groups = (s.wt + tpb - 1) / tpb;
+    if (shrink) {
+        *shrink = 0;
+        while (*shrink < 2 && (uint64_t)batch * s.ht * s.col_groups < 512 && s.wt > tpb / 2) {
+            ++*shrink; tpb /= 2;
+            s.col_groups = (s.wt + tpb - 1) / tpb;
+        }
+    }
     s.n_tiles = (uint64_t)batch * s.ht * s.wt;
     s.row_stride = row_stride; s.batch_stride = batch_stride;
     blocks = (uint64_t)batch * s.ht * s.col_groups;
@@ -605,15 +632,16 @@ int codec_pack_tensor(int fmt, const void *src, int elem, uint32_t batch, uint32
     if (!aligned16(dst)) return fail(TTMI_ERR_INVALID_ARGUMENT, "pack: dst must be 16-byte aligned");
     CodecShape s{};
     uint64_t blocks;
-    if (int rc = tensor_shape(s, batch, h, w, row_stride, batch_stride, elem, blocks)) return rc;
+    int shrink;
+    if (int rc = tensor_shape(s, batch, h, w, row_stride, batch_stride, elem, blocks, &shrink)) return rc;
     const size_t per16 = 16 / elem;
     const bool al = aligned16(src) && w % per16 == 0 && row_stride % per16 == 0 && batch_stride % per16 == 0;
     if (fmt == TTMI_BFLOAT8_B) {
-        if (elem == 4) launch_pack<7, 4, SRC_TENSOR>(al, src, dst, s, (uint32_t)blocks, st);
-        else launch_pack<7, 2, SRC_TENSOR>(al, src, dst, s, (uint32_t)blocks, st);
+        if (elem == 4) launch_pack_tensor<7, 4>(shrink, al, src, dst, s, (uint32_t)blocks, st);
+        else launch_pack_tensor<7, 2>(shrink, al, src, dst, s, (uint32_t)blocks, st);
     } else {
-        if (elem == 4) launch_pack<3, 4, SRC_TENSOR>(al, src, dst, s, (uint32_t)blocks, st);
-        else launch_pack<3, 2, SRC_TENSOR>(al, src, dst, s, (uint32_t)blocks, st);
+        if (elem == 4) launch_pack_tensor<3, 4>(shrink, al, src, dst, s, (uint32_t)blocks, st);
+        else launch_pack_tensor<3, 2>(shrink, al, src, dst, s, (uint32_t)blocks, st);
     }
     return check_launch("pack_kernel");
 }
@@ -624,15 +652,16 @@ int codec_unpack_tensor(int fmt, const uint32_t *words, uint32_t batch, uint32_t
     if (!aligned16(words)) return fail(TTMI_ERR_INVALID_ARGUMENT, "unpack: words must be 16-byte aligned");
     CodecShape s{};
     uint64_t blocks;
-    if (int rc = tensor_shape(s, batch, h, w, w, (size_t)h * w, elem, blocks)) return rc;
+    int shrink;
+    if (int rc = tensor_shape(s, batch, h, w, w, (size_t)h * w, elem, blocks, &shrink)) return rc;
     const size_t per16 = 16 / elem;
     const bool al = aligned16(dst) && w % per16 == 0;
     if (fmt == TTMI_BFLOAT8_B) {
-        if (elem == 4) launch_unpack<7, 4, SRC_TENSOR>(al, words, dst, s, (uint32_t)blocks, st);
-        else launch_unpack<7, 2, SRC_TENSOR>(al, words, dst, s, (uint32_t)blocks, st);
+        if (elem == 4) launch_unpack_tensor<7, 4>(shrink, al, words, dst, s, (uint32_t)blocks, st);
+        else launch_unpack_tensor<7, 2>(shrink, al, words, dst, s, (uint32_t)blocks, st);
     } else {
-        if (elem == 4) launch_unpack<3, 4, SRC_TENSOR>(al, words, dst, s, (uint32_t)blocks, st);
-        else launch_unpack<3, 2, SRC_TENSOR>(al, words, dst, s, (uint32_t)blocks, st);
+        if (elem == 4) launch_unpack_tensor<3, 4>(shrink, al, words, dst, s, (uint32_t)blocks, st);
+        else launch_unpack_tensor<3, 2>(shrink, al, words, dst, s, (uint32_t)blocks, st);
     }
     return check_launch("unpack_kernel");
 }
