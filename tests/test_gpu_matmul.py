@@ -322,42 +322,145 @@ def test_full_size_decode_gemms_on_three_streams():
             assert torch.equal(out.view(torch.int16), j["alone"].reshape(-1).view(torch.int16)), (j["n"], rep)
 
 
+def oracle_unpacked(oracle, fmt, words, k, n, batch=1):
+    """The weights as the reference's host unpacker and untilizer give them back (CPU oracle), [batch, k, n] fp32."""
+    flat = oracle.unpack_bfp_tiles_into_float_vec(fmt, words.cpu().numpy().view(np.uint32), False)
+    return oracle.untilize_nchw_4faces(flat, (1, batch, k, n))[0]
+
+
+def check_on_gpu(c, a_bits, w_unpacked, k, bf16_out=True):
+    """check_against_reference for sizes where the fp64 products are better formed on the GPU: the reference is a float64
+    matmul (torch, on the device) of the exact activations with the oracle-unpacked weights; every element is held to the
+    stated bound, and the PCC is taken over all of them."""
+    a64 = torch.from_numpy(workloads.bf16_bits_to_f32(a_bits)).cuda().double()
+    w64 = torch.from_numpy(np.ascontiguousarray(w_unpacked)).cuda().double()
+    ref = a64 @ w64
+    mag = a64.abs() @ w64.abs()
+    bound = (2.0 ** -8 if bf16_out else 2.0 ** -22) * ref.abs() + 2.0 * k * 2.0 ** -24 * mag + 1e-37
+    got = c.double()
+    worst = float(((got - ref).abs() / bound).max())
+    assert worst <= 1.0, f"elementwise bound exceeded by factor {worst}"
+    pcc = float(torch.corrcoef(torch.stack([ref.reshape(-1), got.reshape(-1)]))[0, 1])
+    assert pcc >= 0.9999, pcc
+    return pcc
+
+
+@pytest.mark.parametrize("layout", [capi.ROW_MAJOR, capi.TILE])
 @pytest.mark.parametrize("name,m,k,n,fmt,batch", workloads.DECODE_FALCON + workloads.DECODE_MISTRAL)
-def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch):
+def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch, layout):
+    """Every decode GEMM of the workloads at full size, in both operand layouts (TILE is what ttnn.matmul takes and returns and
+    what the benchmark times), every output element against the float64 product with the oracle-unpacked weights."""
     a_bits = workloads.activations_bf16(m, k, seed=80)
-    w = workloads.weights_f32(k, n, seed=81)
-    words = capi.pack_tensor(FMT[fmt], dev(w))
-    w_unpacked = oracle.untilize_nchw_4faces(
-        oracle.unpack_bfp_tiles_into_float_vec(FMT[fmt], words.cpu().numpy().view(np.uint32), False), (1, 1, k, n))[0, 0]
-    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, FMT[fmt], 1, 1, m, k, n)
+    words = capi.pack_tensor(FMT[fmt], dev(workloads.weights_f32(k, n, seed=81)))
+    w_unpacked = oracle_unpacked(oracle, FMT[fmt], words, k, n)[0]
+    a = bf16_dev(a_bits)
+    if layout == capi.TILE:
+        c = capi.untilize(capi.matmul_bfp(capi.tilize(a), capi.TILE, words, FMT[fmt], 1, 1, m, k, n, c_layout=capi.TILE), (1, m, n))
+    else:
+        c = capi.matmul_bfp(a, capi.ROW_MAJOR, words, FMT[fmt], 1, 1, m, k, n)
     pcc = check_against_reference(c.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
     print(name, "pcc", pcc)
 
 
-def test_prefill_shape_full_size_sampled_rows(oracle):
-    """[2048,4096] x BFP8 [4096,14336]: all rows computed on the GPU, 48 sampled rows checked in fp64."""
+@pytest.mark.parametrize("layout", [capi.ROW_MAJOR, capi.TILE])
+def test_prefill_shape_full_size_every_row(oracle, layout):
+    """[2048,4096] x BFP8 [4096,14336]: all 2048 x 14336 outputs against the float64 product with the weights as the CPU
+    oracle unpacks them."""
     name, m, k, n, fmt, _ = workloads.PREFILL[0]
     a_bits = workloads.activations_bf16(m, k, seed=82)
-    w = workloads.weights_f32(k, n, seed=83)
-    words = capi.pack_tensor(BFP8, dev(w))
-    w_unpacked = capi.unpack_tensor(BFP8, words, (k, n)).cpu().numpy()
-    assert np.array_equal(oracle.pack_fp32_vec_as_bfp_tiles(BFP8, oracle.tilize_nchw_4faces(w_unpacked[None, None]), False),
-                          words.cpu().numpy().view(np.uint32))
-    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
-    rows = np.random.default_rng(84).choice(m, size=48, replace=False)
-    check_against_reference(c[0][torch.from_numpy(rows).cuda()].float().cpu().numpy(),
-                            workloads.bf16_bits_to_f32(a_bits)[rows], w_unpacked, k)
+    words = capi.pack_tensor(BFP8, dev(workloads.weights_f32(k, n, seed=83)))
+    w_unpacked = oracle_unpacked(oracle, BFP8, words, k, n)[0]
+    a = bf16_dev(a_bits)
+    if layout == capi.TILE:
+        c = capi.untilize(capi.matmul_bfp(capi.tilize(a), capi.TILE, words, BFP8, 1, 1, m, k, n, c_layout=capi.TILE), (1, m, n))
+    else:
+        c = capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    check_on_gpu(c[0], a_bits, w_unpacked, k)
 
 
-def test_bert_like_bmm_full_size(oracle):
+def test_bert_like_bmm_full_size_every_slice(oracle):
     name, m, k, n, fmt, batch = workloads.PREFILL[1]
     a_bits = workloads.activations_bf16(m, k, seed=85, batch=batch)
     w = workloads.weights_f32(k, n, seed=86, batch=batch)
     words, w_unpacked = pack_weights(oracle, w, BFP8)
-    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, BFP8, batch, batch, m, k, n)
-    a = workloads.bf16_bits_to_f32(a_bits)
-    for b in (0, 5, 11):
-        check_against_reference(c[b].float().cpu().numpy(), a[b], w_unpacked[b], k)
+    a = bf16_dev(a_bits)
+    c = capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, batch, batch, m, k, n)
+    c_tiles = capi.untilize(capi.matmul_bfp(capi.tilize(a.reshape(batch, m, k)), capi.TILE, words, BFP8, batch, batch, m, k, n, c_layout=capi.TILE), (batch, m, n))
+    assert torch.equal(c_tiles.view(torch.int16), c.view(torch.int16))
+    for b in range(batch):
+        check_on_gpu(c[b], a_bits.reshape(batch, m, k)[b], w_unpacked[b], k)
+
+
+# ---- rows at the ends of the exponent range ------------------------------------------------------------------------------
+def assemble_tiles(fmt, exps, codes):
+    """Packed tiles from shared exponents [K, N / 16] and codes [K, N] (sign | mantissa), laid out as
+    tt_metal/common/bfloat8.hpp:102-173 does: 64 exponent bytes (face, row), then the faces row by row, element 0 in the
+    low bits; tile (kt, nt) at kt * Nt + nt.  Lets a test hold exponent bytes that no packer writes next to given codes."""
+    k, n = codes.shape
+    kt, nt = k // 32, n // 32
+    tile_bytes = 1088 if fmt == BFP8 else 576
+    out = np.zeros((kt, nt, tile_bytes), dtype=np.uint8)
+    for face in range(4):
+        fr, fc = face >> 1, face & 1
+        e = exps.reshape(kt, 2, 16, nt, 2)[:, fr, :, :, fc]                       # [kt, 16, nt]
+        out[:, :, face * 16:(face + 1) * 16] = e.transpose(0, 2, 1)
+        block = codes.reshape(kt, 2, 16, nt, 2, 16)[:, fr, :, :, fc, :].transpose(0, 2, 1, 3)       # [kt, nt, 16 rows, 16 columns]
+        if fmt == BFP8:
+            out[:, :, 64 + face * 256:64 + (face + 1) * 256] = block.reshape(kt, nt, 256)
+        else:
+            out[:, :, 64 + face * 128:64 + (face + 1) * 128] = (block[..., 0::2] | (block[..., 1::2] << 4)).reshape(kt, nt, 128)
+    return np.ascontiguousarray(out).reshape(-1).view(np.uint32)
+
+
+EDGE_KERNELS = [("wide", 32, None), ("stream", 64, None), ("tile", 256, 128), ("tile", 256, 256), ("tile", 256, 4), ("tile", 384, 384), ("expanded", 512, None)]
+
+
+@pytest.mark.parametrize("kernel,m,block", EDGE_KERNELS)
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_rows_at_the_ends_of_the_exponent_range(oracle, kernel, m, block, fmt, knobs):
+    """What every GEMM kernel does with shared exponents that ordinary weights never have, pinned kernel by kernel:
+      E = 0     (fp32 subnormal sources)  the row is read with the scale of E = 1, the IEEE convention for a zero exponent
+                field; the same in every kernel
+      E = 247   the largest exponent every kernel takes exactly
+      E = 254   exact in the streaming kernels (M < 128), whose operands carry no common factor; in the tiled and expanding
+                kernels the operand, mantissa x 2^(E - 127), overflows for mantissas >= 2: those columns come out non-finite
+      E = 255   (Inf / NaN sources) the 16 columns that share the exponent are non-finite, all others are untouched
+    Expected values are formed here from codes and exponents directly: sign x mantissa x 2^(max(E, 1) - 127 - (W - 1))."""
+    knobs("kernel", kernel)
+    if block:
+        knobs("block", block)
+    w_bits = 7 if fmt == BFP8 else 3
+    rng = np.random.default_rng(130 + m)
+    k, n = 128, 128
+    exps = rng.integers(118, 131, size=(k, n // 16)).astype(np.uint8)
+    codes = rng.integers(0, 1 << (w_bits + 1), size=(k, n)).astype(np.uint8)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    exps[5, :], a[:, 5] = 0, a[:, 5] * 2.0 ** 124            # products of order one: 2^124 x mantissa x 2^(1 - 133)
+    exps[40, :], a[:, 40] = 247, a[:, 40] * 2.0 ** -120
+    exps[77, :], a[:, 77] = 254, a[:, 77] * 2.0 ** -125
+    exps[100, 3] = 255
+    a_bits = workloads.f32_to_bf16_bits_rne(a)
+    a64 = workloads.bf16_bits_to_f32(a_bits).astype(np.float64)
+    mant = (codes & ((1 << w_bits) - 1)).astype(np.float64)
+    sign = np.where(codes >> w_bits, -1.0, 1.0)
+    e_eff = np.maximum(np.repeat(exps, 16, axis=1).astype(np.int64), 1)
+    w64 = sign * mant * np.exp2((e_eff - 127 - (w_bits - 1)).astype(np.float64))
+    w64[100, 48:64] = 0.0                                   # not part of any expectation: those columns must be non-finite
+    words = torch.from_numpy(assemble_tiles(fmt, exps, codes).view(np.int32)).cuda()
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n, out_dtype=torch.float32)[0].cpu().numpy().astype(np.float64)
+    ref = a64 @ w64
+    bound = 2.0 ** -22 * np.abs(ref) + 2.0 * k * 2.0 ** -24 * (np.abs(a64) @ (np.abs(w64) + np.exp2((e_eff - 127).astype(np.float64)))) + 1e-37
+    poisoned = np.zeros(n, dtype=bool)
+    poisoned[48:64] = True                                   # E = 255
+    if kernel in ("tile", "expanded"):
+        poisoned |= (codes[77] & ((1 << w_bits) - 1)) >= 2   # E = 254: mantissa x 2^127 overflows
+    assert not np.isfinite(c[:, poisoned]).any()
+    ok = ~poisoned
+    assert np.isfinite(c[:, ok]).all()
+    assert np.all(np.abs(c[:, ok] - ref[:, ok]) <= bound[:, ok]), float(np.max(np.abs(c[:, ok] - ref[:, ok]) / bound[:, ok]))
+    # the rows at the ends carry weight in the sums: without them the check above would fail
+    without = ref - a64[:, [5, 40, 77]] @ w64[[5, 40, 77]]
+    assert np.max(np.abs(without[:, ok] - ref[:, ok]) / bound[:, ok]) > 100.0
 
 
 @pytest.mark.parametrize("kernel,m", [("wide", 32), ("stream", 64)])

@@ -282,3 +282,15 @@ def test_to_torch_sequence_on_foreign_sign_only_codes(oracle, fmt):
     assert plain[0] == 0x80000000
     seq = oracle.to_torch_bfp_tiles(fmt, words, (32, 32)).view(np.uint32)
     assert seq[0, 0] == 0 and seq[0, 1] == plain[1] and plain[1] != 0
+
+
+def test_known_answers_follow_from_the_reference_text():
+    """tests/golden/derive_known_answers.py re-derives the fixture from the reference's statements (line cited per step),
+    independently of the oracle: the hidden one OR-ed into subnormals and the element-0-in-the-low-bits order are read off the
+    reference's own lines there, and the fixture on file must be what that derivation gives."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("derive_known_answers", os.path.join(HERE, "golden", "derive_known_answers.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert mod.strip_docs(mod.as_file(mod.derive())) == mod.strip_docs(KNOWN)
