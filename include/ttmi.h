@@ -115,6 +115,15 @@ TTMI_API int ttmi_untilize(const void *src, uint32_t elem_size, uint32_t batch, 
 TTMI_API int ttmi_copy_window(int dtype, const void *src, const uint32_t src_shape[4], void *dst, const uint32_t dst_shape[4],
                      const int32_t offset[4], float fill, void *stream);
 
+/* tt::tt_metal::typecast / clone(output_dtype) on a device tensor in TILE layout (tt_eager/tt_dnn/op_library/copy/copy_op.hpp:42-44;
+ * also what tilize(output_dtype) and a block-float matmul output do, tt_eager/tt_dnn/op_library/tilize/tilize_op.hpp:71-73):
+ * n_tiles tiles of 1024 elements in 4-face order change their data type, element order unchanged, in one pass.
+ * Supported: BFLOAT16 | FLOAT32 -> BFLOAT8_B | BFLOAT4_B (the arithmetic of the host packers, one shared exponent per
+ * 16-element face row), BFLOAT8_B | BFLOAT4_B -> BFLOAT16 | FLOAT32 (exact: at most 7 significant bits), BFLOAT16 -> FLOAT32
+ * (exact) and FLOAT32 -> BFLOAT16 (round to nearest even).  The rounding of the Tensix packer that the reference's device op
+ * uses is not in its sources (it lives in the LLK submodules): parity with the device op itself is unpinned. */
+TTMI_API int ttmi_typecast_tiles(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n_tiles, void *stream);
+
 /* tt::tt_metal::unpad on a device tensor in TILE layout (tt_eager/tt_dnn/op_library/unpad/unpad_op.hpp:14-40, the op behind
  * ttnn.Tensor.__getitem__, ttnn/ttnn/operations/core.py:99-108): start and end are tile-aligned there
  * (unpad_op.cpp validate), so whole tiles move and a block-float tensor keeps its codes.

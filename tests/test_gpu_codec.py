@@ -214,3 +214,31 @@ def test_strided_source_and_empty_inputs(oracle):
     # empty tensors are accepted and launch nothing
     assert capi.lib().ttmi_pack_rowmajor_as_bfp_tiles(BFP8, None, capi.FLOAT32, 0, 32, 32, 32, 1024, None, None) == 0
     assert capi.lib().ttmi_unpack_bfp_tiles_into_float_vec(BFP4, None, 0, 0, None, None) == 0
+
+
+@pytest.mark.parametrize("fmt", [capi.BFLOAT8_B, capi.BFLOAT4_B])
+def test_typecast_of_tile_ordered_tensors(oracle, fmt):
+    """ttmi_typecast_tiles: block-float <-> bf16 / fp32 in tile order, one pass each way.  Towards block-float it is the host
+    packers' arithmetic on the face-ordered values (bit-exact against the oracle's sequential pack); back it is exact."""
+    rng = np.random.default_rng(140)
+    n_tiles = 37                                                     # not a multiple of the tiles per block
+    x = (rng.standard_normal(n_tiles * 1024) * np.exp2(rng.integers(-12, 12, size=n_tiles * 1024))).astype(np.float32)
+    x[5000:5016] = 0.0
+    x[7000] = np.float32(1e-41)
+    x32 = torch.from_numpy(x).cuda()
+    want = oracle.pack_fp32_vec_as_bfp_tiles(fmt, x, False)
+    words = capi.typecast_tiles(x32, capi.FLOAT32, fmt)
+    assert np.array_equal(words.cpu().numpy().view(np.uint32), want)
+    back = oracle.unpack_bfp_tiles_into_float_vec(fmt, want, False)
+    assert np.array_equal(capi.typecast_tiles(words, fmt, capi.FLOAT32).cpu().numpy().view(np.uint32), back.view(np.uint32))
+    as_bf16 = capi.typecast_tiles(words, fmt, capi.BFLOAT16)
+    assert as_bf16.dtype == torch.bfloat16 and np.array_equal(as_bf16.float().cpu().numpy(), back)      # at most 7 significant bits
+    # from bf16 tiles: the bf16 values are packed as their exact fp32 values
+    xb = x32.to(torch.bfloat16)
+    assert np.array_equal(capi.typecast_tiles(xb, capi.BFLOAT16, fmt).cpu().numpy().view(np.uint32),
+                          oracle.pack_fp32_vec_as_bfp_tiles(fmt, xb.float().cpu().numpy(), False))
+    # bf16 <-> fp32
+    assert torch.equal(capi.typecast_tiles(xb, capi.BFLOAT16, capi.FLOAT32), xb.float())
+    assert torch.equal(capi.typecast_tiles(x32, capi.FLOAT32, capi.BFLOAT16), xb)                         # round to nearest even, as torch does
+    with pytest.raises(RuntimeError, match="unsupported conversion"):
+        capi.typecast_tiles(words, fmt, fmt)

@@ -687,4 +687,54 @@ int codec_relayout(bool to_tiles, const void *src, uint32_t elem, uint32_t batch
     return check_launch("relayout_kernel");
 }
 
+// bf16 <-> fp32 on flat arrays: fp32 -> bf16 rounds to nearest even, bf16 -> fp32 is exact
+template <bool WIDEN>
+__global__ __launch_bounds__(256) void convert_float_kernel(const void *__restrict__ src, void *__restrict__ dst, uint64_t count) {
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (uint64_t)gridDim.x * 256) {
+        if (WIDEN) {
+            reinterpret_cast<uint32_t *>(dst)[i] = (uint32_t)reinterpret_cast<const uint16_t *>(src)[i] << 16;
+        } else {
+            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+            typedef float f32x2_t __attribute__((ext_vector_type(2)));
+            const f32x2_t v = {reinterpret_cast<const float *>(src)[i], 0.f};
+            reinterpret_cast<uint16_t *>(dst)[i] = (uint16_t)__builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+        }
+    }
+}
+
+// A tensor in tile order (4-face tiles) from one data type to another, element order unchanged: tt::tt_metal::typecast
+// (tt_eager/tt_dnn/op_library/copy/copy_op.hpp:44) for the float formats of this path.  Block-float on either side goes
+// through the codec kernels in their face-ordered chunk mode, reading or writing bf16 / fp32 directly.
+int codec_typecast_tiles(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n_tiles, hipStream_t st) {
+    if (n_tiles == 0) return TTMI_OK;
+    const bool src_bfp = src_dtype == TTMI_BFLOAT8_B || src_dtype == TTMI_BFLOAT4_B;
+    const bool dst_bfp = dst_dtype == TTMI_BFLOAT8_B || dst_dtype == TTMI_BFLOAT4_B;
+    const bool src_float = src_dtype == TTMI_BFLOAT16 || src_dtype == TTMI_FLOAT32;
+    const bool dst_float = dst_dtype == TTMI_BFLOAT16 || dst_dtype == TTMI_FLOAT32;
+    if (!(src_bfp || src_float) || !(dst_bfp || dst_float) || src_dtype == dst_dtype || (src_bfp && dst_bfp))
+        return fail(TTMI_ERR_INVALID_ARGUMENT, "typecast: unsupported conversion %d -> %d", src_dtype, dst_dtype);
+    if (!aligned16(src) || !aligned16(dst)) return fail(TTMI_ERR_INVALID_ARGUMENT, "typecast: src and dst must be 16-byte aligned");
+    CodecShape s{};
+    s.n_tiles = n_tiles;
+    if (src_bfp || dst_bfp) {
+        const int elem = (src_bfp ? dst_dtype : src_dtype) == TTMI_FLOAT32 ? 4 : 2;
+        const uint64_t blocks = (n_tiles + (32 / elem) - 1) / (32 / elem);
+        if (blocks > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "typecast: too many tiles");
+        const int fmt = src_bfp ? src_dtype : dst_dtype;
+        if (dst_bfp) {
+            if (fmt == TTMI_BFLOAT8_B) { if (elem == 4) launch_pack<7, 4, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st); else launch_pack<7, 2, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st); }
+            else { if (elem == 4) launch_pack<3, 4, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st); else launch_pack<3, 2, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st); }
+            return check_launch("pack_kernel");
+        }
+        if (fmt == TTMI_BFLOAT8_B) { if (elem == 4) launch_unpack<7, 4, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st); else launch_unpack<7, 2, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st); }
+        else { if (elem == 4) launch_unpack<3, 4, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st); else launch_unpack<3, 2, SRC_TILE_FACES>(true, src, dst, s, (uint32_t)blocks, st); }
+        return check_launch("unpack_kernel");
+    }
+    const uint64_t count = (uint64_t)n_tiles * 1024;
+    const uint32_t blocks = (uint32_t)((count + 255) / 256 < 256 * 32 ? (count + 255) / 256 : 256 * 32);
+    if (src_dtype == TTMI_BFLOAT16) hipLaunchKernelGGL((convert_float_kernel<true>), dim3(blocks), dim3(256), 0, st, src, dst, count);
+    else hipLaunchKernelGGL((convert_float_kernel<false>), dim3(blocks), dim3(256), 0, st, src, dst, count);
+    return check_launch("convert_float_kernel");
+}
+
 }  // namespace ttmi

@@ -124,6 +124,11 @@ int ttmi_copy_window(int dtype, const void *src, const uint32_t src_shape[4], vo
     return codec_copy_window(dtype, src, src_shape, dst, dst_shape, offset, fill, (hipStream_t)stream);
 }
 
+int ttmi_typecast_tiles(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n_tiles, void *stream) {
+    if (n_tiles && (!src || !dst)) return fail(TTMI_ERR_INVALID_ARGUMENT, "typecast: null pointer");
+    return codec_typecast_tiles(src, src_dtype, dst, dst_dtype, n_tiles, (hipStream_t)stream);
+}
+
 int ttmi_unpad_tiles(int dtype, const void *src, const uint32_t src_tiles[4], void *dst, const uint32_t start_tile[4],
                      const uint32_t dst_tiles[4], void *stream) {
     const uint32_t tile_bytes = ttmi_tile_size(dtype);

@@ -48,6 +48,7 @@ int codec_relayout(bool to_tiles, const void *src, uint32_t elem, uint32_t batch
 int codec_copy_window(int dtype, const void *src, const uint32_t src_shape[4], void *dst, const uint32_t dst_shape[4],
                       const int32_t offset[4], float fill, hipStream_t st);
 
+int codec_typecast_tiles(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n_tiles, hipStream_t st);
 int codec_unpad_tiles(uint32_t tile_bytes, const void *src, const uint32_t src_tiles[4], void *dst, const uint32_t start[4],
                       const uint32_t dst_tiles[4], hipStream_t st);
 

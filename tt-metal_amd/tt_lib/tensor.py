@@ -372,8 +372,6 @@ def _matmul(a: Tensor, b: Tensor, *, bcast_batch: bool, bias: Optional[Tensor] =
         raise RuntimeError("TT_FATAL: bmm (non-bcast matmul) expects input tensors of shapes BCMK*BCKN=BCMN")  # bmm_op.cpp:533
     m, k, n = pa[-2], pa[-1], pb[-1]
     a_buf = a._buf
-    if a.dtype in _BFP:  # block-float activations: exact expansion to bf16 tiles in front of the GEMM
-        a_buf = capi.tilize(capi.unpack_tensor(int(a.dtype), a._buf, (batch_a, m, k), dtype=torch.bfloat16))
     bias_buf = None
     if bias is not None:
         if bias.storage_type() != StorageType.DEVICE:
@@ -383,21 +381,26 @@ def _matmul(a: Tensor, b: Tensor, *, bcast_batch: bool, bias: Optional[Tensor] =
         bb = bias
         bh = bb._padded[-2] if len(bb._padded) > 1 else 1
         # bias is a [.., 32, N] tile row in the reference; row 0 carries the values (matmul.hpp:117-140)
-        if bb.dtype in _BFP:
-            row = capi.unpack_tensor(int(bb.dtype), bb._buf, (1, bh, n), dtype=torch.bfloat16)
-        elif bb.layout == Layout.TILE:
-            row = capi.untilize(bb._buf, (1, bh, n))
-        else:
-            row = bb._buf.view(-1, n)
-        bias_buf = row.reshape(-1, n)[0].contiguous().to(torch.bfloat16)
+        if bb.dtype not in (DataType.BFLOAT16,) + _BFP:
+            raise RuntimeError(f"TT_FATAL: Unsupported data format for the bias: {bb.dtype.name}")
+        with torch.cuda.device(a._device.torch_device):
+            if bb.dtype in _BFP:
+                row = capi.unpack_tensor(int(bb.dtype), bb._buf, (1, bh, n), dtype=torch.bfloat16)
+            elif bb.layout == Layout.TILE:
+                row = capi.untilize(bb._buf, (1, bh, n))
+            else:
+                row = bb._buf.view(-1, n)
+            bias_buf = row.reshape(-1, n)[0].contiguous()      # the first of the tile's 32 rows
     out_dtype = DataType(output_dtype) if output_dtype is not None else a.dtype  # bmm_op.hpp:388: output takes input a's dtype
     if out_dtype not in (DataType.BFLOAT16,) + _BFP:
         raise RuntimeError(f"{op}: output dtype {out_dtype.name} is not supported (BFLOAT16, BFLOAT8_B, BFLOAT4_B)")
     with torch.cuda.device(a._device.torch_device):
+        if a.dtype in _BFP:   # block-float activations: expanded (exactly) to bf16 tiles by one kernel in front of the GEMM
+            a_buf = capi.typecast_tiles(a._buf, int(a.dtype), capi.BFLOAT16)
         c = capi.matmul_bfp(a_buf, capi.TILE, b._buf, int(b.dtype), batch_a, batch_b, m, k, n, bias=bias_buf,
                             activation=activation, c_layout=capi.TILE, out_dtype=torch.bfloat16)
-        if out_dtype in _BFP:  # the packer of the reference's compute kernel, applied to the bf16 result tiles
-            c = capi.pack_chunks(int(out_dtype), c.float(), False)
+        if out_dtype in _BFP:  # the packer of the reference's compute kernel, applied to the bf16 result tiles by one kernel
+            c = capi.typecast_tiles(c, capi.BFLOAT16, int(out_dtype))
     logical = tuple(a._shape[:-1]) + (b._shape[-1],)
     padded = pa[:-1] + (n,)
     return Tensor(None, _raw=(c, logical, padded, out_dtype, Layout.TILE, a._device))
@@ -577,8 +580,7 @@ def _as_bf16_buffer(t: Tensor) -> "torch.Tensor":
     if t.storage_type() != StorageType.DEVICE:
         raise RuntimeError("TT_FATAL: Operands to eltwise ops need to be on device!")
     if t.dtype in _BFP:
-        words = capi.unpack_chunks(int(t.dtype), t._buf, False)      # fp32, same order as the packed data
-        return words.to(torch.bfloat16)                               # <= 7 significant bits: exact
+        return capi.typecast_tiles(t._buf, int(t.dtype), capi.BFLOAT16)     # same element order, <= 7 significant bits: exact
     if t.dtype != DataType.BFLOAT16:
         raise RuntimeError(f"TT_FATAL: Unsupported data format {t.dtype.name} (BFLOAT16, BFLOAT8_B, BFLOAT4_B)")
     return t._buf.reshape(-1)
@@ -594,7 +596,7 @@ def _eltwise(op: int, a: Tensor, b=None, scalar: float = 0.0, name: str = "eltwi
     with torch.cuda.device(a._device.torch_device):
         out = capi.eltwise(op, _as_bf16_buffer(a), _as_bf16_buffer(b) if b is not None else None, scalar)
         if a.dtype in _BFP:      # output takes input a's dtype (eltwise_binary_op.hpp:124-126)
-            out = capi.pack_chunks(int(a.dtype), out.float(), False)
+            out = capi.typecast_tiles(out, capi.BFLOAT16, int(a.dtype))
         elif a.layout == Layout.ROW_MAJOR:
             out = out.view(a._padded)
     return a._like(out)
@@ -709,16 +711,19 @@ def typecast(input_tensor: Tensor, dtype: DataType, output_mem_config: Optional[
     if (input_tensor.dtype in _BFP or dtype in _BFP) and input_tensor.layout != Layout.TILE:
         raise RuntimeError("TT_FATAL: block-float tensors on device are in TILE layout")
     with torch.cuda.device(input_tensor._device.torch_device):
-        if input_tensor.dtype in _BFP:
-            values = capi.unpack_chunks(int(input_tensor.dtype), input_tensor._buf, False)      # fp32 in tile order, exact
+        src, src_dtype = input_tensor._buf, int(input_tensor.dtype)
+        if input_tensor.dtype in _BFP and dtype in _BFP:        # through bf16, which holds every block-float value exactly
+            src, src_dtype = capi.typecast_tiles(src, src_dtype, capi.BFLOAT16), capi.BFLOAT16
+        if input_tensor.layout == Layout.ROW_MAJOR:
+            # dense row-major floats: the element order does not matter to a bf16 <-> fp32 conversion; whole "tiles" of
+            # 1024 elements are what the entry point counts in, so the tail is padded for the call and cut off again
+            flat = src.reshape(-1)
+            pad = (-flat.numel()) % 1024
+            if pad:
+                flat = torch.cat([flat, flat.new_zeros(pad)])
+            out = capi.typecast_tiles(flat, src_dtype, int(dtype))[:flat.numel() - pad].view(input_tensor._padded)
         else:
-            values = input_tensor._buf.reshape(-1).float()
-        if dtype in _BFP:
-            out = capi.pack_chunks(int(dtype), values, False)
-        else:
-            out = values.to(_TORCH[dtype])
-            if input_tensor.layout == Layout.ROW_MAJOR:
-                out = out.view(input_tensor._padded)
+            out = capi.typecast_tiles(src, src_dtype, int(dtype))
     return input_tensor._like(out, dtype=dtype)
 
 

@@ -23,7 +23,7 @@ SYMBOLS = (
     "ttmi_pack_fp32_vec_as_bfp_tiles", "ttmi_unpack_bfp_tiles_into_float_vec",
     "ttmi_pack_rowmajor_as_bfp_tiles", "ttmi_unpack_bfp_tiles_as_rowmajor",
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
-    "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_device_status", "ttmi_matmul_bfp_static",
+    "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_typecast_tiles", "ttmi_device_status", "ttmi_matmul_bfp_static",
 )
 
 _lib = None
@@ -68,6 +68,8 @@ def lib() -> ctypes.CDLL:
         L.ttmi_unpad_tiles.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(u32), vp]
         L.ttmi_matmul_bfp_static.restype = i32
         L.ttmi_matmul_bfp_static.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp]
+        L.ttmi_typecast_tiles.restype = i32
+        L.ttmi_typecast_tiles.argtypes = [vp, i32, vp, i32, sz, vp]
         L.ttmi_device_status.restype = i32
         L.ttmi_device_status.argtypes = []
         L.ttmi_eltwise_bf16.restype = i32
@@ -253,3 +255,23 @@ def unpad_tiles(dtype: int, tiles, src_tiles, start_tile, dst_tiles):
 def device_status() -> None:
     """Raises what a kernel on the current device has reported since the last query (a wait that gave up)."""
     check(lib().ttmi_device_status())
+
+
+_TORCH_OF = {}
+
+
+def typecast_tiles(src, src_dtype: int, dst_dtype: int):
+    """A flat cuda buffer in tile order from one data type to another (block-float <-> bf16 / fp32, bf16 <-> fp32), one kernel."""
+    import torch
+
+    if not _TORCH_OF:
+        _TORCH_OF.update({BFLOAT16: torch.bfloat16, FLOAT32: torch.float32, BFLOAT8_B: torch.int32, BFLOAT4_B: torch.int32})
+    src = src.contiguous().reshape(-1)
+    nbytes = src.numel() * src.element_size()
+    if nbytes % TILE_BYTES[src_dtype]:
+        raise RuntimeError("typecast: the buffer does not hold whole tiles")
+    n_tiles = nbytes // TILE_BYTES[src_dtype]
+    out = torch.empty(n_tiles * TILE_BYTES[dst_dtype] // torch.empty(0, dtype=_TORCH_OF[dst_dtype]).element_size(), dtype=_TORCH_OF[dst_dtype],
+                      device=src.device)
+    check(lib().ttmi_typecast_tiles(_dev(src), src_dtype, _dev(out), dst_dtype, n_tiles, _stream()))
+    return out

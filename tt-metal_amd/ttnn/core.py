@@ -43,10 +43,12 @@ def from_torch(tensor: "torch.Tensor", dtype: Optional[DataType] = None, *, layo
         logical = tuple(src.shape)
         padded = logical[:-2] + (_pad32(logical[-2]), _pad32(logical[-1]))
         fmt = int(dtype)
-        target = device.torch_device if device is not None else None
-        words = _run_on_gpu(src, lambda d: capi.pack_tensor(fmt, d), target)
         if device is not None:
-            words = words.to(device.torch_device)
+            # the source goes to the device once and the packed words stay there
+            with torch.cuda.device(device.torch_device):
+                words = capi.pack_tensor(fmt, src.to(device.torch_device))
+        else:
+            words = _run_on_gpu(src, lambda d: capi.pack_tensor(fmt, d))
         return Tensor(None, _raw=(words, logical, padded, DataType(dtype), Layout.TILE, device))
 
     t = Tensor(tensor, dtype)
