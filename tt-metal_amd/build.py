@@ -72,18 +72,22 @@ def build(force: bool = False, verbose: bool = False) -> str:
 
 
 def build_bindings(force: bool = False, verbose: bool = False) -> str:
-    """Builds the pybind11 module tt-metal_amd/lib/_ttmi*.so (host C++ only; links libttmi.so next to it)."""
+    """Builds the pybind11 module tt-metal_amd/lib/_ttmi*.so: the host layer (csrc/host/tensor_ops.cpp: Tensor, validation,
+    conversion sequences, dispatch) and the bindings, host C++ only; links libttmi.so next to it and the HIP runtime."""
     import sysconfig
 
     import pybind11
 
     build(force=False, verbose=verbose)
-    src = os.path.join(CSRC, "ttmi_pybind.cpp")
+    sources = [os.path.join(CSRC, "ttmi_pybind.cpp"), os.path.join(CSRC, "host", "tensor_ops.cpp")]
+    deps = sources + [os.path.join(CSRC, "host", "tensor_ops.hpp"), os.path.join(ROOT, "include", "ttmi.h"), LIB]
     out = os.path.join(LIB_DIR, "_ttmi" + sysconfig.get_config_var("EXT_SUFFIX"))
-    if force or _stale(out, [src, os.path.join(ROOT, "include", "ttmi.h"), LIB]):
-        cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
-               "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"], "-I", os.path.join(ROOT, "include"),
-               src, "-o", out, "-L", LIB_DIR, "-lttmi", "-Wl,-rpath,$ORIGIN"]
+    if force or _stale(out, deps):
+        rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+        cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__",
+               "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"], "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+               "-I", os.path.join(rocm, "include")] + sources + [
+               "-o", out, "-L", LIB_DIR, "-lttmi", "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(rocm, "lib")]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)

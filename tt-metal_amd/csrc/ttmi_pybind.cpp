@@ -1,16 +1,24 @@
 // pybind11 module `_ttmi`: the C ABI of include/ttmi.h with the shape of the reference's own bindings.
 //
+// Two layers.  (1) Tensor and the operations on it (host/tensor_ops.hpp): shapes, validation, conversion sequences and
+// dispatch in C++, as the reference keeps them in tt_lib._C / ttnn._ttnn; the Python packages ttnn/ and tt_lib/ are
+// signature shims over this.  Memory and the stream come from Python callbacks (torch's allocator, torch's current
+// stream).  (2) The entry points of the C ABI on raw device addresses, for callers that manage their own buffers.
+//
 // The reference reaches this path through pybind11 modules (tt_lib._C: tt_eager/tt_lib/csrc/tt_lib_bindings_tensor_pytensor.cpp,
 // tt_lib_bindings_tensor_custom_bmm_ops.cpp; ttnn._ttnn: ttnn/cpp/pybind11/operations/matmul.hpp).  This module is the
 // same layer over libttmi.so: buffers are device addresses (integers, e.g. torch.Tensor.data_ptr()), `stream` is a
 // hipStream_t as an integer, every failure raises RuntimeError with ttmi_last_error(), and the GIL is released around
 // the calls.  Names follow the entry points they stand for.
+#include <pybind11/functional.h>
 #include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
 
 #include <cstdint>
 #include <stdexcept>
 #include <string>
 
+#include "host/tensor_ops.hpp"
 #include "ttmi.h"
 
 namespace py = pybind11;
@@ -34,8 +42,121 @@ int activation_code(const py::object &activation) {   // ttnn/ttnn/operations/ma
 
 }  // namespace
 
+namespace host = ttmi::host;
+
+// a Python object (a torch tensor) as the owner of a Buffer; dropped under the GIL
+std::shared_ptr<void> keep_alive(py::object object) {
+    return std::shared_ptr<void>(new py::object(std::move(object)), [](void *p) {
+        py::gil_scoped_acquire gil;
+        delete static_cast<py::object *>(p);
+    });
+}
+py::object owner_of(const host::Tensor &t) {
+    if (!t.buffer.owner) return py::none();
+    return *static_cast<py::object *>(t.buffer.owner.get());
+}
+std::optional<host::DataType> optional_dtype(const py::object &dtype) {
+    if (dtype.is_none()) return std::nullopt;
+    return (host::DataType)py::cast<int>(dtype);
+}
+const host::Tensor *optional_tensor(const py::object &t) { return t.is_none() ? nullptr : &py::cast<const host::Tensor &>(t); }
+
+void bind_tensor_layer(py::module_ &m) {
+    py::class_<host::Tensor>(m, "Tensor", "Shape with and without tile padding, data type, layout and a buffer on the host or on a GPU")
+        .def_property_readonly("shape", [](const host::Tensor &t) { return py::tuple(py::cast(t.shape)); })
+        .def_property_readonly("padded_shape", [](const host::Tensor &t) { return py::tuple(py::cast(t.padded)); })
+        .def_property_readonly("dtype", [](const host::Tensor &t) { return (int)t.dtype; })
+        .def_property_readonly("layout", [](const host::Tensor &t) { return (int)t.layout; })
+        .def_property_readonly("device", [](const host::Tensor &t) { return t.buffer.device; })
+        .def_property_readonly("nbytes", [](const host::Tensor &t) { return t.buffer.nbytes; })
+        .def_property_readonly("data_ptr", [](const host::Tensor &t) { return (uintptr_t)t.buffer.data; })
+        .def_property_readonly("storage", &owner_of, "the object that owns the memory (a flat torch.uint8 tensor)")
+        .def("volume", &host::Tensor::volume);
+
+    m.def("set_runtime",
+          [](py::function allocate, py::function stream, py::function gpu_available) {
+              host::Runtime rt;
+              rt.allocate = [allocate](size_t nbytes, int device) {
+                  py::object storage = allocate(nbytes, device);                  // flat uint8 tensor on that device (-1: host)
+                  host::Buffer b;
+                  b.data = reinterpret_cast<void *>(py::cast<uintptr_t>(storage.attr("data_ptr")()));
+                  b.nbytes = nbytes;
+                  b.device = device;
+                  b.owner = keep_alive(std::move(storage));
+                  return b;
+              };
+              rt.stream = [stream](int device) { return reinterpret_cast<void *>(py::cast<uintptr_t>(stream(device))); };
+              rt.gpu_available = [gpu_available]() { return py::cast<bool>(gpu_available()); };
+              host::set_runtime(std::move(rt));
+              // the callbacks are Python objects: they go before the interpreter does
+              static bool registered = false;
+              if (!registered) {
+                  py::module_::import("atexit").attr("register")(py::cpp_function([]() { host::set_runtime(host::Runtime{}); }));
+                  registered = true;
+              }
+          },
+          py::arg("allocate"), py::arg("stream"), py::arg("gpu_available"),
+          "allocate(nbytes, device) -> flat uint8 tensor (device -1: host); stream(device) -> hipStream_t as an integer; gpu_available() -> bool");
+
+    m.def("wrap",
+          [](py::object storage, uintptr_t data, size_t nbytes, int device, host::Dims shape, host::Dims padded, int dtype, int layout) {
+              host::Buffer b;
+              b.data = reinterpret_cast<void *>(data); b.nbytes = nbytes; b.device = device; b.owner = keep_alive(std::move(storage));
+              return host::wrap(std::move(b), shape, padded, (host::DataType)dtype, (host::Layout)layout);
+          },
+          "a Tensor over memory that a Python object owns");
+    m.def("from_host", [](uintptr_t data, host::Dims shape, int dtype) { return host::from_host(reinterpret_cast<const void *>(data), shape, (host::DataType)dtype); },
+          "tt_lib.tensor.Tensor(torch_tensor, data_type), tt_lib_bindings_tensor_pytensor.cpp:26-167");
+    m.def("to_layout", [](const host::Tensor &t, int layout) { return host::to_layout(t, (host::Layout)layout); });
+    m.def("to_device", &host::to_device);
+    m.def("to_host", &host::to_host);
+    m.def("reshape", &host::reshape);
+    m.def("to_torch", &host::to_torch);
+    m.def("pad", &host::pad);
+    m.def("unpad", &host::unpad);
+    m.def("pad_to_tile", &host::pad_to_tile);
+    m.def("unpad_from_tile", &host::unpad_from_tile);
+    m.def("device_unpad", &host::device_unpad);
+    m.def("matmul",
+          [](const host::Tensor &a, const host::Tensor &b, bool bcast_batch, const py::object &bias, int activation, const py::object &output_dtype,
+             const std::string &op) { return host::matmul(a, b, bcast_batch, optional_tensor(bias), activation, optional_dtype(output_dtype), op); },
+          py::arg("a"), py::arg("b"), py::arg("bcast_batch"), py::arg("bias") = py::none(), py::arg("activation") = 0, py::arg("output_dtype") = py::none(),
+          py::arg("op") = "matmul", "tt::operations::primary::matmul, tt_eager/tt_dnn/op_library/bmm/bmm_op.cpp:828-1049");
+    m.def("ttnn_matmul",
+          [](const std::string &name, const host::Tensor &a, const host::Tensor &b, const py::object &bias, const py::object &activation,
+             const py::object &dtype) {
+              std::optional<std::string> act;
+              if (!activation.is_none()) act = py::cast<std::string>(py::str(activation));
+              return host::ttnn_matmul(name, a, b, optional_tensor(bias), act, optional_dtype(dtype));
+          },
+          py::arg("operation_name"), py::arg("a"), py::arg("b"), py::arg("bias") = py::none(), py::arg("activation") = py::none(), py::arg("dtype") = py::none(),
+          "ttnn.matmul / ttnn.linear, ttnn/cpp/ttnn/operations/matmul.hpp:44-214");
+    m.def("activation_code", [](const py::object &activation) {
+        std::optional<std::string> act;
+        if (!activation.is_none()) act = py::cast<std::string>(py::str(activation));
+        return host::activation_code(act);
+    });
+    m.def("eltwise",
+          [](int op, const host::Tensor &a, const py::object &b, float scalar, const std::string &name) { return host::eltwise(op, a, optional_tensor(b), scalar, name); },
+          py::arg("op"), py::arg("a"), py::arg("b") = py::none(), py::arg("scalar") = 0.0f, py::arg("name") = "eltwise");
+    m.def("typecast", [](const host::Tensor &t, int dtype) { return host::typecast(t, (host::DataType)dtype); });
+    m.def("clone", [](const host::Tensor &t, const py::object &dtype) { return host::clone(t, optional_dtype(dtype)); });
+    m.def("tilize", [](const host::Tensor &t, const py::object &dtype) { return host::tilize(t, optional_dtype(dtype)); });
+    m.def("ttnn_from_torch_block_float",
+          [](uintptr_t data, int src_dtype, host::Dims shape, int dtype, int device) {
+              return host::ttnn_from_torch_block_float(reinterpret_cast<const void *>(data), (host::DataType)src_dtype, shape, (host::DataType)dtype, device);
+          },
+          "ttnn.from_torch(dtype=bfloat8_b|bfloat4_b, layout=TILE_LAYOUT), ttnn/ttnn/operations/core.py:245-311, as one fused kernel");
+    m.def("ttnn_to_torch", &host::ttnn_to_torch);
+    m.def("ttnn_to_layout", [](const host::Tensor &t, int layout, const py::object &dtype) { return host::ttnn_to_layout(t, (host::Layout)layout, optional_dtype(dtype)); });
+    m.def("ttnn_getitem_prefix", &host::ttnn_getitem_prefix);
+    m.def("dump_tensor", &host::dump_tensor);
+    m.def("load_tensor", &host::load_tensor);
+}
+
 PYBIND11_MODULE(_ttmi, m) {
-    m.doc() = "Block-float tensors of tt-metal / TT-NN on MI355X: pybind11 layer over the C ABI (include/ttmi.h)";
+    m.doc() = "Block-float tensors of tt-metal / TT-NN on MI355X: the host layer (Tensor and its operations) and the C ABI (include/ttmi.h)";
+    bind_tensor_layer(m);
 
     m.attr("BFLOAT16") = (int)TTMI_BFLOAT16;
     m.attr("FLOAT32") = (int)TTMI_FLOAT32;
@@ -114,7 +235,7 @@ PYBIND11_MODULE(_ttmi, m) {
           py::arg("c_dtype") = (int)TTMI_BFLOAT16, py::arg("workspace") = 0, py::arg("workspace_bytes") = 0, py::arg("stream") = 0,
           "ttnn.linear / ttnn.matmul with block-float weights, ttnn/cpp/ttnn/operations/matmul.hpp:44-214");
     // ttnn.mul / add / sub and gelu / relu / silu on bf16 tensors of equal shape (ttnn/ttnn/operations/binary.py:321-424)
-    m.def("eltwise",
+    m.def("eltwise_bf16",
           [](int op, uintptr_t a, uintptr_t b, float scalar, uintptr_t c, size_t count, uintptr_t stream) {
               py::gil_scoped_release release;
               check(ttmi_eltwise_bf16(op, ptr<const void>(a), ptr<const void>(b), scalar, ptr<void>(c), count, ptr<void>(stream)));

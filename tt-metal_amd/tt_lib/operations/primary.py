@@ -21,7 +21,7 @@ def matmul(input_tensor_a, input_tensor_b, bias=None, program_config=None, outpu
     if fused not in _ACT:
         raise RuntimeError(f"{fused} is not supported as activation function")
     batch_b = 1
-    for s in input_tensor_b.shape.with_tile_padding()[:-2]:
-        batch_b *= s
+    for extent in tuple(input_tensor_b.shape.with_tile_padding())[:-2]:
+        batch_b *= extent
     return _t._matmul(input_tensor_a, input_tensor_b, bcast_batch=batch_b == 1, bias=bias, activation=_ACT[fused],
                       output_dtype=output_dtype, op="primary.matmul")

@@ -2,8 +2,9 @@
 
 Mirrors ttnn/ttnn/types.py:11-48, ttnn/ttnn/operations/core.py (from_torch, to_torch, to_layout, to_device,
 from_device, reshape) and ttnn/ttnn/operations/matmul.py (matmul, linear) of tt-metal, same names, keyword
-arguments and error conditions.  Conversions and the GEMM run as HIP kernels behind the C ABI; nothing here
-computes on the CPU, and without the built library or without a GPU these functions raise RuntimeError.
+arguments and error conditions.  A signature shim: the Tensor object, the shape and padding rules, validation and
+dispatch live in the C++ host layer of the pybind11 module ``_ttmi``; conversions and the GEMM run as HIP kernels behind
+the C ABI.  Nothing computes on the CPU, and without the built library or without a GPU these functions raise RuntimeError.
 Tensix-only knobs (core grids, program configs, math fidelity, memory configs) are accepted and ignored.
 """
 from __future__ import annotations
