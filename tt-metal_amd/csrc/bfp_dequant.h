@@ -35,6 +35,51 @@ template <> struct Wfmt<3> {
     static constexpr float unscale = 1.0f / 4.0f;                           // 2^(127 - bias_exp)
 };
 
+// LDS stage of one wavefront of the 128-column kernel = the 4 adjacent packed tiles of one unit, brought in as `runs`
+// contiguous runs of tiles, each run by run_loads direct global->LDS loads in which lane l takes chunk l of the run: four
+// neighbouring lanes then ask for one aligned 64-byte piece of memory, which is what the address coalescing of the
+// vector memory pipe wants (with a pad slot per face, as Wfmt has it, every piece is split over two groups of four
+// lanes, and the loads, not the memory, bound the kernel: measured 2 us of 17 on the Falcon h_to_4h shape).  A run lies in
+// LDS as it lies in memory (per tile: 64 exponent bytes, then the faces), and what one ds_read touches is kept in
+// different banks without pad slots:
+//   BFP8  run = 2 tiles.  In faces with fc = 1 every lane fetches the chunk (= face row) next to its own, so that rows
+//         2i and 2i + 1 lie swapped: fc moves a lane by 16 bytes.  The second run starts 32 bytes off a multiple of 256.
+//         (tile: 64 bytes, row group kh: 128 bytes, word q: 4 bytes: all 64 lanes of a ds_read2_b32 in different banks.)
+//         Lanes with fc = 1 get the rows of a pair in the other order; slab_expand_hidden takes that out again in the
+//         byte selectors of its v_perm_b32.
+//   BFP4  run = 1 tile (36 of the 64 lanes fetch).  Run r starts 48 r bytes off a multiple of 1024: tile 16-byte phase
+//         3r mod 4, face column fc: 128 bytes, row group kh: 64 bytes, word q / 2: 4 bytes.
+template <int W> struct WideFmt;
+template <> struct WideFmt<7> {
+    static constexpr int tile_bytes = 1088, chunks = 68, face_chunks = 16, face_bytes = 256, row_bytes = 16;
+    static constexpr int run_tiles = 2, runs = 2, run_loads = 3, loads = runs * run_loads;
+    static constexpr int run_stride = run_loads * 1024 + 32, unit_bytes = runs * run_stride;
+};
+template <> struct WideFmt<3> {
+    static constexpr int tile_bytes = 576, chunks = 36, face_chunks = 8, face_bytes = 128, row_bytes = 8;
+    static constexpr int run_tiles = 1, runs = 4, run_loads = 1, loads = runs * run_loads;
+    static constexpr int run_stride = run_loads * 1024 + 48, unit_bytes = runs * run_stride;
+};
+// chunk (16 bytes, counted from the start of the unit's 4 tiles) that this lane fetches in load l of a unit
+template <int W> __device__ __forceinline__ void wide_stage_chunks(int lane, uint32_t (&chunk_of)[WideFmt<W>::loads]) {
+    using F = WideFmt<W>;
+#pragma unroll
+    for (int l = 0; l < F::loads; ++l) {
+        const uint32_t run = l / F::run_loads;
+        uint32_t c = min((uint32_t)((l % F::run_loads) * 64 + lane), (uint32_t)(F::run_tiles * F::chunks - 1));   // idle lanes repeat the last chunk
+        if (W == 7) {
+            const uint32_t in_tile = c % F::chunks;
+            if (in_tile >= 4 && (((in_tile - 4) / F::face_chunks) & 1)) c ^= 1;
+        }
+        chunk_of[l] = run * F::run_tiles * F::chunks + c;
+    }
+}
+// byte offset inside a stage of tile t (0..3) of the unit
+template <int W> __device__ __forceinline__ uint32_t wide_tile_at(int t) {
+    using F = WideFmt<W>;
+    return (t / F::run_tiles) * F::run_stride + (t % F::run_tiles) * F::tile_bytes;
+}
+
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 0xf) | (0x7 << 4) | (0xf << 8) | ((N >> 4) << 14));
@@ -164,7 +209,13 @@ __device__ __forceinline__ uint32_t hidden_pair_field(const u32x2 e01, int p) {
     return spread << 7;
 }
 
-template <int W> __device__ __forceinline__ void slab_expand_hidden(const SlabRaw &r, int q, bf16x8 (&hi)[4], bf16x8 (&lo)[4]) {
+// byte selectors of the BFP8 expansion for operand j: with `swapped` the two words of a row pair arrive in the other order
+__device__ __forceinline__ uint32_t hidden_pair_selector(int j, bool swapped) {
+    const uint32_t first = swapped ? 4u + j : (uint32_t)j, second = swapped ? (uint32_t)j : 4u + j;   // bytes 0..3: words[2p], 4..7: words[2p + 1]
+    return (second << 24) | (second << 16) | (first << 8) | first;
+}
+
+template <int W> __device__ __forceinline__ void slab_expand_hidden(const SlabRaw &r, int q, const uint32_t (&sel8)[4], bf16x8 (&hi)[4], bf16x8 (&lo)[4]) {
     const uint32_t words[8] = {r.w01[0], r.w01[1], r.w23[0], r.w23[1], r.w45[0], r.w45[1], r.w67[0], r.w67[1]};
     uint32_t hi_w[4][4], lo_w[4][4];     // [operand j][row pair p]
 #pragma unroll
@@ -174,8 +225,7 @@ template <int W> __device__ __forceinline__ void slab_expand_hidden(const SlabRa
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 // both codes of column j, each in both bytes of its half
-                const uint32_t sel = ((4u + j) << 24) | ((4u + j) << 16) | ((uint32_t)j << 8) | (uint32_t)j;
-                const uint32_t both = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], sel);
+                const uint32_t both = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], sel8[j]);
                 hi_w[j][p] = (both & 0x807f807fu) | field;
                 lo_w[j][p] = (both & 0x80008000u) | field;
             }

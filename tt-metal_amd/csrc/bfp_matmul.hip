@@ -211,7 +211,8 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
         wait_slab(raw);
         if (refill) fetch(stage_tag);
         bf16x8 hi[4], lo[4];
-        slab_expand_hidden<W>(raw, q, hi, lo);
+        const uint32_t sel8[4] = {hidden_pair_selector(0, false), hidden_pair_selector(1, false), hidden_pair_selector(2, false), hidden_pair_selector(3, false)};
+        slab_expand_hidden<W>(raw, q, sel8, hi, lo);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
@@ -435,8 +436,9 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
 //   c32 / 8.  The activations are the A operand of the same instruction: row c32 of the band, the same 8 k.
 //   One workgroup = one k range of one output group (split >= 1); after the loop acc[j][i] is row 8(i/4) + 4kh + i%4,
 //   column 4*c32 + j.  Wavefront w keeps rows 8w..8w+7 of the workgroup's sums.
-// A stage of the LDS ring holds the two tile pairs of a unit, each laid out as Wfmt describes; the second pair is
-// shifted by PAIR_PAD bytes so that the 64 lanes of one ds_read2_b32 fall into 64 different banks.
+// A stage of the LDS ring holds the four tiles of a unit as WideFmt describes (bfp_dequant.h): as they lie in memory,
+// fetched so that four neighbouring lanes ask for one aligned 64-byte piece, and placed so that the 64 lanes of one
+// ds_read2_b32 fall into 64 different banks.
 // ---------------------------------------------------------------------------------------------------------
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 constexpr int WIDE_TILES = 4;
@@ -455,27 +457,27 @@ constexpr size_t WIDE_SLOT_BYTES = 32 * WIDE_COLS * sizeof(float);
 
 template <int W, int ACT>
 __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const MatmulDev p) {
-    using F = Wfmt<W>;
-    constexpr int PAIR_PAD = W == 7 ? 64 : 128;
-    constexpr int PAIR_STRIDE = F::stage_bytes + PAIR_PAD;
-    constexpr int UNIT_BYTES = 2 * PAIR_STRIDE;
+    using F = WideFmt<W>;
+    constexpr int UNIT_BYTES = F::unit_bytes;
     constexpr int WAVE_LDS = WIDE_STAGES * UNIT_BYTES;
     constexpr int LDS_BYTES = WIDE_REDUCE_BYTES > WAVES * WAVE_LDS ? WIDE_REDUCE_BYTES : WAVES * WAVE_LDS;
     constexpr int NLOAD = F::loads;
-    constexpr int PER = 2 * NLOAD + 2;                 // vector-memory requests per unit
+    constexpr int PER = NLOAD + 2;                     // vector-memory requests per unit
     __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
 
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: branches on it are uniform
     const int c32 = lane & 31, kh = lane >> 5;
-    const int t_of_lane = c32 >> 3, pair = t_of_lane >> 1, t_in = t_of_lane & 1, fc = (c32 >> 2) & 1, q = c32 & 3;
+    const int t_of_lane = c32 >> 3, fc = (c32 >> 2) & 1, q = c32 & 3;
 
     uint32_t chunk_of[NLOAD];
-    stage_chunks<W>(lane, chunk_of);
-    // this lane's LDS addresses for slab 0 of stage 0; slab 1 is 32 bytes (exponents) / 4 faces (mantissas) further
-    const uint32_t exp_at = lds_base + wave * WAVE_LDS + pair * PAIR_STRIDE + F::exp_base + t_in * 64 + fc * 16 + kh * 8;
-    const uint32_t mant_at = lds_base + wave * WAVE_LDS + pair * PAIR_STRIDE + (t_in * 2 + fc) * F::face_stride + (kh * 8) * F::row_bytes +
-                             (W == 7 ? q * 4 : (q >> 1) * 4);
+    wide_stage_chunks<W>(lane, chunk_of);
+    // this lane's LDS addresses for slab 0 of stage 0; slab 1 is 32 bytes (exponents) / 2 faces (mantissas) further
+    const uint32_t tile_at = lds_base + wave * WAVE_LDS + wide_tile_at<W>(t_of_lane);
+    const uint32_t exp_at = tile_at + fc * 16 + kh * 8;
+    const uint32_t mant_at = tile_at + 64 + fc * F::face_bytes + (kh * 8) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);
+    // BFP8: lanes with fc = 1 find the two rows of a pair in the other order (WideFmt); the selectors take that out again
+    const uint32_t sel8[4] = {hidden_pair_selector(0, fc != 0), hidden_pair_selector(1, fc != 0), hidden_pair_selector(2, fc != 0), hidden_pair_selector(3, fc != 0)};
 
     // ---- this workgroup's output group and k range ---------------------------------------------------------
     const uint32_t me = blockIdx.x;
@@ -488,11 +490,9 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
 
     // tiles past the matrix edge repeat the last chunk that exists and are never stored
     const uint32_t chunks_valid = n_valid * F::chunks;
-    uint32_t src_off[2][NLOAD];
+    uint32_t src_off[NLOAD];
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
-#pragma unroll
-        for (int l = 0; l < NLOAD; ++l) src_off[pr][l] = min(pr * 2 * F::chunks + chunk_of[l], chunks_valid - 1) * 16;
+    for (int l = 0; l < NLOAD; ++l) src_off[l] = min(chunk_of[l], chunks_valid - 1) * 16;
     const uint8_t *wptr = p.b + ((uint64_t)(p.b_batch == 1 ? 0 : bb) * p.kt * p.nt + (uint64_t)(k_begin + wave) * p.nt + nt0) * F::tile_bytes;
     const uint64_t w_step = (uint64_t)WAVES * p.nt * F::tile_bytes;
     // activations of one unit for this lane: row c32 of the band, k = kt*32 + 16s + 8kh .. + 7 for s = 0, 1;
@@ -532,12 +532,10 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     auto fetch = [&](auto stage_tag) __attribute__((always_inline)) {
         constexpr int S = decltype(stage_tag)::value;
 #pragma unroll
-        for (int pr = 0; pr < 2; ++pr)
-#pragma unroll
-            for (int l = 0; l < NLOAD; ++l)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[pr][l]),
-                                                 (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * UNIT_BYTES + pr * PAIR_STRIDE + l * 1024),
-                                                 16, 0, WEIGHTS_ONCE);
+        for (int l = 0; l < NLOAD; ++l)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[l]),
+                                             (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * UNIT_BYTES + (l / F::run_loads) * F::run_stride + (l % F::run_loads) * 1024),
+                                             16, 0, WEIGHTS_ONCE);
         wptr += w_step;
         asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][0]) : "v"(aptr) : "memory");
         asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][1]) : "v"(aptr + a_second) : "memory");
@@ -559,7 +557,7 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
             }
         SlabRaw raw0, raw1;
         slab_read<W, S * UNIT_BYTES, S * UNIT_BYTES>(exp_at, mant_at, raw0);
-        slab_read<W, S * UNIT_BYTES + 32, S * UNIT_BYTES + 4 * F::face_stride>(exp_at, mant_at, raw1);
+        slab_read<W, S * UNIT_BYTES + 32, S * UNIT_BYTES + 2 * F::face_bytes>(exp_at, mant_at, raw1);
         wait_slabs(raw0, raw1);
         if (refill) fetch(stage_tag);
         // hidden-one form (bfp_dequant.h): A.W = 2 (A.hi - A.lo); the subtraction is an MFMA with the negated activations
@@ -569,12 +567,12 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         for (int s = 0; s < 2; ++s)
 #pragma unroll
             for (int e = 0; e < 4; ++e) a_neg[s][e] = a_now[s][e] ^ 0x80008000u;
-        slab_expand_hidden<W>(raw0, q, hi, lo);
+        slab_expand_hidden<W>(raw0, q, sel8, hi, lo);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[0]), hi[j], acc[j], 0, 0, 0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[0]), lo[j], acc[j], 0, 0, 0);
-        slab_expand_hidden<W>(raw1, q, hi, lo);
+        slab_expand_hidden<W>(raw1, q, sel8, hi, lo);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[1]), hi[j], acc[j], 0, 0, 0);
 #pragma unroll
