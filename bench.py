@@ -2,6 +2,7 @@
 """Benchmark of the block-float hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--legs all|primary|none]
+    python bench.py --summarise trace KERNEL_TRACE.csv | pmc COUNTERS.csv [KERNEL] | traffic FETCH.csv WRITE.csv
 
 A "step" is one pass of the primary workload over one batch of synthetic input with everything resident in HBM:
 by default the Falcon-7B decode MLP (bf16 [32,4544] x BFP8_B [4544,18176], then [32,18176] x BFP8_B [18176,4544]).
@@ -27,16 +28,11 @@ for _p in (ROOT, os.path.join(ROOT, "tt-metal_amd")):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 ROTATE_BYTES = 512 << 20
-# HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, on this same command;
-# summary and scaling factors in profiles/bench_all_workloads_hbm_traffic.md).  Counters cannot be read from inside
-# this process, so the figures of that run are carried here; None where the run could not tell two launches apart.
-MEASURED_TRAFFIC_BYTES = {
-    "falcon_h_to_4h": 114_087_000, "falcon_4h_to_h": 111_008_000, "mistral_qkv": 41_964_000, "mistral_o": 31_525_000,
-    "mistral_gate": 57_695_000, "mistral_up": 57_695_000, "mistral_down": 47_651_000,
-    "prefill_ff1": 625_057_000, "bert_bmm": 35_619_000,
-    "pack_bfp4_4k_pack": 76_677_000, "pack_bfp4_4k_unpack": 76_642_000,
-    "pack_bfp8_1k_pack": 5_446_000 * 1024 // 1000, "pack_bfp8_1k_unpack": 5_276_000 * 1024 // 1000,
-}
+# HBM bytes per launch come from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, on this same command
+# with --counter-calibration).  Counters cannot be read from inside this process: `bench.py --summarise traffic FETCH.csv
+# WRITE.csv` turns the two counter files into the summary below, and every run reads roofline.traffic from it (null for a
+# leg the summary does not list).
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "bench_all_workloads_hbm_traffic.md")
 WORKLOAD_NAMES = {
     "decode_falcon": "decode_falcon: bf16 [32,4544] x BFP8_B [4544,18176], then [32,18176] x BFP8_B [18176,4544] (Falcon-7B decode MLP)",
     "decode_mistral": "decode_mistral: M=32 bf16 x fused QKV / O (BFP8_B) and gate / up / down (BFP4_B) of a Mistral-7B layer",
@@ -59,11 +55,26 @@ def parse_args():
     ap.add_argument("--counter-calibration", action="store_true",
                     help="first launch a plain elementwise copy of 256 MiB three times, so that a hardware-counter run "
                          "(FETCH_SIZE / WRITE_SIZE) can be scaled by what the same counter reads for a known transfer")
+    ap.add_argument("--summarise", nargs="+", metavar=("KIND", "FILE"),
+                    help="no benchmark: print a summary of rocprofv3 output of this command (trace FILE | pmc FILE [KERNEL] | traffic FETCH WRITE)")
     return ap.parse_args()
 
 
 def main():
     args = parse_args()
+    if args.summarise:
+        from ttmi import counters
+
+        kind, files = args.summarise[0], args.summarise[1:]
+        if kind == "trace" and len(files) == 1:
+            print(counters.summarise_trace(files[0]))
+        elif kind == "pmc" and len(files) in (1, 2):
+            print(counters.summarise_pmc(files[0], files[1] if len(files) == 2 else None))
+        elif kind == "traffic" and len(files) == 2:
+            print(counters.traffic_lines(files[0], files[1]))
+        else:
+            sys.exit("bench.py --summarise trace FILE | pmc FILE [KERNEL] | traffic FETCH_FILE WRITE_FILE")
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1", file=sys.stderr)
         sys.exit(2)
@@ -380,8 +391,11 @@ def main():
                    "host_threads": host_threads,
                    "to_torch_unpack_melem_s_1thread": round(x.size / t_unpack / 1e6, 1)}
 
+    from ttmi import counters
+
+    measured_traffic = counters.read_traffic(TRAFFIC_SUMMARY)
     for leg in (l for wl in order for l in results[wl]):
-        leg["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(leg["workload"])
+        leg["roofline"]["traffic"] = measured_traffic.get(leg["workload"])
 
     line = {
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,

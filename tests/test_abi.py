@@ -172,3 +172,60 @@ def test_test_knobs_are_validated_and_cleared(knobs):
     assert ws(1, 32, 64, 64, 3) == 2 * 1 * 4096                 # forced onto the expanding kernel: one 64-column group, two k tiles
     L.ttmi_test_set_knob.restype = ctypes.c_int
     assert L.ttmi_test_set_knob(99, 0, 1) == 1 and b"unknown test knob" in L.ttmi_last_error()
+
+
+@pytest.mark.parametrize("bits,tile_bytes", [(7, 1088), (3, 576)])
+def test_lds_stage_of_the_wide_kernel(bits, tile_bytes):
+    """The LDS stage of the 128-column GEMM kernel, from the addresses its own code computes (test entry point): every
+    mantissa word and exponent byte a lane reads is the one of its tile, face, k row and column quad; the 64 lanes of every
+    pass of a ds_read2_b32 and of the exponent read fall into 64 different banks of 4 bytes; and every four neighbouring
+    lanes of a load fetch one aligned 64-byte piece of memory (what the vector memory pipe coalesces)."""
+    from ttmi import capi
+
+    if not os.path.exists(capi.LIB_PATH):
+        pytest.skip("libttmi.so not built")
+    L = capi.lib()
+    L.ttmi_test_wide_layout.restype = None
+    L.ttmi_test_wide_layout.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_uint32)]
+    lanes = []
+    for lane in range(64):
+        out = (ctypes.c_uint32 * 16)()
+        L.ttmi_test_wide_layout(bits, lane, out)
+        lanes.append([int(x) for x in out])
+    loads, load_stride, unit_bytes, slab_bytes, row_step = lanes[0][:5]
+    pair_offsets = lanes[0][5:9]
+    row_bytes, face_bytes = (16, 256) if bits == 7 else (8, 128)
+    assert row_step == row_bytes
+    stage = {}                                               # LDS byte of the stage -> byte of the unit's 4 tiles in memory
+    for l in range(loads):
+        for lane in range(64):
+            chunk = lanes[lane][11 + l]
+            assert chunk < 4 * tile_bytes // 16
+            for b in range(16):
+                at = l * load_stride + lane * 16 + b
+                assert at < unit_bytes
+                stage[at] = chunk * 16 + b
+        for quad in range(16):
+            assert len({lanes[quad * 4 + j][11 + l] // 4 for j in range(4)}) == 1
+    for s in range(2):
+        exp_banks = set()
+        for lane in range(64):
+            c32, kh = lane & 31, lane >> 5
+            t, fc = c32 >> 3, (c32 >> 2) & 1
+            at = lanes[lane][9] + 32 * s
+            assert [stage[at + b] for b in range(8)] == [t * tile_bytes + (2 * s + fc) * 16 + kh * 8 + b for b in range(8)]
+            exp_banks.update({(at // 4) % 64, (at // 4 + 1) % 64})
+        assert len(exp_banks) == 32                           # 16 different addresses of 8 bytes, the four lanes of a column quad share one
+        for i in range(4):
+            for second in range(2):
+                banks = set()
+                for lane in range(64):
+                    c32, kh = lane & 31, lane >> 5
+                    t, fc, q = c32 >> 3, (c32 >> 2) & 1, c32 & 3
+                    word = q if bits == 7 else q >> 1
+                    at = lanes[lane][10] + s * slab_bytes + pair_offsets[i] + second * row_step
+                    want = t * tile_bytes + 64 + (2 * s + fc) * face_bytes + (8 * kh + 2 * i + second) * row_bytes + word * 4
+                    assert [stage[at + b] for b in range(4)] == [want + b for b in range(4)]
+                    banks.add(((at // 4) % 64, at))
+                assert len({b for b, _ in banks}) == len({a for _, a in banks})     # different addresses, different banks
+                assert len({a for _, a in banks}) == (64 if bits == 7 else 32)         # BFP4: two lanes share a word

@@ -35,49 +35,67 @@ template <> struct Wfmt<3> {
     static constexpr float unscale = 1.0f / 4.0f;                           // 2^(127 - bias_exp)
 };
 
-// LDS stage of one wavefront of the 128-column kernel = the 4 adjacent packed tiles of one unit, brought in as `runs`
-// contiguous runs of tiles, each run by run_loads direct global->LDS loads in which lane l takes chunk l of the run: four
-// neighbouring lanes then ask for one aligned 64-byte piece of memory, which is what the address coalescing of the
-// vector memory pipe wants (with a pad slot per face, as Wfmt has it, every piece is split over two groups of four
-// lanes, and the loads, not the memory, bound the kernel: measured 2 us of 17 on the Falcon h_to_4h shape).  A run lies in
-// LDS as it lies in memory (per tile: 64 exponent bytes, then the faces), and what one ds_read touches is kept in
-// different banks without pad slots:
-//   BFP8  run = 2 tiles.  In faces with fc = 1 every lane fetches the chunk (= face row) next to its own, so that rows
-//         2i and 2i + 1 lie swapped: fc moves a lane by 16 bytes.  The second run starts 32 bytes off a multiple of 256.
-//         (tile: 64 bytes, row group kh: 128 bytes, word q: 4 bytes: all 64 lanes of a ds_read2_b32 in different banks.)
-//         Lanes with fc = 1 get the rows of a pair in the other order; slab_expand_hidden takes that out again in the
-//         byte selectors of its v_perm_b32.
-//   BFP4  run = 1 tile (36 of the 64 lanes fetch).  Run r starts 48 r bytes off a multiple of 1024: tile 16-byte phase
-//         3r mod 4, face column fc: 128 bytes, row group kh: 64 bytes, word q / 2: 4 bytes.
+// LDS stage of one wavefront of the 128-column kernel = the 4 adjacent packed tiles of one unit, brought in by direct
+// global->LDS loads in which four neighbouring lanes always fetch one aligned 64-byte piece of memory ("quad": 4 face rows
+// of BFP8, 8 of BFP4).  That is what the address coalescing of the vector memory pipe wants; with a pad slot per face, as
+// Wfmt has it, every piece is split over two groups of four lanes, and the loads, not the memory, bound the kernel
+// (measured on the Falcon h_to_4h shape without arithmetic: 17.4 us against 15.4 us).  What one ds_read touches still
+// lies in 64 different banks, because a quad may go to any quad position of its load and every load may start at any
+// multiple of 16 bytes:
+//   tile t (0..3) has a load of its own that starts 16 t bytes off a multiple of 64, so tiles differ in the 16-byte phase;
+//   BFP8  the 16 quads of a tile's faces (memory order: face f = 2s + fc, row group kh, row quad rq) are placed at
+//         position 8s + 4rq + 2fc + kh: one pass of a ds_read2_b32 (s, rq and the row inside the quad are common to all
+//         lanes) finds the four (fc, kh) of a tile in four different 64-byte phases.  The exponents of the four tiles come
+//         with a fifth load (16 lanes).
+//   BFP4  a tile is 9 quads in memory order (exponents, then face f = 2s + fc, row group kh): fc and kh already give four
+//         different 64-byte phases.
 template <int W> struct WideFmt;
 template <> struct WideFmt<7> {
-    static constexpr int tile_bytes = 1088, chunks = 68, face_chunks = 16, face_bytes = 256, row_bytes = 16;
-    static constexpr int run_tiles = 2, runs = 2, run_loads = 3, loads = runs * run_loads;
-    static constexpr int run_stride = run_loads * 1024 + 32, unit_bytes = runs * run_stride;
+    static constexpr int tile_bytes = 1088, chunks = 68, row_bytes = 16;
+    static constexpr int loads = 5;                                    // 4 tiles' faces + the exponents
+    static constexpr int load_stride = 1024 + 16;
+    static constexpr int exp_base = 4 * load_stride, unit_bytes = exp_base + 1024;
+    static constexpr int slab_bytes = 512;                             // mantissas of slab 1 lie this far behind slab 0
+    // byte offsets of the four ds_read2_b32 of a slab (rows 2i and 2i + 1) from the lane's address
+    static constexpr int pair_offset(int i) { return (i >> 1) * 256 + (i & 1) * 32; }
+    static constexpr int row_step = 16;
 };
 template <> struct WideFmt<3> {
-    static constexpr int tile_bytes = 576, chunks = 36, face_chunks = 8, face_bytes = 128, row_bytes = 8;
-    static constexpr int run_tiles = 1, runs = 4, run_loads = 1, loads = runs * run_loads;
-    static constexpr int run_stride = run_loads * 1024 + 48, unit_bytes = runs * run_stride;
+    static constexpr int tile_bytes = 576, chunks = 36, row_bytes = 8;
+    static constexpr int loads = 4;                                    // one per tile: 36 of the 64 lanes fetch
+    static constexpr int load_stride = 1024 + 48;                      // 48 t mod 64 = 0, 48, 32, 16
+    static constexpr int exp_base = 0, unit_bytes = 4 * load_stride;
+    static constexpr int slab_bytes = 256;
+    static constexpr int pair_offset(int i) { return i * 16; }
+    static constexpr int row_step = 8;
 };
 // chunk (16 bytes, counted from the start of the unit's 4 tiles) that this lane fetches in load l of a unit
-template <int W> __device__ __forceinline__ void wide_stage_chunks(int lane, uint32_t (&chunk_of)[WideFmt<W>::loads]) {
+template <int W> __host__ __device__ __forceinline__ void wide_stage_chunks(int lane, uint32_t (&chunk_of)[WideFmt<W>::loads]) {
     using F = WideFmt<W>;
 #pragma unroll
     for (int l = 0; l < F::loads; ++l) {
-        const uint32_t run = l / F::run_loads;
-        uint32_t c = min((uint32_t)((l % F::run_loads) * 64 + lane), (uint32_t)(F::run_tiles * F::chunks - 1));   // idle lanes repeat the last chunk
-        if (W == 7) {
-            const uint32_t in_tile = c % F::chunks;
-            if (in_tile >= 4 && (((in_tile - 4) / F::face_chunks) & 1)) c ^= 1;
+        uint32_t c;
+        if (W == 7 && l < 4) {
+            const uint32_t pos = lane >> 2, s = pos >> 3, rq = (pos >> 2) & 1, fc = (pos >> 1) & 1, kh = pos & 1;
+            c = l * F::chunks + 4 + 4 * (8 * s + 4 * fc + 2 * kh + rq) + (lane & 3);
+        } else if (W == 7) {
+            const uint32_t e = lane < 15 ? (uint32_t)lane : 15u;        // idle lanes repeat the last chunk
+            c = (e >> 2) * F::chunks + (e & 3);
+        } else {
+            c = l * F::chunks + (lane < F::chunks - 1 ? (uint32_t)lane : (uint32_t)F::chunks - 1);
         }
-        chunk_of[l] = run * F::run_tiles * F::chunks + c;
+        chunk_of[l] = c;
     }
 }
-// byte offset inside a stage of tile t (0..3) of the unit
-template <int W> __device__ __forceinline__ uint32_t wide_tile_at(int t) {
+// this lane's LDS byte offsets inside a stage for slab 0: exponents (8 bytes: k rows 8kh .. 8kh + 7 of its face) and
+// mantissa word of k row 8kh (lane: tile t, face column fc, word q, row group kh)
+template <int W> __host__ __device__ __forceinline__ uint32_t wide_exp_at(int t, int fc, int kh) {
     using F = WideFmt<W>;
-    return (t / F::run_tiles) * F::run_stride + (t % F::run_tiles) * F::tile_bytes;
+    return (W == 7 ? F::exp_base + t * 64 : t * F::load_stride) + fc * 16 + kh * 8;
+}
+template <int W> __host__ __device__ __forceinline__ uint32_t wide_mant_at(int t, int fc, int q, int kh) {
+    using F = WideFmt<W>;
+    return W == 7 ? t * F::load_stride + (2 * fc + kh) * 64 + q * 4 : t * F::load_stride + 64 + fc * 128 + kh * 64 + (q >> 1) * 4;
 }
 
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
@@ -179,6 +197,17 @@ template <int W, int EXP_OFF, int MANT_OFF> __device__ __forceinline__ void slab
     asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w45) : "v"(mant), "n"(4 * R), "n"(5 * R));
     asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w67) : "v"(mant), "n"(6 * R), "n"(7 * R));
 }
+// the same for a stage laid out as WideFmt describes
+template <int W, int EXP_OFF, int MANT_OFF> __device__ __forceinline__ void wide_slab_read(uint32_t exp_at, uint32_t mant_at, SlabRaw &r) {
+    using F = WideFmt<W>;
+    constexpr int R = F::row_step / 4;
+    const uint32_t mant = mant_at + MANT_OFF;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(r.e01) : "v"(exp_at), "n"(EXP_OFF));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w01) : "v"(mant), "n"(F::pair_offset(0) / 4), "n"(F::pair_offset(0) / 4 + R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w23) : "v"(mant), "n"(F::pair_offset(1) / 4), "n"(F::pair_offset(1) / 4 + R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w45) : "v"(mant), "n"(F::pair_offset(2) / 4), "n"(F::pair_offset(2) / 4 + R));
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r.w67) : "v"(mant), "n"(F::pair_offset(3) / 4), "n"(F::pair_offset(3) / 4 + R));
+}
 __device__ __forceinline__ void wait_slab(SlabRaw &a) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.e01), "+v"(a.w01), "+v"(a.w23), "+v"(a.w45), "+v"(a.w67)::"memory");
 }
@@ -209,13 +238,7 @@ __device__ __forceinline__ uint32_t hidden_pair_field(const u32x2 e01, int p) {
     return spread << 7;
 }
 
-// byte selectors of the BFP8 expansion for operand j: with `swapped` the two words of a row pair arrive in the other order
-__device__ __forceinline__ uint32_t hidden_pair_selector(int j, bool swapped) {
-    const uint32_t first = swapped ? 4u + j : (uint32_t)j, second = swapped ? (uint32_t)j : 4u + j;   // bytes 0..3: words[2p], 4..7: words[2p + 1]
-    return (second << 24) | (second << 16) | (first << 8) | first;
-}
-
-template <int W> __device__ __forceinline__ void slab_expand_hidden(const SlabRaw &r, int q, const uint32_t (&sel8)[4], bf16x8 (&hi)[4], bf16x8 (&lo)[4]) {
+template <int W> __device__ __forceinline__ void slab_expand_hidden(const SlabRaw &r, int q, bf16x8 (&hi)[4], bf16x8 (&lo)[4]) {
     const uint32_t words[8] = {r.w01[0], r.w01[1], r.w23[0], r.w23[1], r.w45[0], r.w45[1], r.w67[0], r.w67[1]};
     uint32_t hi_w[4][4], lo_w[4][4];     // [operand j][row pair p]
 #pragma unroll
@@ -225,7 +248,8 @@ template <int W> __device__ __forceinline__ void slab_expand_hidden(const SlabRa
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 // both codes of column j, each in both bytes of its half
-                const uint32_t both = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], sel8[j]);
+                const uint32_t sel = ((4u + j) << 24) | ((4u + j) << 16) | ((uint32_t)j << 8) | (uint32_t)j;
+                const uint32_t both = __builtin_amdgcn_perm(words[2 * p + 1], words[2 * p], sel);
                 hi_w[j][p] = (both & 0x807f807fu) | field;
                 lo_w[j][p] = (both & 0x80008000u) | field;
             }

@@ -11,10 +11,11 @@
 //   unit       one k-tile (32 rows of W) of one output group; an output group is a 32-row band of one batch slice
 //              times 64 columns (2 adjacent packed tiles, one contiguous run in memory)
 //   wavefront  brings the 2 tiles of a unit into its private LDS ring with direct global->LDS loads (no staging
-//              registers), two units ahead of the arithmetic; per unit it builds four B operands and issues eight
-//              v_mfma_f32_16x16x32_bf16.  Lane (c, g) — c = lane % 16, g = lane / 16 — holds, for operand j, column
-//              4c+j of the group and k rows 8g..8g+7: byte j of the 8 mantissa words it reads from LDS.  The packed
-//              layout (16 consecutive columns of one k row share a word run) never has to be transposed.
+//              registers), units ahead of the arithmetic; per unit it builds four pairs of B operands in hidden-one form
+//              (bfp_dequant.h: no conversion, no multiplication) and issues sixteen v_mfma_f32_16x16x32_bf16.  Lane
+//              (c, g) — c = lane % 16, g = lane / 16 — holds, for operand j, column 4c+j of the group and k rows
+//              8g..8g+7: byte j of the 8 mantissa words it reads from LDS.  The packed layout (16 consecutive columns of
+//              one k row share a word run) never has to be transposed.
 //   workgroup  4 wavefronts take the units of a contiguous range round-robin, add their partial sums through LDS
 //              and store; the range is one of the nearly equal parts the host cuts every output's k range into, as
 //              many as fill the chip.  Outputs whose k range is shared between workgroups are finished by the
@@ -211,8 +212,7 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void matmul_stream_kernel(const Ma
         wait_slab(raw);
         if (refill) fetch(stage_tag);
         bf16x8 hi[4], lo[4];
-        const uint32_t sel8[4] = {hidden_pair_selector(0, false), hidden_pair_selector(1, false), hidden_pair_selector(2, false), hidden_pair_selector(3, false)};
-        slab_expand_hidden<W>(raw, q, sel8, hi, lo);
+        slab_expand_hidden<W>(raw, q, hi, lo);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
@@ -472,12 +472,9 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
 
     uint32_t chunk_of[NLOAD];
     wide_stage_chunks<W>(lane, chunk_of);
-    // this lane's LDS addresses for slab 0 of stage 0; slab 1 is 32 bytes (exponents) / 2 faces (mantissas) further
-    const uint32_t tile_at = lds_base + wave * WAVE_LDS + wide_tile_at<W>(t_of_lane);
-    const uint32_t exp_at = tile_at + fc * 16 + kh * 8;
-    const uint32_t mant_at = tile_at + 64 + fc * F::face_bytes + (kh * 8) * F::row_bytes + (W == 7 ? q * 4 : (q >> 1) * 4);
-    // BFP8: lanes with fc = 1 find the two rows of a pair in the other order (WideFmt); the selectors take that out again
-    const uint32_t sel8[4] = {hidden_pair_selector(0, fc != 0), hidden_pair_selector(1, fc != 0), hidden_pair_selector(2, fc != 0), hidden_pair_selector(3, fc != 0)};
+    // this lane's LDS addresses for slab 0 of stage 0; slab 1 is 32 bytes (exponents) / F::slab_bytes (mantissas) further
+    const uint32_t exp_at = lds_base + wave * WAVE_LDS + wide_exp_at<W>(t_of_lane, fc, kh);
+    const uint32_t mant_at = lds_base + wave * WAVE_LDS + wide_mant_at<W>(t_of_lane, fc, q, kh);
 
     // ---- this workgroup's output group and k range ---------------------------------------------------------
     const uint32_t me = blockIdx.x;
@@ -534,7 +531,7 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
 #pragma unroll
         for (int l = 0; l < NLOAD; ++l)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[l]),
-                                             (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * UNIT_BYTES + (l / F::run_loads) * F::run_stride + (l % F::run_loads) * 1024),
+                                             (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * UNIT_BYTES + l * F::load_stride),
                                              16, 0, WEIGHTS_ONCE);
         wptr += w_step;
         asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][0]) : "v"(aptr) : "memory");
@@ -556,8 +553,8 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
                 a_now[s][e] = moved;
             }
         SlabRaw raw0, raw1;
-        slab_read<W, S * UNIT_BYTES, S * UNIT_BYTES>(exp_at, mant_at, raw0);
-        slab_read<W, S * UNIT_BYTES + 32, S * UNIT_BYTES + 2 * F::face_bytes>(exp_at, mant_at, raw1);
+        wide_slab_read<W, S * UNIT_BYTES, S * UNIT_BYTES>(exp_at, mant_at, raw0);
+        wide_slab_read<W, S * UNIT_BYTES + 32, S * UNIT_BYTES + F::slab_bytes>(exp_at, mant_at, raw1);
         wait_slabs(raw0, raw1);
         if (refill) fetch(stage_tag);
         // hidden-one form (bfp_dequant.h): A.W = 2 (A.hi - A.lo); the subtraction is an MFMA with the negated activations
@@ -567,12 +564,12 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         for (int s = 0; s < 2; ++s)
 #pragma unroll
             for (int e = 0; e < 4; ++e) a_neg[s][e] = a_now[s][e] ^ 0x80008000u;
-        slab_expand_hidden<W>(raw0, q, sel8, hi, lo);
+        slab_expand_hidden<W>(raw0, q, hi, lo);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[0]), hi[j], acc[j], 0, 0, 0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[0]), lo[j], acc[j], 0, 0, 0);
-        slab_expand_hidden<W>(raw1, q, sel8, hi, lo);
+        slab_expand_hidden<W>(raw1, q, hi, lo);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[1]), hi[j], acc[j], 0, 0, 0);
 #pragma unroll
@@ -931,11 +928,29 @@ extern "C" int ttmi_matmul_bfp_static(const void *a, int a_layout, const uint32_
 
 // Test entry points (not declared in include/ttmi.h): the decomposition the host chooses for a shape, and the two index
 // functions the kernels cut the work with, so that their invariants can be checked without a GPU.
+// Test entry point: the LDS stage of the 128-column kernel as its code computes it, for lane `lane` of a wavefront.
+//   out[0] loads per unit, out[1] bytes between the LDS destinations of consecutive loads, out[2] stage bytes,
+//   out[3] bytes from slab 0 to slab 1 (mantissas), out[4] bytes between the two rows of a ds_read2_b32,
+//   out[5..8] byte offsets of the four ds_read2_b32 of a slab, out[9] exponent address, out[10] mantissa address
+//   (both inside the stage, slab 0), out[11..] the chunk of the unit that the lane fetches in every load
+template <int W> static void wide_layout_of(int lane, uint32_t *out) {
+    using F = ttmi::WideFmt<W>;
+    const int c32 = lane & 31, kh = lane >> 5, t = c32 >> 3, fc = (c32 >> 2) & 1, q = c32 & 3;
+    out[0] = F::loads; out[1] = F::load_stride; out[2] = F::unit_bytes; out[3] = F::slab_bytes; out[4] = F::row_step;
+    for (int i = 0; i < 4; ++i) out[5 + i] = F::pair_offset(i);
+    out[9] = ttmi::wide_exp_at<W>(t, fc, kh); out[10] = ttmi::wide_mant_at<W>(t, fc, q, kh);
+    uint32_t chunk_of[F::loads];
+    ttmi::wide_stage_chunks<W>(lane, chunk_of);
+    for (int l = 0; l < F::loads; ++l) out[11 + l] = chunk_of[l];
+}
 extern "C" {
 __attribute__((visibility("default"))) void ttmi_test_stream_decomposition(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int wide,
                                                                            uint32_t out[4]) {
     const ttmi::Decomposition d = ttmi::decompose(batch, m, k, n, wide != 0);
     out[0] = (uint32_t)d.groups; out[1] = d.kt; out[2] = d.split; out[3] = d.workgroups;
+}
+__attribute__((visibility("default"))) void ttmi_test_wide_layout(int mantissa_bits, int lane, uint32_t out[16]) {
+    if (mantissa_bits == 7) wide_layout_of<7>(lane, out); else wide_layout_of<3>(lane, out);
 }
 __attribute__((visibility("default"))) uint32_t ttmi_test_range_start(uint32_t kt, uint32_t split, uint32_t i) { return ttmi::range_start(kt, split, i); }
 __attribute__((visibility("default"))) uint32_t ttmi_test_workgroup_of(uint32_t kt, uint32_t split, uint32_t unit) { return ttmi::workgroup_of(kt, split, unit); }
