@@ -157,10 +157,23 @@ def main():
 
         ms = time_loop(run, steps, warmup)
         roof = hbm_roofline(nbytes, ms) if hbm_bound else mfma_roofline(flops, ms)
+        vendor_ms = None
+        if not hbm_bound:
+            # for scale only: the vendor library's plain bf16 GEMM (torch.matmul -> hipBLASLt / rocBLAS) on the same M, K, N with
+            # dense bf16 weights already in memory, i.e. without any block-float work; the better of B as [K,N] and as [N,K]^T
+            dense = torch.randn((b, k, n), dtype=torch.bfloat16, device="cuda")
+            dense_t = dense.transpose(1, 2).contiguous()
+            a_dense = torch.randn((b, m, k), dtype=torch.bfloat16, device="cuda")
+            vendor_ms = min(time_loop(lambda i: torch.matmul(a_dense, dense), steps, 2),
+                            time_loop(lambda i: torch.matmul(a_dense, dense_t.transpose(1, 2)), steps, 2))
+            del dense, dense_t, a_dense
         leg = {"workload": name, "shape": [b, m, k, n], "weights": fmt, "ms": round(ms, 5),
                "tflops": round(flops / (ms * 1e-3) / 1e12, 2), "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1),
                "algorithmic_bytes": nbytes, "flops": flops, "weight_copies_rotated": ncopies,
                "layout": "row_major" if args.row_major else "tile", "roofline": roof}
+        if vendor_ms is not None:
+            leg["vendor_bf16_gemm_ms"] = round(vendor_ms, 5)
+            leg["vendor_bf16_gemm_frac"] = round(flops / (vendor_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
         return leg, (run, wcopies, acopies, c)
 
     def block_leg(name, steps, warmup, seed):

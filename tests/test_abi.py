@@ -178,7 +178,8 @@ def test_test_knobs_are_validated_and_cleared(knobs):
 def test_lds_stage_of_the_wide_kernel(bits, tile_bytes):
     """The LDS stage of the 128-column GEMM kernel, from the addresses its own code computes (test entry point): every
     mantissa word and exponent byte a lane reads is the one of its tile, face, k row and column quad; the 64 lanes of every
-    pass of a ds_read2_b32 and of the exponent read fall into 64 different banks of 4 bytes; and every four neighbouring
+    pass of a ds_read2_b32 and of the exponent read fall into 64 different banks of 4 bytes, and the 32 lanes of either half
+    into 32 different banks when only address bits 2..6 choose the bank; and every four neighbouring
     lanes of a load fetch one aligned 64-byte piece of memory (what the vector memory pipe coalesces)."""
     from ttmi import capi
 
@@ -229,3 +230,9 @@ def test_lds_stage_of_the_wide_kernel(bits, tile_bytes):
                     banks.add(((at // 4) % 64, at))
                 assert len({b for b, _ in banks}) == len({a for _, a in banks})     # different addresses, different banks
                 assert len({a for _, a in banks}) == (64 if bits == 7 else 32)         # BFP4: two lanes share a word
+                # the same for half a wavefront at a time on 32 banks (what the bank-conflict counter of the hardware fits)
+                for half in range(2):
+                    addresses = set()
+                    for lane in range(32 * half, 32 * half + 32):
+                        addresses.add(lanes[lane][10] + s * slab_bytes + pair_offsets[i] + second * row_step)
+                    assert len({(a // 4) % 32 for a in addresses}) == len(addresses)

@@ -318,8 +318,11 @@ def test_full_size_decode_gemms_on_three_streams():
                                          j["stream"].cuda_stream))
     torch.cuda.synchronize()
     for j in jobs:
-        for rep, out in enumerate(j["outs"]):
-            assert torch.equal(out.view(torch.int16), j["alone"].reshape(-1).view(torch.int16)), (j["n"], rep)
+        again = capi.matmul_bfp(j["a"], capi.TILE, j["w"], j["fmt"], 1, 1, j["m"], j["k"], j["n"], c_layout=capi.TILE)
+        want = j["alone"].reshape(-1).view(torch.int16)
+        differing = {"alone again": int((again.reshape(-1).view(torch.int16) != want).sum())}
+        differing.update({f"launch {rep}": int((out.view(torch.int16) != want).sum()) for rep, out in enumerate(j["outs"])})
+        assert not any(differing.values()), (j["n"], differing)
 
 
 def oracle_unpacked(oracle, fmt, words, k, n, batch=1):
@@ -512,3 +515,30 @@ def test_library_scratch_is_per_stream(oracle):
     for per_stream in results:
         for c in per_stream:
             assert torch.equal(c.view(torch.int16), want.view(torch.int16))
+
+
+def test_library_slots_beyond_the_first_launch_are_empty_too():
+    """The library's slot buffer grows geometrically, so a launch may find room for more slots than any launch before it
+    has used: those must be empty as well (the whole buffer is filled when it is new, not only what the first launch
+    needs).  Three GEMMs on a new stream whose slot needs are 64, 80 and 112 workgroups x 16 KB: the second makes the
+    buffer grow to 2 MB, the third fits without growing.  Each is compared with the same GEMM on a caller's workspace,
+    which is filled on every call."""
+    L = capi.lib()
+    stream = torch.cuda.Stream()
+    m, k = 32, 2048
+    for groups in (8, 10, 14):
+        n = 128 * groups
+        gen = torch.Generator(device="cuda").manual_seed(groups)
+        a = capi.tilize(torch.randn(m, k, device="cuda", generator=gen).bfloat16())
+        w = capi.pack_tensor(BFP8, torch.randn(k, n, device="cuda", generator=gen) * 0.02)
+        need = L.ttmi_matmul_bfp_workspace_bytes(1, m, k, n, BFP8)
+        assert need == groups * 8 * 16384
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        want = torch.empty(m * n, dtype=torch.bfloat16, device="cuda")
+        got = torch.empty(m * n, dtype=torch.bfloat16, device="cuda")
+        torch.cuda.synchronize()
+        args = (a.data_ptr(), capi.TILE, w.data_ptr(), BFP8, 1, 1, m, k, n, None, capi.ACT_NONE)
+        capi.check(L.ttmi_matmul_bfp(*args, want.data_ptr(), capi.TILE, capi.BFLOAT16, ws.data_ptr(), need, stream.cuda_stream))
+        capi.check(L.ttmi_matmul_bfp(*args, got.data_ptr(), capi.TILE, capi.BFLOAT16, None, 0, stream.cuda_stream))
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), groups

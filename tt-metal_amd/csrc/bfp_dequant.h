@@ -42,13 +42,16 @@ template <> struct Wfmt<3> {
 // (measured on the Falcon h_to_4h shape without arithmetic: 17.4 us against 15.4 us).  What one ds_read touches still
 // lies in 64 different banks, because a quad may go to any quad position of its load and every load may start at any
 // multiple of 16 bytes:
-//   tile t (0..3) has a load of its own that starts 16 t bytes off a multiple of 64, so tiles differ in the 16-byte phase;
+//   tile t (0..3) has a load of its own that starts 16 t (BFP4: 48 t) bytes off a multiple of 64, so tiles differ in the
+//         16-byte phase;
 //   BFP8  the 16 quads of a tile's faces (memory order: face f = 2s + fc, row group kh, row quad rq) are placed at
-//         position 8s + 4rq + 2fc + kh: one pass of a ds_read2_b32 (s, rq and the row inside the quad are common to all
-//         lanes) finds the four (fc, kh) of a tile in four different 64-byte phases.  The exponents of the four tiles come
-//         with a fifth load (16 lanes).
-//   BFP4  a tile is 9 quads in memory order (exponents, then face f = 2s + fc, row group kh): fc and kh already give four
-//         different 64-byte phases.
+//         position 8s + 4rq + 2kh + fc: one pass of a ds_read2_b32 (s, rq and the row inside the quad are common to all
+//         lanes) finds the four (kh, fc) of a tile in four different 64-byte phases, fc in the lowest.  The exponents of
+//         the four tiles come with a fifth load (16 lanes).
+//   BFP4  a tile is 9 quads: the exponents, then the quad of (face 2s + fc, row group kh) at position 1 + 4s + 2kh + fc.
+// With fc in the lowest position bit the 32 lanes of a half wavefront (kh is the upper half) already differ modulo 128
+// bytes: the counters say that a ds_read2_b32 is served half a wavefront at a time from 32 banks (a layout that was
+// conflict-free only modulo 256 bytes read 4 conflict cycles per instruction).
 template <int W> struct WideFmt;
 template <> struct WideFmt<7> {
     static constexpr int tile_bytes = 1088, chunks = 68, row_bytes = 16;
@@ -76,13 +79,16 @@ template <int W> __host__ __device__ __forceinline__ void wide_stage_chunks(int 
     for (int l = 0; l < F::loads; ++l) {
         uint32_t c;
         if (W == 7 && l < 4) {
-            const uint32_t pos = lane >> 2, s = pos >> 3, rq = (pos >> 2) & 1, fc = (pos >> 1) & 1, kh = pos & 1;
-            c = l * F::chunks + 4 + 4 * (8 * s + 4 * fc + 2 * kh + rq) + (lane & 3);
+            const uint32_t pos = lane >> 2, s = pos >> 3, rq = (pos >> 2) & 1, kh = (pos >> 1) & 1, fc = pos & 1;
+            c = l * F::chunks + 4 + 4 * (8 * s + 4 * fc + 2 * kh + rq) + (lane & 3);   // the memory quad that belongs at this position
         } else if (W == 7) {
             const uint32_t e = lane < 15 ? (uint32_t)lane : 15u;        // idle lanes repeat the last chunk
             c = (e >> 2) * F::chunks + (e & 3);
         } else {
-            c = l * F::chunks + (lane < F::chunks - 1 ? (uint32_t)lane : (uint32_t)F::chunks - 1);
+            const uint32_t slot = lane < F::chunks - 1 ? (uint32_t)lane : (uint32_t)F::chunks - 1;      // idle lanes repeat the last chunk
+            uint32_t quad = slot >> 2;
+            if (quad >= 1) { const uint32_t p = quad - 1, s = p >> 2, kh = (p >> 1) & 1, fc = p & 1; quad = 1 + 4 * s + 2 * fc + kh; }
+            c = l * F::chunks + 4 * quad + (slot & 3);
         }
         chunk_of[l] = c;
     }
@@ -95,7 +101,7 @@ template <int W> __host__ __device__ __forceinline__ uint32_t wide_exp_at(int t,
 }
 template <int W> __host__ __device__ __forceinline__ uint32_t wide_mant_at(int t, int fc, int q, int kh) {
     using F = WideFmt<W>;
-    return W == 7 ? t * F::load_stride + (2 * fc + kh) * 64 + q * 4 : t * F::load_stride + 64 + fc * 128 + kh * 64 + (q >> 1) * 4;
+    return W == 7 ? t * F::load_stride + (2 * kh + fc) * 64 + q * 4 : t * F::load_stride + 64 + (2 * kh + fc) * 64 + (q >> 1) * 4;
 }
 
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)

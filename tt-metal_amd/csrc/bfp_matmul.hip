@@ -798,21 +798,23 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     const size_t need = slot_bytes_needed(d, wide);
     void *slots = nullptr;
     bool fill = false;
+    size_t fill_bytes = need;
     if (need == 0) {
     } else if (x.workspace) {
         if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
         if (reinterpret_cast<uintptr_t>(x.workspace) & 255u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 256-byte aligned");
         slots = x.workspace;
         fill = true;                                // a caller's buffer may hold anything
-    } else if (int rc = scratch_get(SCRATCH_SLOTS, st, need, &slots, &fill)) {
+    } else if (int rc = scratch_get(SCRATCH_SLOTS, st, need, &slots, &fill, &fill_bytes)) {
         // the library's own slots, one buffer per stream: every word is SLOT_EMPTY once filled, and every launch that
         // completes leaves it that way
         return rc;
     }
     if (fill) {
-        // every slot of this launch becomes empty (with a kernel, not a memset node: the caller may be capturing the
-        // stream into a graph)
-        const uint32_t chunks = (uint32_t)(need / 16);
+        // every slot becomes empty: of a caller's workspace those of this launch, of the library's buffer all it can hold
+        // (a later launch that needs more of them is not told that the buffer is fresh); with a kernel, not a memset
+        // node: the caller may be capturing the stream into a graph
+        const uint32_t chunks = (uint32_t)(fill_bytes / 16);
         hipLaunchKernelGGL(fill_slots_kernel, dim3((chunks + 255) / 256 < 2048 ? (chunks + 255) / 256 : 2048), dim3(256), 0, st, (u32x4 *)slots, chunks);
         if (int rc = check_launch("fill_slots_kernel")) return rc;
     }

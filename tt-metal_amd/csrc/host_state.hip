@@ -40,7 +40,7 @@ size_t scratch_grown_size(size_t have, size_t need) {
     return (want + 255) & ~(size_t)255;
 }
 
-int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fresh) {
+int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fresh, size_t *capacity) {
     int dev = 0;
     if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
     std::lock_guard<std::mutex> lock(g_guard);
@@ -56,6 +56,7 @@ int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fr
     }
     if (b.generation != g_generation[kind]) { b.generation = g_generation[kind]; *fresh = true; }
     *ptr = b.ptr;
+    if (capacity) *capacity = b.bytes;
     return TTMI_OK;
 }
 

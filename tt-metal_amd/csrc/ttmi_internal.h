@@ -17,8 +17,9 @@ int check_hip(hipError_t e, const char *what);
 // ---- host state (host_state.hip) --------------------------------------------------------------------------------------
 enum { SCRATCH_SLOTS = 0, SCRATCH_EXPANDED = 1 };
 // The library's own device buffer of at least `bytes` for this purpose on the current device and this stream.  *fresh is
-// set when the contents are undefined (a new buffer, or one invalidated since): the caller initialises it on `stream`.
-int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fresh);
+// set when the contents are undefined (a new buffer, or one invalidated since): the caller initialises ALL of it on `stream`
+// (*capacity bytes: buffers grow geometrically, so a later, larger request may be served without being fresh).
+int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fresh, size_t *capacity = nullptr);
 void scratch_invalidate(int kind);
 size_t scratch_grown_size(size_t have, size_t need);
 // Device and host address of the current device's error word (either may be null).
