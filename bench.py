@@ -212,12 +212,20 @@ def main():
                               ("el", (capi.OP_MUL, h1.data_ptr(), h3.data_ptr(), 0.0, h1.data_ptr(), h1.numel(), stream)),
                               ("mm", mm(h1, cp["w2"], 14336, 4096, "bfp4_b", capi.ACT_NONE, out))])
 
+        if name == "mistral_mlp_block_fused":
+            # the same block with silu(x w1) * (x w3) as ONE launch (ttmi_matmul_bfp_gated), then w2: two launches instead of four
+            plans = [[("gated", (x.data_ptr(), capi.TILE, cp["w1"].data_ptr(), cp["w3"].data_ptr(), FMT["bfp4_b"], 1, 1, m, 4096, 14336, None,
+                                 capi.ACT_SILU, h1.data_ptr(), capi.TILE, capi.BFLOAT16, None, 0, stream)),
+                      ("mm", mm(h1, cp["w2"], 14336, 4096, "bfp4_b", capi.ACT_NONE, out))] for cp in copies]
+
         def run(i):
             for kind, call in plans[i % ncopies]:
-                capi.check(L.ttmi_matmul_bfp(*call) if kind == "mm" else L.ttmi_eltwise_bf16(*call))
+                capi.check(L.ttmi_matmul_bfp(*call) if kind == "mm" else L.ttmi_matmul_bfp_gated(*call) if kind == "gated" else L.ttmi_eltwise_bf16(*call))
 
         ms = time_loop(run, steps, warmup)
         nbytes = sum(workloads.gemm_bytes(m, g[1], g[2], g[3], None) for g in gemms) + (3 * m * hidden * 2 if len(gemms) == 3 else 0)
+        if name == "mistral_mlp_block_fused":      # x once, no [32, 14336] intermediates but the one that feeds w2
+            nbytes = sum((g[1] // 32) * (g[2] // 32) * 576 for g in gemms) + m * 4096 * 2 + 2 * m * hidden * 2 + m * 4096 * 2
         flops = sum(workloads.gemm_flops(m, g[1], g[2], None) for g in gemms)
         leg = {"workload": name, "launches": len(plans[0]), "ms": round(ms, 5), "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
                "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "algorithmic_bytes": nbytes, "flops": flops,
@@ -300,6 +308,9 @@ def main():
                 if block and not args.row_major:
                     sub.append(block_leg(block, sub_steps, warmup, 4321))
                     torch.cuda.empty_cache()
+                    if wl == "decode_mistral":
+                        sub.append(block_leg("mistral_mlp_block_fused", sub_steps, warmup, 4321))
+                        torch.cuda.empty_cache()
             results[wl] = sub
         else:
             fmt = capi.BFLOAT4_B if wl == "pack_bfp4_4k" else capi.BFLOAT8_B

@@ -157,6 +157,17 @@ TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
                     int c_dtype, void *workspace, size_t workspace_bytes, void *stream);
 
+/* A gated pair of GEMMs in one launch:  C[b, m, n] = act(A . B_gate + bias) * (A . B_up), what a gated MLP issues as
+ * ttnn.linear(x, w1, activation="silu"), ttnn.linear(x, w3) and ttnn.mul (models/demos/mistral7b/tt/mistral_mlp.py:43-82:
+ * three device ops and two [m, n] intermediates there).  Both weight tensors have the shape, format and layout that
+ * ttmi_matmul_bfp takes for b; the other arguments mean what they mean there.  The two GEMMs share their activation loads,
+ * their launch and the hand-over of partial sums.  Meant for decode shapes (the weights are streamed once per 32 rows of A).
+ * The workspace, when the caller brings one, has ttmi_matmul_bfp_gated_workspace_bytes() bytes. */
+TTMI_API size_t ttmi_matmul_bfp_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
+TTMI_API int ttmi_matmul_bfp_gated(const void *a, int a_layout, const uint32_t *b_gate, const uint32_t *b_up, int b_fmt, uint32_t batch,
+                          uint32_t b_batch, uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c,
+                          int c_layout, int c_dtype, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ttmi_matmul_bfp for callers that cannot allocate device memory: code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and results as
  * ttmi_matmul_bfp without the workspace pair; the scratch of the kernels lies in a static device array of

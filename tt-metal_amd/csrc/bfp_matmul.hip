@@ -34,6 +34,7 @@ namespace ttmi {
 struct MatmulDev {
     const uint8_t *a;        // bf16
     const uint8_t *b;        // packed tiles
+    const uint8_t *b2;       // gated form only: the second weight matrix (same shape and format), C = act(A.b) * (A.b2)
     const uint16_t *bias;    // bf16 [n] or null
     uint8_t *c;              // output (bf16 or fp32)
     float *slots;            // 2 slots of 32x64 fp32 per workgroup, for outputs shared between workgroups (see SLOT_EMPTY)
@@ -455,14 +456,17 @@ constexpr int WIDE_STAGES = TTMI_WIDE_STAGES;
 constexpr int WIDE_REDUCE_BYTES = WAVES * 32 * 64 * 4;     // every wavefront lays out half of its 64 accumulator registers
 constexpr size_t WIDE_SLOT_BYTES = 32 * WIDE_COLS * sizeof(float);
 
-template <int W, int ACT>
-__global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const MatmulDev p) {
+// NB = 2 is the gated form, C = act(A . B) * (A . B2) (silu(x w1) * (x w3) of a gated MLP in one launch): a unit is then
+// the same k-tile and column group of both weight matrices, which share the activations; every workgroup keeps two sets
+// of sums and hands over two slots.
+template <int W, int ACT, int NB>
+__global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wide_kernel(const MatmulDev p) {
     using F = WideFmt<W>;
-    constexpr int UNIT_BYTES = F::unit_bytes;
+    constexpr int UNIT_BYTES = NB * F::unit_bytes;     // a stage holds the unit's tiles of every weight matrix
     constexpr int WAVE_LDS = WIDE_STAGES * UNIT_BYTES;
     constexpr int LDS_BYTES = WIDE_REDUCE_BYTES > WAVES * WAVE_LDS ? WIDE_REDUCE_BYTES : WAVES * WAVE_LDS;
     constexpr int NLOAD = F::loads;
-    constexpr int PER = NLOAD + 2;                     // vector-memory requests per unit
+    constexpr int PER = NB * NLOAD + 2;                // vector-memory requests per unit
     __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
 
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
@@ -490,7 +494,10 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     uint32_t src_off[NLOAD];
 #pragma unroll
     for (int l = 0; l < NLOAD; ++l) src_off[l] = min(chunk_of[l], chunks_valid - 1) * 16;
-    const uint8_t *wptr = p.b + ((uint64_t)(p.b_batch == 1 ? 0 : bb) * p.kt * p.nt + (uint64_t)(k_begin + wave) * p.nt + nt0) * F::tile_bytes;
+    const uint64_t w_first = ((uint64_t)(p.b_batch == 1 ? 0 : bb) * p.kt * p.nt + (uint64_t)(k_begin + wave) * p.nt + nt0) * F::tile_bytes;
+    const uint8_t *wptr[NB];
+    wptr[0] = p.b + w_first;
+    if (NB == 2) wptr[NB - 1] = p.b2 + w_first;
     const uint64_t w_step = (uint64_t)WAVES * p.nt * F::tile_bytes;
     // activations of one unit for this lane: row c32 of the band, k = kt*32 + 16s + 8kh .. + 7 for s = 0, 1;
     // rows past M read row M-1 and are never stored
@@ -505,11 +512,13 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         a_second = 32; a_step = WAVES * 64;
     }
 
-    f32x16 acc[4];
+    f32x16 acc[NB][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[nb][j][i] = 0.f;
     // The ring registers are cleared by instructions the compiler cannot see through: entries it knows to be zero it
     // would keep in a shared constant register and copy loaded entries around at joins, while their loads are in flight.
     u32x4 a_ring[WIDE_STAGES][2];
@@ -529,11 +538,14 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     auto fetch = [&](auto stage_tag) __attribute__((always_inline)) {
         constexpr int S = decltype(stage_tag)::value;
 #pragma unroll
-        for (int l = 0; l < NLOAD; ++l)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr + src_off[l]),
-                                             (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * UNIT_BYTES + l * F::load_stride),
-                                             16, 0, WEIGHTS_ONCE);
-        wptr += w_step;
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int l = 0; l < NLOAD; ++l)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wptr[nb] + src_off[l]),
+                                                 (__attribute__((address_space(3))) void *)(lds + wave * WAVE_LDS + S * UNIT_BYTES + nb * F::unit_bytes + l * F::load_stride),
+                                                 16, 0, WEIGHTS_ONCE);
+            wptr[nb] += w_step;
+        }
         asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][0]) : "v"(aptr) : "memory");
         asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][1]) : "v"(aptr + a_second) : "memory");
         aptr += a_step;
@@ -552,28 +564,33 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
                 asm volatile("v_mov_b32 %0, %1" : "=v"(moved) : "v"(a_ring[S][s][e]));
                 a_now[s][e] = moved;
             }
-        SlabRaw raw0, raw1;
-        wide_slab_read<W, S * UNIT_BYTES, S * UNIT_BYTES>(exp_at, mant_at, raw0);
-        wide_slab_read<W, S * UNIT_BYTES + 32, S * UNIT_BYTES + F::slab_bytes>(exp_at, mant_at, raw1);
-        wait_slabs(raw0, raw1);
-        if (refill) fetch(stage_tag);
         // hidden-one form (bfp_dequant.h): A.W = 2 (A.hi - A.lo); the subtraction is an MFMA with the negated activations
-        bf16x8 hi[4], lo[4];
         u32x4 a_neg[2];
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
             for (int e = 0; e < 4; ++e) a_neg[s][e] = a_now[s][e] ^ 0x80008000u;
-        slab_expand_hidden<W>(raw0, q, hi, lo);
+        // one weight matrix after the other; the stage is handed to the unit WIDE_STAGES ahead once its last LDS read has returned
+        static_for(std::make_integer_sequence<int, NB>{}, [&](auto nb_tag) __attribute__((always_inline)) {
+            constexpr int nb = decltype(nb_tag)::value;
+            constexpr int AT = S * UNIT_BYTES + nb * F::unit_bytes;
+            SlabRaw raw0, raw1;
+            wide_slab_read<W, AT, AT>(exp_at, mant_at, raw0);
+            wide_slab_read<W, AT + 32, AT + F::slab_bytes>(exp_at, mant_at, raw1);
+            wait_slabs(raw0, raw1);
+            if (nb == NB - 1 && refill) fetch(stage_tag);
+            bf16x8 hi[4], lo[4];
+            slab_expand_hidden<W>(raw0, q, hi, lo);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[0]), hi[j], acc[j], 0, 0, 0);
+            for (int j = 0; j < 4; ++j) acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[0]), hi[j], acc[nb][j], 0, 0, 0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[0]), lo[j], acc[j], 0, 0, 0);
-        slab_expand_hidden<W>(raw1, q, hi, lo);
+            for (int j = 0; j < 4; ++j) acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[0]), lo[j], acc[nb][j], 0, 0, 0);
+            slab_expand_hidden<W>(raw1, q, hi, lo);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[1]), hi[j], acc[j], 0, 0, 0);
+            for (int j = 0; j < 4; ++j) acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[1]), hi[j], acc[nb][j], 0, 0, 0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[1]), lo[j], acc[j], 0, 0, 0);
+            for (int j = 0; j < 4; ++j) acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[1]), lo[j], acc[nb][j], 0, 0, 0);
+        });
     };
 
     // This wavefront's units: k_begin + wave, + WAVES, ...; unit i lives in stage i % STAGES and is requested STAGES
@@ -606,35 +623,37 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     // In two passes (operands j = 0, 1, then 2, 3; 32 KB each) every wavefront writes its accumulator registers as
     // float4 (acc[j][4q4 .. 4q4+3]); wavefront w then keeps q4 = w: rows 8w + 4kh + r (r = 0..3), columns 4*c32 + j.
     float4 *red = reinterpret_cast<float4 *>(lds);
-    float mine[4][4];   // [r][j]
+    float mine[NB][4][4];   // [weight matrix][r][j]
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int pass = 0; pass < 2 * NB; ++pass) {
+        const int nb = pass >> 1;
         __syncthreads();
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
-                const int j = pass * 2 + jj;
-                red[(wave * 8 + jj * 4 + q4) * 64 + lane] = make_float4(acc[j][4 * q4], acc[j][4 * q4 + 1], acc[j][4 * q4 + 2], acc[j][4 * q4 + 3]);
+                const int j = (pass & 1) * 2 + jj;
+                red[(wave * 8 + jj * 4 + q4) * 64 + lane] = make_float4(acc[nb][j][4 * q4], acc[nb][j][4 * q4 + 1], acc[nb][j][4 * q4 + 2], acc[nb][j][4 * q4 + 3]);
             }
         __syncthreads();
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
-            const int j = pass * 2 + jj;
+            const int j = (pass & 1) * 2 + jj;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
             for (int sw = 0; sw < WAVES; ++sw) {
                 const float4 x = red[(sw * 8 + jj * 4 + wave) * 64 + lane];
                 v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
             }
-            mine[0][j] = v.x; mine[1][j] = v.y; mine[2][j] = v.z; mine[3][j] = v.w;
+            mine[nb][0][j] = v.x; mine[nb][1][j] = v.y; mine[nb][2][j] = v.z; mine[nb][3][j] = v.w;
         }
     }
 
     // ---- store, or hand over ------------------------------------------------------------------------------------
     // A chunk = 4 adjacent columns of one row = what one lane holds per r: chunk number (w * 4 + r) * 64 + lane, 1024
-    // per output group.  Stores chunk `idx` of output group `group` (sums still carry the common factor).
-    auto store_chunk = [&](uint32_t group, uint32_t idx, const float (&sums)[4]) __attribute__((always_inline)) {
+    // per output group.  Stores chunk `idx` of output group `group` (sums still carry the common factor; in the gated form
+    // the activation applies to the first matrix's sums, which the second matrix's sums then multiply).
+    auto store_chunk = [&](uint32_t group, uint32_t idx, const float (&sums)[NB][4]) __attribute__((always_inline)) {
         const uint32_t lane_of = idx & 63, r_of = (idx >> 6) & 3, w_of = idx >> 8;
         const uint32_t c32_of = lane_of & 31, t_of = c32_of >> 3, fc_of = (c32_of >> 2) & 1, q_of = c32_of & 3;
         const uint32_t band_of = group / p.ngroups, mt_of = band_of % p.mt, bb_of = band_of / p.mt;
@@ -645,9 +664,10 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
         float v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            float x = sums[j] * hidden_unscale;
+            float x = sums[0][j] * hidden_unscale;
             if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
             v[j] = apply_activation<ACT>(x);
+            if (NB == 2) v[j] *= sums[NB - 1][j] * hidden_unscale;
         }
         uint64_t elem;   // element offset of the 4-column run in C
         if (p.c_tiled) {
@@ -667,7 +687,14 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
 
     if (p.split == 1) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) store_chunk(og, (wave * 4 + r) * 64 + lane, mine[r]);
+        for (int r = 0; r < 4; ++r) {
+            float sums[NB][4];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) sums[nb][j] = mine[nb][r][j];
+            store_chunk(og, (wave * 4 + r) * 64 + lane, sums);
+        }
         return;
     }
     // Outputs shared between `split` workgroups.  Every workgroup publishes its 1024 chunks in its slot; the sums of
@@ -679,13 +706,17 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     // dispatched later, so they finish.
     float4 *const all_slots = reinterpret_cast<float4 *>(p.slots);
     if (computes) {
-        float4 *slot = all_slots + ((uint64_t)me * 16 + wave * 4) * 64 + lane;
+        // slot (me, nb) = 1024 chunks from chunk (me * NB + nb) * 1024 on
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            u32x4 v;
+        for (int nb = 0; nb < NB; ++nb) {
+            float4 *slot = all_slots + (((uint64_t)me * NB + nb) * 16 + wave * 4) * 64 + lane;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[r][j]));
-            if (!p.drop_partial_sums) slot_store(slot + r * 64, v);
+            for (int r = 0; r < 4; ++r) {
+                u32x4 v;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[nb][r][j]));
+                if (!p.drop_partial_sums) slot_store(slot + r * 64, v);
+            }
         }
     }
     if (og == 0) return;
@@ -695,26 +726,30 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
     for (uint32_t idx0 = lo; idx0 < hi; idx0 += 256) {
         const bool active = idx0 + threadIdx.x < hi;                       // idle lanes re-read the last chunk and drop it
         const uint32_t idx = active ? idx0 + threadIdx.x : hi - 1;
-        float4 *const at = all_slots + (uint64_t)target * p.split * 1024 + idx;   // contributor c: at + c * 1024
+        float4 *const at = all_slots + (uint64_t)target * p.split * NB * 1024 + idx;   // contributor c, matrix nb: at + (c * NB + nb) * 1024
         uint32_t spins = 0;
         bool waiting;
         // workgroups with nothing else to do poll cheaply first (one contributor); then everything, checked word by word
         if (!computes) do {
-            u32x4 probe = slot_load_issue(at + (uint64_t)(p.split - 1) * 1024);
+            u32x4 probe = slot_load_issue(at + (uint64_t)(p.split * NB - 1) * 1024);
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(probe)::"memory");
             const bool missing = active && (probe[0] == SLOT_EMPTY || probe[1] == SLOT_EMPTY || probe[2] == SLOT_EMPTY || probe[3] == SLOT_EMPTY);
             waiting = __ballot(missing) != 0 && ++spins < p.spin_limit;
             if (waiting) __builtin_amdgcn_s_sleep(8);
         } while (waiting);
-        float sums[4] = {0.f, 0.f, 0.f, 0.f};
+        float sums[NB][4];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sums[nb][j] = 0.f;
         // N contributors at a time, N a compile-time constant: loads under a condition would have the compiler merge
         // loaded and unloaded registers (that is, copy them) while the loads are in flight
         auto collect = [&](auto count_tag, uint32_t c0) __attribute__((always_inline)) {
-            constexpr int N = decltype(count_tag)::value;
+            constexpr int N = decltype(count_tag)::value * NB;          // slots: those of a contributor lie side by side
             u32x4 got[N];
             do {
 #pragma unroll
-                for (int u = 0; u < N; ++u) got[u] = slot_load_issue(at + (uint64_t)(c0 + u) * 1024);
+                for (int u = 0; u < N; ++u) got[u] = slot_load_issue(at + ((uint64_t)c0 * NB + u) * 1024);
 #pragma unroll
                 for (int u = 0; u < N; ++u) asm volatile("s_waitcnt vmcnt(0)" : "+v"(got[u])::"memory");
                 bool missing = false;
@@ -730,8 +765,8 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
 #pragma unroll
             for (int u = 0; u < N; ++u) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) sums[j] += __uint_as_float(got[u][j]);
-                if (active) slot_store(at + (uint64_t)(c0 + u) * 1024, empty);          // ready for the next launch
+                for (int j = 0; j < 4; ++j) sums[u % NB][j] += __uint_as_float(got[u][j]);
+                if (active) slot_store(at + ((uint64_t)c0 * NB + u) * 1024, empty);      // ready for the next launch
             }
         };
         uint32_t c0 = 0;
@@ -755,7 +790,7 @@ __global__ __launch_bounds__(256, WIDE_WGS_PER_CU) void matmul_wide_kernel(const
 // ---------------------------------------------------------------------------------------------------------
 struct Decomposition { uint32_t mt, kt, nt, ngroups, workgroups, split; uint64_t groups, units; };
 
-static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, bool wide) {
+static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, bool wide, bool gated = false) {
     Decomposition d{};
     const uint32_t group_tiles = wide ? WIDE_TILES : GROUP_TILES;
     d.mt = (m + 31) / 32; d.kt = k / 32; d.nt = n / 32;
@@ -767,7 +802,9 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     // there, x 2 otherwise (every extra k range of an output costs a slot store, a slot read and a slot reset).  128-column kernel: two
     // workgroups per CU (all it can hold, the collecting workgroups included) when that takes few parts per output, one
     // per CU when the outputs are few (measured: many short k ranges cost more than the second workgroup gains).
-    const bool few = d.groups < 100;
+    // The gated form does twice the work per workgroup and hands over twice as much: one workgroup per CU, i.e. half as
+    // many k ranges per output (measured on Mistral's gate / up shape: 25.3-25.8 us against 26.3 us with two per CU).
+    const bool few = d.groups < 100 || gated;
     const uint64_t resident = knob_or(TTMI_KNOB_MATMUL_WORKGROUPS, wide ? (few ? 256 : 256 * WIDE_WGS_PER_CU) : d.groups >= 256 ? 768 : 512);
     uint64_t parts = d.groups >= resident ? 1 : wide && !few ? resident / (d.groups + 1) : resident / d.groups;
     if (parts == 0) parts = 1;
@@ -778,24 +815,26 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     return d;
 }
 
-static size_t slot_bytes_needed(const Decomposition &d, bool wide) {
+static size_t slot_bytes_needed(const Decomposition &d, bool wide, bool gated = false) {
     if (d.split == 1) return 0;                     // every output belongs to one workgroup: no slot is touched
-    return wide ? (size_t)d.workgroups * WIDE_SLOT_BYTES : (size_t)2 * d.workgroups * SLOT_BYTES;
+    return wide ? (size_t)d.workgroups * WIDE_SLOT_BYTES * (gated ? 2 : 1) : (size_t)2 * d.workgroups * SLOT_BYTES;
 }
 
 static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
-    const Decomposition d = decompose(x.batch, x.m, x.k, x.n, wide);
+    const Decomposition d = decompose(x.batch, x.m, x.k, x.n, wide, x.b2 != nullptr);
     MatmulDev p{};
-    p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
+    p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.b2 = (const uint8_t *)x.b2; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
+    const bool gated = x.b2 != nullptr;
+    if (gated && !wide) return fail(TTMI_ERR_UNSUPPORTED, "matmul: the gated form runs on the 128-column kernel only");
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
     p.mt = d.mt; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.groups = (uint32_t)d.groups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
     p.split = d.split;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE;
     p.c_f32 = x.c_dtype == TTMI_FLOAT32;
-    if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
+    if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.b2) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
     if (d.units > 0x7fffffffull || d.groups * d.split > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
-    const size_t need = slot_bytes_needed(d, wide);
+    const size_t need = slot_bytes_needed(d, wide, gated);
     void *slots = nullptr;
     bool fill = false;
     size_t fill_bytes = need;
@@ -830,7 +869,8 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     p.spin_limit = knob_or(TTMI_KNOB_SPIN_LIMIT, SLOT_SPIN_LIMIT);
     p.drop_partial_sums = (int)knob_or(TTMI_KNOB_DROP_PARTIAL_SUMS, 0);
 #define TTMI_LAUNCH(W, ACT)                                                                                     \
-    if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
+    if (wide && gated) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 2>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
+    else if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
     else hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
 #define TTMI_LAUNCH_ACT(W)                                              \
     switch (x.activation) {                                             \
@@ -862,6 +902,11 @@ static Kernel choose_kernel(uint32_t m) {
     return m <= 32 ? Kernel::Wide : Kernel::Stream;
 }
 
+size_t matmul_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
+    if (!batch || !m || !k || !n) return 0;
+    return slot_bytes_needed(decompose(batch, m, k, n, true, true), true, true);
+}
+
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int) {
     if (!batch || !m || !k || !n) return 0;
     const Kernel kernel = choose_kernel(m);
@@ -884,6 +929,13 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
         case Kernel::Wide: return matmul_bfp_wide(x, st);
         default: return matmul_bfp_stream(x, st);
     }
+}
+
+// c = act(a . b + bias) * (a . b2) in one launch of the 128-column kernel (any number of rows: the weights are streamed
+// once per 32-row band, so it is meant for decode shapes).
+int matmul_bfp_gated(const MatmulArgs &x, hipStream_t st) {
+    if (int rc = ttmi_device_status()) return rc;
+    return launch_streaming(x, st, true);
 }
 
 }  // namespace ttmi

@@ -150,6 +150,21 @@ int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, u
     return matmul_bfp(args, (hipStream_t)stream);
 }
 
+size_t ttmi_matmul_bfp_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt) {
+    (void)b_fmt;
+    return matmul_gated_workspace_bytes(batch, m, k, n);
+}
+
+int ttmi_matmul_bfp_gated(const void *a, int a_layout, const uint32_t *b_gate, const uint32_t *b_up, int b_fmt, uint32_t batch, uint32_t b_batch,
+                          uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout, int c_dtype,
+                          void *workspace, size_t workspace_bytes, void *stream) {
+    if (int rc = validate_matmul(a, a_layout, b_gate, b_fmt, batch, b_batch, m, k, n, activation, c, c_layout, c_dtype)) return rc;
+    if (!b_up) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: null pointer");
+    MatmulArgs args{a, a_layout, b_gate, b_fmt, batch, b_batch, m, k, n, bias, activation, c, c_layout, c_dtype, workspace, workspace_bytes};
+    args.b2 = b_up;
+    return matmul_bfp_gated(args, (hipStream_t)stream);
+}
+
 int ttmi_eltwise_bf16(int op, const void *a, const void *b, float scalar, void *c, size_t count, void *stream) {
     if (count && (!a || !c)) return fail(TTMI_ERR_INVALID_ARGUMENT, "eltwise: null pointer");
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15u)

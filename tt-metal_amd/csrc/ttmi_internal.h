@@ -62,6 +62,7 @@ struct MatmulArgs {
     const void *bias; int activation;
     void *c; int c_layout, c_dtype;
     void *workspace; size_t workspace_bytes;
+    const uint32_t *b2 = nullptr;   // gated form (128-column kernel only): c = act(a . b) * (a . b2)
     bool no_alloc = false;          // the call may not allocate: `workspace` is all the scratch there is, its last 256 bytes stand
                                     // in for the error word when the device has none yet
 };
@@ -72,6 +73,8 @@ size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n
 int matmul_bfp(const MatmulArgs &args, hipStream_t st);         // streaming kernel (decode shapes) or the tiled one
 int matmul_bfp_stream(const MatmulArgs &args, hipStream_t st);
 int matmul_bfp_wide(const MatmulArgs &args, hipStream_t st);     // the streaming kernel with 128-column units
+size_t matmul_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n);
+int matmul_bfp_gated(const MatmulArgs &args, hipStream_t st);   // args.b2 set
 int matmul_bfp_tiled(const MatmulArgs &args, hipStream_t st);
 int matmul_bfp_expanded(const MatmulArgs &args, hipStream_t st);   // expand the weights to bf16 once, then a bf16 GEMM
 size_t matmul_expanded_workspace_bytes(uint32_t b_batch, uint32_t k, uint32_t n);

@@ -24,6 +24,7 @@ SYMBOLS = (
     "ttmi_pack_rowmajor_as_bfp_tiles", "ttmi_unpack_bfp_tiles_as_rowmajor",
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
     "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_typecast_tiles", "ttmi_device_status", "ttmi_matmul_bfp_static",
+    "ttmi_matmul_bfp_gated_workspace_bytes", "ttmi_matmul_bfp_gated",
 )
 
 _lib = None
@@ -66,6 +67,10 @@ def lib() -> ctypes.CDLL:
         L.ttmi_copy_window.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(ctypes.c_int32), ctypes.c_float, vp]
         L.ttmi_unpad_tiles.restype = i32
         L.ttmi_unpad_tiles.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(u32), vp]
+        L.ttmi_matmul_bfp_gated_workspace_bytes.restype = ctypes.c_size_t
+        L.ttmi_matmul_bfp_gated_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
+        L.ttmi_matmul_bfp_gated.restype = i32
+        L.ttmi_matmul_bfp_gated.argtypes = [vp, i32, vp, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, ctypes.c_size_t, vp]
         L.ttmi_matmul_bfp_static.restype = i32
         L.ttmi_matmul_bfp_static.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp]
         L.ttmi_typecast_tiles.restype = i32
@@ -196,6 +201,26 @@ def matmul_bfp(a, a_layout: int, b_words, b_fmt: int, batch: int, b_batch: int, 
         ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
     check(lib().ttmi_matmul_bfp(
         _dev(a), a_layout, _dev(b_words), b_fmt, batch, b_batch, m, k, n,
+        _dev(bias) if bias is not None else None, activation, _dev(c), c_layout, _torch_dtype_code(c),
+        ws_ptr, ws_bytes, _stream()))
+    if c_layout == ROW_MAJOR:
+        return c.view(batch, m, n)
+    return c
+
+
+def matmul_bfp_gated(a, a_layout: int, gate_words, up_words, b_fmt: int, batch: int, b_batch: int, m: int, k: int, n: int, *,
+                     bias=None, activation: int = ACT_SILU, c_layout: int = ROW_MAJOR, out_dtype=None, workspace=None):
+    """act(a . gate + bias) * (a . up) in one launch (ttmi_matmul_bfp_gated); arguments as for matmul_bfp."""
+    import torch
+
+    out_dtype = out_dtype or torch.bfloat16
+    mp = padded(m) if c_layout == TILE else m
+    c = torch.empty(batch * mp * n, dtype=out_dtype, device=a.device)
+    ws_ptr, ws_bytes = None, 0
+    if workspace is not None:
+        ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
+    check(lib().ttmi_matmul_bfp_gated(
+        _dev(a), a_layout, _dev(gate_words), _dev(up_words), b_fmt, batch, b_batch, m, k, n,
         _dev(bias) if bias is not None else None, activation, _dev(c), c_layout, _torch_dtype_code(c),
         ws_ptr, ws_bytes, _stream()))
     if c_layout == ROW_MAJOR:
