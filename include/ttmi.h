@@ -146,7 +146,10 @@ TTMI_API size_t ttmi_matmul_bfp_workspace_bytes(uint32_t batch, uint32_t m, uint
  *   b        packed tiles, b_fmt TTMI_BFLOAT8_B | TTMI_BFLOAT4_B, tile (kt, nt) at index kt*Nt + nt, k and n
  *            multiples of 32; b_batch is `batch` (bmm) or 1 (weights broadcast over the batch: bcast_batch)
  *   bias     NULL or bf16 [n] (row-broadcast add, matmul.hpp:117-214)
- *   c        c_dtype TTMI_BFLOAT16 (round to nearest even) or TTMI_FLOAT32; c_layout as for a
+ *   c        c_dtype TTMI_BFLOAT16 (round to nearest even) or TTMI_FLOAT32; c_layout as for a.  Or c_dtype TTMI_BFLOAT8_B |
+ *            TTMI_BFLOAT4_B with c_layout TTMI_TILE (output_dtype of tt::operations::primary::matmul, bmm_op.hpp:318-346):
+ *            packed tiles of the bf16-rounded result with the host packers' arithmetic (what ttmi_typecast_tiles gives for
+ *            the bf16 output) — packed in the epilogue of the decode kernel (up to 32 rows), by one more launch otherwise
  *   workspace NULL (the library keeps a per-device buffer of its own, allocated on first use) or at least
  *            ttmi_matmul_bfp_workspace_bytes() bytes of device memory, 256-byte aligned.  Up to 127 rows it holds
  *            partial sums of workgroups that share an output (a few MB); from 512 rows on the weights expanded to

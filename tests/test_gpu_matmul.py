@@ -542,3 +542,28 @@ def test_library_slots_beyond_the_first_launch_are_empty_too():
         capi.check(L.ttmi_matmul_bfp(*args, got.data_ptr(), capi.TILE, capi.BFLOAT16, None, 0, stream.cuda_stream))
         torch.cuda.synchronize()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), groups
+
+
+@pytest.mark.parametrize("out_fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("batch,m,k,n", [(1, 32, 64, 128), (1, 32, 2048, 256), (1, 32, 4096, 96), (2, 32, 1024, 2080), (1, 64, 512, 160),
+                                         (1, 256, 128, 256), (1, 512, 64, 160)])
+def test_block_float_output(oracle, out_fmt, fmt, batch, m, k, n):
+    """Output dtype BFLOAT8_B / BFLOAT4_B (TILE layout): the words are those that packing the bf16 output of the same GEMM
+    gives (ttmi_typecast_tiles, itself pinned against the oracle's packer) — in the epilogue of the 128-column kernel,
+    stored directly and through the hand-over of partial sums, with a column group that is not full; through a buffer of
+    the library and one more launch for the other kernels — and unpack to the oracle's unpacking of those words."""
+    a_bits = workloads.activations_bf16(m, k, seed=400, batch=batch)
+    words, _ = pack_weights(oracle, workloads.weights_f32(k, n, seed=401), fmt)
+    a_tiles = capi.tilize(bf16_dev(a_bits).reshape(batch, m, k))
+    bias_bits = workloads.f32_to_bf16_bits_rne(workloads.normal_tensor((n,), seed=402))
+    for kwargs in ({}, {"bias": bf16_dev(bias_bits), "activation": capi.ACT_GELU}):
+        dense = capi.matmul_bfp(a_tiles, capi.TILE, words, fmt, batch, 1, m, k, n, c_layout=capi.TILE, **kwargs)
+        want = capi.typecast_tiles(dense, capi.BFLOAT16, out_fmt)
+        got = capi.matmul_bfp(a_tiles, capi.TILE, words, fmt, batch, 1, m, k, n, c_layout=capi.TILE, out_bfp=out_fmt, **kwargs)
+        assert torch.equal(got, want)
+    host = oracle.pack_fp32_vec_as_bfp_tiles(out_fmt, dense.float().cpu().numpy().reshape(-1), False)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), host)
+    with pytest.raises(RuntimeError, match="TILE layout"):
+        capi.check(capi.lib().ttmi_matmul_bfp(a_tiles.data_ptr(), capi.TILE, words.data_ptr(), fmt, batch, 1, m, k, n, None, 0, got.data_ptr(),
+                                              capi.ROW_MAJOR, out_fmt, None, 0, None))

@@ -16,6 +16,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#include "bfp_dequant.h"
 #include "ttmi_internal.h"
 
 namespace ttmi {
@@ -35,31 +36,7 @@ template <int W> struct Fmt;
 template <> struct Fmt<7> { static constexpr int tile_bytes = 1088, row_bytes = 16, face_bytes = 256; };
 template <> struct Fmt<3> { static constexpr int tile_bytes = 576, row_bytes = 8, face_bytes = 128; };
 
-// max over the 2 or 4 lanes that share a face row (lanes are aligned quads / pairs)
-template <int LPR> __device__ __forceinline__ uint32_t row_max(uint32_t v) {
-    uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, true);
-    v = v > o ? v : o;
-    if (LPR == 4) {
-        o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E /* quad_perm:[2,3,0,1] */, 0xf, 0xf, true);
-        v = v > o ? v : o;
-    }
-    return v;
-}
-
-// Code of one element (tt_metal/common/bfloat8.hpp:23-87, blockfloat_common.hpp:67-147): hidden one OR-ed in even
-// for a zero exponent field, truncating shift by the exponent gap, round half up, saturate, sign dropped when the
-// mantissa rounds to zero, +-0 -> 0.  The two shifts are folded into one:
-//     ((m >> gap) + h) >> s  ==  (m + (h << gap)) >> (gap + s)        (h = 2^(s-1), s = 24 - W)
-// and every gap above 31 - s gives 0 either way (m < 2^24), so the gap is clamped there and nothing overflows.
-template <int W> __device__ __forceinline__ uint32_t to_code(uint32_t bits, uint32_t shared) {
-    constexpr uint32_t s = 24 - W, h = 1u << (s - 1), top = (1u << W) - 1u;
-    const uint32_t gap = min(shared - ((bits >> 23) & 0xffu), 31u - s);
-    const uint32_t m24 = (bits & 0x007fffffu) | 0x00800000u;
-    uint32_t m = min(((h << gap) + m24) >> (gap + s), top);
-    m = (bits & 0x7fffffffu) ? m : 0u;
-    return m ? (((bits >> 31) << W) | m) : 0u;
-}
-
+// row_max (shared exponent of a face row over its lanes) and to_code (one element's code) live in bfp_dequant.h
 template <int W> __device__ __forceinline__ uint32_t from_code(uint32_t code, uint32_t shared) {
     const uint32_t man = code & ((1u << W) - 1u);
     const uint32_t sign = ((code >> W) & 1u) << 31;

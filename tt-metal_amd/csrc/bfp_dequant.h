@@ -280,6 +280,33 @@ template <int W> __device__ __forceinline__ void slab_expand_hidden(const SlabRa
     }
 }
 
+// ---- the packer's arithmetic for one element and one face row (used by the codec kernels and by GEMM epilogues that
+// write block-float output) -------------------------------------------------------------------------------------------
+// max over the 2 or 4 lanes that share a face row (lanes are aligned quads / pairs)
+template <int LPR> __device__ __forceinline__ uint32_t row_max(uint32_t v) {
+    uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, true);
+    v = v > o ? v : o;
+    if (LPR == 4) {
+        o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E /* quad_perm:[2,3,0,1] */, 0xf, 0xf, true);
+        v = v > o ? v : o;
+    }
+    return v;
+}
+
+// Code of one element (tt_metal/common/bfloat8.hpp:23-87, blockfloat_common.hpp:67-147): hidden one OR-ed in even
+// for a zero exponent field, truncating shift by the exponent gap, round half up, saturate, sign dropped when the
+// mantissa rounds to zero, +-0 -> 0.  The two shifts are folded into one:
+//     ((m >> gap) + h) >> s  ==  (m + (h << gap)) >> (gap + s)        (h = 2^(s-1), s = 24 - W)
+// and every gap above 31 - s gives 0 either way (m < 2^24), so the gap is clamped there and nothing overflows.
+template <int W> __device__ __forceinline__ uint32_t to_code(uint32_t bits, uint32_t shared) {
+    constexpr uint32_t s = 24 - W, h = 1u << (s - 1), top = (1u << W) - 1u;
+    const uint32_t gap = min(shared - ((bits >> 23) & 0xffu), 31u - s);
+    const uint32_t m24 = (bits & 0x007fffffu) | 0x00800000u;
+    uint32_t m = min(((h << gap) + m24) >> (gap + s), top);
+    m = (bits & 0x7fffffffu) ? m : 0u;
+    return m ? (((bits >> 31) << W) | m) : 0u;
+}
+
 // Epilogue of the tiled GEMM kernels for one wavefront: a 128-row x 64-column part of C (one 64-column weight group) whose
 // accumulators lie as v_mfma_f32_32x32x16 leaves them, with the column order of the weight expansion:
 //   acc[rb][cb][i] = row 32 rb + 8 (i / 4) + 4 kh + i % 4, column 32 t + 16 fc + 4 q + 2 half + cb of the 64, for lane

@@ -48,6 +48,7 @@ struct MatmulDev {
     uint32_t units;          // U = batch * mt * ngroups * kt
     uint32_t split;          // k ranges per output group (>= 1)
     int a_tiled, c_tiled, c_f32;
+    int c_bfp;               // 128-column kernel only: 0, or the mantissa bits (7 | 3) of a block-float output in TILE layout
 };
 
 constexpr int GROUP_TILES = 2;                       // n tiles per output group
@@ -669,6 +670,33 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
             v[j] = apply_activation<ACT>(x);
             if (NB == 2) v[j] *= sums[NB - 1][j] * hidden_unscale;
         }
+        if (p.c_bfp) {
+            // Block-float output (TILE layout): the sums are rounded to bf16 as for a bf16 output and packed with the host
+            // packers' arithmetic; the shared exponent of the face row is a max over its 16 columns = this aligned lane quad.
+            uint32_t bits[4], e_max = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                const uint32_t two = f32x2_to_bf16x2_rne(v[j], v[j + 1]);
+                bits[j] = two << 16; bits[j + 1] = two & 0xffff0000u;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) e_max = max(e_max, (bits[j] >> 23) & 0xffu);
+            const uint32_t shared = row_max<4>(e_max);
+            const uint64_t tile = ((uint64_t)bb_of * p.mt + mt_of) * p.nt + nt_of;
+            const uint32_t face = (row_in_band >> 4) * 2 + fc_of, row_in_face = row_in_band & 15;
+            if (p.c_bfp == 7) {
+                uint8_t *at = p.c + tile * 1088;
+                const uint32_t word = to_code<7>(bits[0], shared) | (to_code<7>(bits[1], shared) << 8) | (to_code<7>(bits[2], shared) << 16) | (to_code<7>(bits[3], shared) << 24);
+                *reinterpret_cast<uint32_t *>(at + 64 + face * 256 + row_in_face * 16 + q_of * 4) = word;
+                if (q_of == 0) at[face * 16 + row_in_face] = (uint8_t)shared;
+            } else {
+                uint8_t *at = p.c + tile * 576;
+                const uint32_t half = to_code<3>(bits[0], shared) | (to_code<3>(bits[1], shared) << 4) | (to_code<3>(bits[2], shared) << 8) | (to_code<3>(bits[3], shared) << 12);
+                *reinterpret_cast<uint16_t *>(at + 64 + face * 128 + row_in_face * 8 + q_of * 2) = (uint16_t)half;
+                if (q_of == 0) at[face * 16 + row_in_face] = (uint8_t)shared;
+            }
+            return;
+        }
         uint64_t elem;   // element offset of the 4-column run in C
         if (p.c_tiled) {
             const uint64_t tile = ((uint64_t)bb_of * p.mt + mt_of) * p.nt + nt_of;
@@ -721,7 +749,8 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     }
     if (og == 0) return;
     const uint32_t target = og - 1;
-    const uint32_t lo = (part * 1024u) / p.split, hi = ((part + 1) * 1024u) / p.split;
+    // ranges of whole lane quads: the four chunks of a face row (16 columns) stay with four neighbouring threads
+    const uint32_t lo = ((part * 256u) / p.split) * 4u, hi = (((part + 1) * 256u) / p.split) * 4u;
     const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
     for (uint32_t idx0 = lo; idx0 < hi; idx0 += 256) {
         const bool active = idx0 + threadIdx.x < hi;                       // idle lanes re-read the last chunk and drop it
@@ -831,6 +860,8 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     p.split = d.split;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE;
     p.c_f32 = x.c_dtype == TTMI_FLOAT32;
+    p.c_bfp = x.c_dtype == TTMI_BFLOAT8_B ? 7 : x.c_dtype == TTMI_BFLOAT4_B ? 3 : 0;
+    if (p.c_bfp && !(wide && p.c_tiled)) return fail(TTMI_ERR_UNSUPPORTED, "matmul: this kernel writes no block-float output");
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.b2) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
     if (d.units > 0x7fffffffull || d.groups * d.split > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
@@ -923,7 +954,22 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
     // what an earlier launch on this device has reported (a wait for partial sums that gave up) surfaces here
     if (!x.no_alloc || error_word_if_exists(nullptr, nullptr))
         if (int rc = ttmi_device_status()) return rc;
-    switch (choose_kernel(x.m)) {
+    const Kernel kernel = choose_kernel(x.m);
+    const bool c_bfp = x.c_dtype == TTMI_BFLOAT8_B || x.c_dtype == TTMI_BFLOAT4_B;
+    if (c_bfp && kernel != Kernel::Wide) {
+        // Only the 128-column kernel packs in its epilogue.  The others write bf16 tiles into a buffer of the library (one
+        // per stream) and one typecast pass packs them: the same bits, one more launch.
+        if (x.no_alloc) return fail(TTMI_ERR_UNSUPPORTED, "matmul: a block-float output of this shape needs a buffer that this entry point may not allocate");
+        void *tiles = nullptr;
+        bool fresh;
+        const size_t n_tiles = (size_t)x.batch * ((x.m + 31) / 32) * (x.n / 32);
+        if (int rc = scratch_get(SCRATCH_OUTPUT, st, n_tiles * 2048, &tiles, &fresh)) return rc;
+        MatmulArgs y = x;
+        y.c = tiles; y.c_dtype = TTMI_BFLOAT16;
+        if (int rc = matmul_bfp(y, st)) return rc;
+        return codec_typecast_tiles(tiles, TTMI_BFLOAT16, x.c, x.c_dtype, n_tiles, st);
+    }
+    switch (kernel) {
         case Kernel::Expanded: return matmul_bfp_expanded(x, st);
         case Kernel::Tile: return matmul_bfp_tiled(x, st);
         case Kernel::Wide: return matmul_bfp_wide(x, st);

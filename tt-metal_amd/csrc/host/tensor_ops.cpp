@@ -421,13 +421,15 @@ Tensor matmul(const Tensor &a, const Tensor &b, bool bcast_batch, const Tensor *
         }
     }
     const uint64_t a_elements = (uint64_t)batch_a * m * k, c_elements = (uint64_t)batch_a * m * n;
-    // block-float activations are expanded (exactly) to bf16 tiles by one kernel in front of the GEMM, a block-float output is
-    // packed from the bf16 result tiles by one kernel behind it (the host packers' arithmetic: parity with the Tensix packer unpinned)
+    // block-float activations are expanded (exactly) to bf16 tiles by one kernel in front of the GEMM; a block-float output is
+    // packed by the GEMM itself — in the epilogue of the decode kernel, behind the others by one more launch inside the
+    // library (the host packers' arithmetic on the bf16-rounded sums: parity with the Tensix packer unpinned)
     Buffer a_tiles = is_block_float(a.dtype) ? typecast_tiles(a.buffer, a.dtype, DataType::BFLOAT16, a_elements, device) : a.buffer;
-    Buffer c = allocate(c_elements * 2, device);
+    const bool packed_out = is_block_float(out_dtype);
+    Buffer c = allocate(packed_out ? storage_bytes(out_dtype, Layout::TILE, {batch_a, m, n}) : c_elements * 2, device);
     check(ttmi_matmul_bfp(a_tiles.data, TTMI_TILE, (const uint32_t *)b.buffer.data, (int)b.dtype, batch_a, batch_b, m, k, n,
-                          bias ? bias_row.data : nullptr, activation, c.data, TTMI_TILE, TTMI_BFLOAT16, nullptr, 0, stream_of(device)));
-    if (is_block_float(out_dtype)) c = typecast_tiles(c, DataType::BFLOAT16, out_dtype, c_elements, device);
+                          bias ? bias_row.data : nullptr, activation, c.data, TTMI_TILE, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0,
+                          stream_of(device)));
     Tensor out;
     out.buffer = std::move(c);
     out.shape.assign(a.shape.begin(), a.shape.end() - 1);

@@ -30,7 +30,7 @@ struct Key {
 std::mutex g_guard;
 std::map<Key, Buffer> g_live;
 std::vector<void *> g_retired;
-uint64_t g_generation[2] = {0, 0};       // raised by scratch_invalidate: contents of every buffer of that kind are suspect
+uint64_t g_generation[SCRATCH_KINDS] = {};       // raised by scratch_invalidate: contents of every buffer of that kind are suspect
 }  // namespace
 
 size_t scratch_grown_size(size_t have, size_t need) {

@@ -38,7 +38,9 @@ int validate_matmul(const void *a, int a_layout, const uint32_t *b, int b_fmt, u
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: unknown layout");
     if (b_batch != 1 && b_batch != batch)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: weight batch (%u) must be 1 or equal to the activation batch (%u)", b_batch, batch);
-    if (c_dtype != TTMI_BFLOAT16 && c_dtype != TTMI_FLOAT32) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: output dtype must be BFLOAT16 or FLOAT32");
+    if (c_dtype != TTMI_BFLOAT16 && c_dtype != TTMI_FLOAT32 && !is_bfp(c_dtype))
+        return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: output dtype must be BFLOAT16, FLOAT32, BFLOAT8_B or BFLOAT4_B");
+    if (is_bfp(c_dtype) && c_layout != TTMI_TILE) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a block-float output needs TILE layout");
     if (activation < TTMI_ACT_NONE || activation > TTMI_ACT_SILU) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: unknown activation %d", activation);
     return TTMI_OK;
 }

@@ -15,7 +15,7 @@ int check_launch(const char *what);
 int check_hip(hipError_t e, const char *what);
 
 // ---- host state (host_state.hip) --------------------------------------------------------------------------------------
-enum { SCRATCH_SLOTS = 0, SCRATCH_EXPANDED = 1 };
+enum { SCRATCH_SLOTS = 0, SCRATCH_EXPANDED = 1, SCRATCH_OUTPUT = 2, SCRATCH_KINDS = 3 };
 // The library's own device buffer of at least `bytes` for this purpose on the current device and this stream.  *fresh is
 // set when the contents are undefined (a new buffer, or one invalidated since): the caller initialises ALL of it on `stream`
 // (*capacity bytes: buffers grow geometrically, so a later, larger request may be served without being fresh).

@@ -189,19 +189,23 @@ def untilize(tiles, shape):
 
 
 def matmul_bfp(a, a_layout: int, b_words, b_fmt: int, batch: int, b_batch: int, m: int, k: int, n: int, *,
-               bias=None, activation: int = ACT_NONE, c_layout: int = ROW_MAJOR, out_dtype=None, workspace=None):
-    """a: cuda bf16 (dense [batch,m,k] or tile order); b_words: packed weights; returns C (dense or tile order)."""
+               bias=None, activation: int = ACT_NONE, c_layout: int = ROW_MAJOR, out_dtype=None, workspace=None, out_bfp: int | None = None):
+    """a: cuda bf16 (dense [batch,m,k] or tile order); b_words: packed weights; returns C (dense or tile order).
+    out_bfp = BFLOAT8_B | BFLOAT4_B (TILE layout only): C as packed words."""
     import torch
 
     out_dtype = out_dtype or torch.bfloat16
     mp = padded(m) if c_layout == TILE else m
-    c = torch.empty(batch * mp * n, dtype=out_dtype, device=a.device)
+    if out_bfp is not None:
+        c = torch.empty(batch * (mp // 32) * (n // 32) * TILE_BYTES[out_bfp] // 4, dtype=torch.int32, device=a.device)
+    else:
+        c = torch.empty(batch * mp * n, dtype=out_dtype, device=a.device)
     ws_ptr, ws_bytes = None, 0
     if workspace is not None:
         ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
     check(lib().ttmi_matmul_bfp(
         _dev(a), a_layout, _dev(b_words), b_fmt, batch, b_batch, m, k, n,
-        _dev(bias) if bias is not None else None, activation, _dev(c), c_layout, _torch_dtype_code(c),
+        _dev(bias) if bias is not None else None, activation, _dev(c), c_layout, out_bfp if out_bfp is not None else _torch_dtype_code(c),
         ws_ptr, ws_bytes, _stream()))
     if c_layout == ROW_MAJOR:
         return c.view(batch, m, n)
