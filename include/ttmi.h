@@ -160,6 +160,18 @@ TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
                     int c_dtype, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ttnn.matmul / tt_lib.tensor.matmul / bmm with two bf16 operands (ttnn/cpp/ttnn/operations/matmul.hpp:39-42,
+ * tt_eager/tt_dnn/op_library/bmm/bmm_op.hpp:388-456):  C[b, m, n] = act(A[b, m, k] . B[(b | 0), k, n] + bias[n]).
+ *   b        bf16 in TILE layout (4-face tiles of 2048 bytes, tile (kt, nt) of slice s at index (s*Kt + kt)*Nt + nt), k and n
+ *            multiples of 32
+ * Everything else as for ttmi_matmul_bfp.  Two launches: the weights are re-laid-out into the operand layout of the matrix
+ * cores (workspace: 2 bytes per weight, ttmi_matmul_bf16_workspace_bytes(); NULL = a buffer of the library), then the
+ * bf16 GEMM that ttmi_matmul_bfp uses from 512 rows on runs on them.  Not a tuned path: block-float weights are. */
+TTMI_API size_t ttmi_matmul_bf16_workspace_bytes(uint32_t b_batch, uint32_t k, uint32_t n);
+TTMI_API int ttmi_matmul_bf16(const void *a, int a_layout, const void *b, uint32_t batch, uint32_t b_batch, uint32_t m, uint32_t k,
+                     uint32_t n, const void *bias, int activation, void *c, int c_layout, int c_dtype, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
 /* A gated pair of GEMMs in one launch:  C[b, m, n] = act(A . B_gate + bias) * (A . B_up), what a gated MLP issues as
  * ttnn.linear(x, w1, activation="silu"), ttnn.linear(x, w3) and ttnn.mul (models/demos/mistral7b/tt/mistral_mlp.py:43-82:
  * three device ops and two [m, n] intermediates there).  Both weight tensors have the shape, format and layout that

@@ -567,3 +567,33 @@ def test_block_float_output(oracle, out_fmt, fmt, batch, m, k, n):
     with pytest.raises(RuntimeError, match="TILE layout"):
         capi.check(capi.lib().ttmi_matmul_bfp(a_tiles.data_ptr(), capi.TILE, words.data_ptr(), fmt, batch, 1, m, k, n, None, 0, got.data_ptr(),
                                               capi.ROW_MAJOR, out_fmt, None, 0, None))
+
+
+@pytest.mark.parametrize("batch,b_batch,m,k,n", [(1, 1, 32, 64, 64), (1, 1, 32, 4544, 256), (2, 2, 40, 160, 96), (3, 1, 300, 96, 288), (1, 1, 512, 256, 544)])
+def test_bf16_weights(batch, b_batch, m, k, n):
+    """Two bf16 operands (ttmi_matmul_bf16): weights in TILE layout, re-laid-out and multiplied by the bf16 GEMM of the
+    expanding path; against a float64 matmul of the same values with the bound of the block-float GEMMs; TILE and
+    row-major activations give the same bits; bias and activation; block-float output."""
+    a_bits = workloads.activations_bf16(m, k, seed=500, batch=batch)
+    w_bits = workloads.f32_to_bf16_bits_rne(workloads.weights_f32(k, n, seed=501, batch=b_batch))
+    a = workloads.bf16_bits_to_f32(a_bits).reshape(batch, m, k)
+    w = workloads.bf16_bits_to_f32(w_bits).reshape(b_batch, k, n)
+    a_dev = bf16_dev(a_bits).reshape(batch, m, k)
+    w_tiles = capi.tilize(bf16_dev(w_bits).reshape(b_batch, k, n))
+    c = capi.matmul_bf16(a_dev, capi.ROW_MAJOR, w_tiles, batch, b_batch, m, k, n, out_dtype=torch.float32)
+    for b in range(batch):
+        check_against_reference(c[b].cpu().numpy(), a[b], w[b if b_batch > 1 else 0], k, bf16_out=False)
+    c16 = capi.matmul_bf16(a_dev, capi.ROW_MAJOR, w_tiles, batch, b_batch, m, k, n)
+    for b in range(batch):
+        check_against_reference(c16[b].float().cpu().numpy(), a[b], w[b if b_batch > 1 else 0], k)
+    if m % 32 == 0:
+        tiles = capi.matmul_bf16(capi.tilize(a_dev), capi.TILE, w_tiles, batch, b_batch, m, k, n, c_layout=capi.TILE)
+        assert torch.equal(capi.untilize(tiles, (batch, m, n)).view(torch.int16), c16.view(torch.int16))
+    bias_bits = workloads.f32_to_bf16_bits_rne(workloads.normal_tensor((n,), seed=502))
+    g = capi.matmul_bf16(a_dev, capi.ROW_MAJOR, w_tiles, batch, b_batch, m, k, n, bias=bf16_dev(bias_bits), activation=capi.ACT_RELU, out_dtype=torch.float32)
+    assert torch.allclose(g, torch.relu(c + torch.from_numpy(workloads.bf16_bits_to_f32(bias_bits)).cuda()), rtol=1e-5, atol=1e-5)
+    need = capi.lib().ttmi_matmul_bf16_workspace_bytes(b_batch, k, n)
+    assert need == b_batch * (k // 32) * ((n // 32 + 1) // 2) * 4096
+    ws = torch.full((need,), 0x5A, dtype=torch.uint8, device="cuda")
+    again = capi.matmul_bf16(a_dev, capi.ROW_MAJOR, w_tiles, batch, b_batch, m, k, n, workspace=ws)
+    assert torch.equal(again.view(torch.int16), c16.view(torch.int16))

@@ -139,6 +139,26 @@ def test_matmul_errors(device):
     assert (a2 @ b2).shape == (2, 32, 32)
 
 
+def test_matmul_of_two_bfloat16_tensors(device):
+    """ttnn.matmul / ttnn.linear with two bf16 operands (matmul.hpp:39-42): the surface is the same, the weights take the
+    re-layout path of ttmi_matmul_bf16."""
+    import ttnn
+
+    torch.manual_seed(11)
+    x = torch.randn((2, 64, 96), dtype=torch.bfloat16)
+    w = torch.randn((96, 160), dtype=torch.bfloat16)
+    bias = torch.randn((1, 160), dtype=torch.bfloat16)
+    tx = ttnn.from_torch(x, layout=ttnn.TILE_LAYOUT, device=device)
+    tw = ttnn.from_torch(w, layout=ttnn.TILE_LAYOUT, device=device)
+    tb = ttnn.from_torch(bias, layout=ttnn.TILE_LAYOUT, device=device)
+    got = ttnn.to_torch(ttnn.matmul(tx, tw)).float()
+    ref = x.double() @ w.double()
+    assert got.shape == (2, 64, 160)
+    assert torch.allclose(got.double(), ref, rtol=2 ** -7, atol=2e-2)
+    got = ttnn.to_torch(ttnn.linear(tx, tw, bias=tb, activation="relu")).float()
+    assert torch.allclose(got.double(), torch.relu(ref + bias.double()), rtol=2 ** -7, atol=2e-2)
+
+
 @pytest.mark.parametrize("name", ["BFLOAT8_B", "BFLOAT4_B"])
 @pytest.mark.parametrize("shape", [(1, 1, 32, 32), (2, 3, 64, 96)])
 def test_tt_lib_tensor_conversion(oracle, shape, name):

@@ -977,6 +977,22 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
     }
 }
 
+// bf16 x bf16: the weights are brought into the operand layout of the expanding GEMM's second pass (a re-layout instead of
+// an expansion), whatever the number of rows; a block-float output goes through the library's output buffer.
+int matmul_bf16(const MatmulArgs &x, hipStream_t st) {
+    if (int rc = ttmi_device_status()) return rc;
+    const bool c_bfp = x.c_dtype == TTMI_BFLOAT8_B || x.c_dtype == TTMI_BFLOAT4_B;
+    if (!c_bfp) return matmul_bfp_expanded(x, st);
+    void *tiles = nullptr;
+    bool fresh;
+    const size_t n_tiles = (size_t)x.batch * ((x.m + 31) / 32) * (x.n / 32);
+    if (int rc = scratch_get(SCRATCH_OUTPUT, st, n_tiles * 2048, &tiles, &fresh)) return rc;
+    MatmulArgs y = x;
+    y.c = tiles; y.c_dtype = TTMI_BFLOAT16;
+    if (int rc = matmul_bfp_expanded(y, st)) return rc;
+    return codec_typecast_tiles(tiles, TTMI_BFLOAT16, x.c, x.c_dtype, n_tiles, st);
+}
+
 // c = act(a . b + bias) * (a . b2) in one launch of the 128-column kernel (any number of rows: the weights are streamed
 // once per 32-row band, so it is meant for decode shapes).
 int matmul_bfp_gated(const MatmulArgs &x, hipStream_t st) {

@@ -87,6 +87,49 @@ __global__ __launch_bounds__(256) void expand_kernel(const uint8_t *__restrict__
     }
 }
 
+// The same workspace layout from bf16 weights in TILE layout (4-face tiles of 2048 bytes): a pure re-layout, so that a
+// bf16 x bf16 GEMM (ttnn.matmul with two bf16 operands) runs on matmul_expanded_kernel too.  One wavefront per (k tile row,
+// 64-column group): the 2 tiles go to LDS with 16 bytes per lane, and every lane gathers the 8 k rows of its column for the
+// four operands.
+__global__ __launch_bounds__(256) void relayout_bf16_kernel(const uint8_t *__restrict__ b, uint8_t *__restrict__ out, uint32_t nt, uint32_t groups,
+                                                            uint32_t items) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[4 * 4096];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const uint32_t item = blockIdx.x * 4 + wave;
+    if (item >= items) return;                                   // no barrier in this kernel
+    const uint32_t g = item % groups, row = item / groups;       // row = slice * kt + k tile row
+    const uint32_t nt0 = g * 2, n_valid = min(2u, nt - nt0);
+    const int c = lane & 31, kh = lane >> 5;
+    const int c16 = c & 15, half = c >> 4;
+    const int t_of_lane = c16 >> 3, fc = (c16 >> 2) & 1, q = c16 & 3;
+    const uint8_t *src = b + ((uint64_t)row * nt + nt0) * 2048;
+    uint8_t *stage = lds + wave * 4096;
+    // a tile past the matrix edge repeats the last one that exists (its columns are never stored by the GEMM)
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+        const uint32_t chunk = l * 64 + lane;                     // 16-byte chunk of the 2 tiles
+        const uint32_t tile = min(chunk >> 7, n_valid - 1);
+        *reinterpret_cast<u32x4 *>(stage + chunk * 16) = *reinterpret_cast<const u32x4 *>(src + tile * 2048 + (chunk & 127) * 16);
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xC07F);                           // the wavefront's own LDS writes have landed
+    uint8_t *dst = out + (uint64_t)item * GROUP_BYTES + lane * 16;
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+            // element (k row 16s + 8kh + i, column fc*16 + q*4 + half*2 + cb) of tile t_of_lane: face 2s + fc, 32 bytes per face row
+            const uint32_t at = t_of_lane * 2048 + (2 * s + fc) * 512 + (8 * kh) * 32 + (q * 4 + half * 2 + cb) * 2;
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = (uint32_t) * reinterpret_cast<const uint16_t *>(stage + at + (2 * i) * 32) |
+                       ((uint32_t) * reinterpret_cast<const uint16_t *>(stage + at + (2 * i + 1) * 32) << 16);
+            *reinterpret_cast<u32x4 *>(dst + (s * 2 + cb) * 1024) = u32x4{w[0], w[1], w[2], w[3]};
+        }
+}
+
 struct ExpandedDev {
     const uint8_t *a;        // bf16
     const uint8_t *w;        // expanded weights (workspace)
@@ -240,13 +283,14 @@ size_t matmul_expanded_workspace_bytes(uint32_t b_batch, uint32_t k, uint32_t n)
     return (size_t)((uint64_t)b_batch * (k / 32) * groups * GROUP_BYTES);
 }
 
+// x.b: packed block-float tiles (x.b_fmt BFLOAT8_B | BFLOAT4_B) or bf16 tiles (x.b_fmt BFLOAT16)
 int matmul_bfp_expanded(const MatmulArgs &x, hipStream_t st) {
     ExpandedDev p{};
     p.a = (const uint8_t *)x.a; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
     p.kt = x.k / 32; p.nt = x.n / 32; p.groups = (p.nt + 1) / 2;
     p.tiles_m = (x.m + 255) / 256; p.tiles_n = (x.n + 255) / 256; p.tiles_n8 = (p.tiles_n + 7) / 8;
-    p.unscale = x.b_fmt == TTMI_BFLOAT8_B ? Wfmt<7>::unscale : Wfmt<3>::unscale;
+    p.unscale = x.b_fmt == TTMI_BFLOAT8_B ? Wfmt<7>::unscale : x.b_fmt == TTMI_BFLOAT4_B ? Wfmt<3>::unscale : 1.0f;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE; p.c_f32 = x.c_dtype == TTMI_FLOAT32;
     const uint64_t blocks = (uint64_t)x.batch * p.tiles_m * p.tiles_n8 * 8;
     const uint64_t items = (uint64_t)x.b_batch * p.kt * p.groups;
@@ -270,8 +314,10 @@ int matmul_bfp_expanded(const MatmulArgs &x, hipStream_t st) {
     const uint32_t expand_blocks = (uint32_t)((items + 3) / 4);
     if (x.b_fmt == TTMI_BFLOAT8_B)
         hipLaunchKernelGGL((expand_kernel<7>), dim3(expand_blocks), dim3(256), 0, st, (const uint8_t *)x.b, (uint8_t *)expanded, p.kt, p.nt, p.groups, (uint32_t)items);
-    else
+    else if (x.b_fmt == TTMI_BFLOAT4_B)
         hipLaunchKernelGGL((expand_kernel<3>), dim3(expand_blocks), dim3(256), 0, st, (const uint8_t *)x.b, (uint8_t *)expanded, p.kt, p.nt, p.groups, (uint32_t)items);
+    else
+        hipLaunchKernelGGL(relayout_bf16_kernel, dim3(expand_blocks), dim3(256), 0, st, (const uint8_t *)x.b, (uint8_t *)expanded, p.nt, p.groups, (uint32_t)items);
     if (int rc = check_launch("expand_kernel")) return rc;
     switch (x.activation) {
         case TTMI_ACT_RELU: hipLaunchKernelGGL((matmul_expanded_kernel<TTMI_ACT_RELU>), dim3((uint32_t)blocks), dim3(512), 0, st, p); break;

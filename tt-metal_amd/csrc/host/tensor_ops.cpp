@@ -386,8 +386,8 @@ Tensor matmul(const Tensor &a, const Tensor &b, bool bcast_batch, const Tensor *
     if (pa.back() != pb[pb.size() - 2])
         raise("TT_FATAL: The width of the first tensor must be equal to the height of the second tensor (a.shape[-1] = " + std::to_string(pa.back()) +
               ", b.shape[-2] = " + std::to_string(pb[pb.size() - 2]) + ")");
-    if (!is_block_float(b.dtype))
-        raise(op + ": this build accelerates block-float weights (BFLOAT8_B / BFLOAT4_B); got " + name_of(b.dtype));
+    if (!is_block_float(b.dtype) && b.dtype != DataType::BFLOAT16)
+        raise(std::string("TT_FATAL: Unsupported data format for input b: ") + name_of(b.dtype));               // bmm_op.cpp:839
     if (a.dtype != DataType::BFLOAT16 && !is_block_float(a.dtype))
         raise(std::string("TT_FATAL: Unsupported data format for input a: ") + name_of(a.dtype));      // bmm_op.cpp:839
     const uint32_t batch_a = (uint32_t)product(pa, 0, pa.size() - 2), batch_b = (uint32_t)product(pb, 0, pb.size() - 2);
@@ -427,9 +427,13 @@ Tensor matmul(const Tensor &a, const Tensor &b, bool bcast_batch, const Tensor *
     Buffer a_tiles = is_block_float(a.dtype) ? typecast_tiles(a.buffer, a.dtype, DataType::BFLOAT16, a_elements, device) : a.buffer;
     const bool packed_out = is_block_float(out_dtype);
     Buffer c = allocate(packed_out ? storage_bytes(out_dtype, Layout::TILE, {batch_a, m, n}) : c_elements * 2, device);
-    check(ttmi_matmul_bfp(a_tiles.data, TTMI_TILE, (const uint32_t *)b.buffer.data, (int)b.dtype, batch_a, batch_b, m, k, n,
-                          bias ? bias_row.data : nullptr, activation, c.data, TTMI_TILE, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0,
-                          stream_of(device)));
+    if (b.dtype == DataType::BFLOAT16)      // two bf16 operands: not the tuned path (the weights are re-laid-out on every call), but the same surface
+        check(ttmi_matmul_bf16(a_tiles.data, TTMI_TILE, b.buffer.data, batch_a, batch_b, m, k, n, bias ? bias_row.data : nullptr, activation, c.data,
+                               TTMI_TILE, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0, stream_of(device)));
+    else
+        check(ttmi_matmul_bfp(a_tiles.data, TTMI_TILE, (const uint32_t *)b.buffer.data, (int)b.dtype, batch_a, batch_b, m, k, n,
+                              bias ? bias_row.data : nullptr, activation, c.data, TTMI_TILE, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0,
+                              stream_of(device)));
     Tensor out;
     out.buffer = std::move(c);
     out.shape.assign(a.shape.begin(), a.shape.end() - 1);

@@ -75,6 +75,7 @@ int matmul_bfp_stream(const MatmulArgs &args, hipStream_t st);
 int matmul_bfp_wide(const MatmulArgs &args, hipStream_t st);     // the streaming kernel with 128-column units
 size_t matmul_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n);
 int matmul_bfp_gated(const MatmulArgs &args, hipStream_t st);   // args.b2 set
+int matmul_bf16(const MatmulArgs &args, hipStream_t st);        // args.b: bf16 tiles, args.b_fmt = TTMI_BFLOAT16
 int matmul_bfp_tiled(const MatmulArgs &args, hipStream_t st);
 int matmul_bfp_expanded(const MatmulArgs &args, hipStream_t st);   // expand the weights to bf16 once, then a bf16 GEMM
 size_t matmul_expanded_workspace_bytes(uint32_t b_batch, uint32_t k, uint32_t n);

@@ -24,7 +24,7 @@ SYMBOLS = (
     "ttmi_pack_rowmajor_as_bfp_tiles", "ttmi_unpack_bfp_tiles_as_rowmajor",
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
     "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_typecast_tiles", "ttmi_device_status", "ttmi_matmul_bfp_static",
-    "ttmi_matmul_bfp_gated_workspace_bytes", "ttmi_matmul_bfp_gated",
+    "ttmi_matmul_bfp_gated_workspace_bytes", "ttmi_matmul_bfp_gated", "ttmi_matmul_bf16_workspace_bytes", "ttmi_matmul_bf16",
 )
 
 _lib = None
@@ -71,6 +71,10 @@ def lib() -> ctypes.CDLL:
         L.ttmi_matmul_bfp_gated_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
         L.ttmi_matmul_bfp_gated.restype = i32
         L.ttmi_matmul_bfp_gated.argtypes = [vp, i32, vp, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, ctypes.c_size_t, vp]
+        L.ttmi_matmul_bf16_workspace_bytes.restype = ctypes.c_size_t
+        L.ttmi_matmul_bf16_workspace_bytes.argtypes = [u32, u32, u32]
+        L.ttmi_matmul_bf16.restype = i32
+        L.ttmi_matmul_bf16.argtypes = [vp, i32, vp, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, ctypes.c_size_t, vp]
         L.ttmi_matmul_bfp_static.restype = i32
         L.ttmi_matmul_bfp_static.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp]
         L.ttmi_typecast_tiles.restype = i32
@@ -210,6 +214,22 @@ def matmul_bfp(a, a_layout: int, b_words, b_fmt: int, batch: int, b_batch: int, 
     if c_layout == ROW_MAJOR:
         return c.view(batch, m, n)
     return c
+
+
+def matmul_bf16(a, a_layout: int, b_tiles, batch: int, b_batch: int, m: int, k: int, n: int, *, bias=None, activation: int = ACT_NONE,
+                c_layout: int = ROW_MAJOR, out_dtype=None, workspace=None):
+    """bf16 x bf16 (ttmi_matmul_bf16): b_tiles = bf16 weights in TILE layout; the rest as for matmul_bfp."""
+    import torch
+
+    out_dtype = out_dtype or torch.bfloat16
+    mp = padded(m) if c_layout == TILE else m
+    c = torch.empty(batch * mp * n, dtype=out_dtype, device=a.device)
+    ws_ptr, ws_bytes = None, 0
+    if workspace is not None:
+        ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
+    check(lib().ttmi_matmul_bf16(_dev(a), a_layout, _dev(b_tiles), batch, b_batch, m, k, n, _dev(bias) if bias is not None else None, activation,
+                                 _dev(c), c_layout, _torch_dtype_code(c), ws_ptr, ws_bytes, _stream()))
+    return c.view(batch, m, n) if c_layout == ROW_MAJOR else c
 
 
 def matmul_bfp_gated(a, a_layout: int, gate_words, up_words, b_fmt: int, batch: int, b_batch: int, m: int, k: int, n: int, *,
