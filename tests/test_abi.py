@@ -51,7 +51,8 @@ def test_matmul_workspace_sizes_follow_the_decomposition():
     assert ws(1, 32, 4544, 18176, 3) == 142 * 3 * 16384        # 142 groups of 128 columns, 512 // 143 = 3 k ranges each
     assert ws(1, 32, 18176, 4544, 3) == 36 * 7 * 16384         # 36 groups (the last one half empty), 256 // 36 = 7
     assert ws(1, 32, 64, 4096, 3) == 0                         # 2 k-tiles: never shared
-    assert ws(1, 64, 4544, 18176, 3) == 0                      # two bands, 64-column kernel: 568 groups fill the chip
+    assert ws(1, 64, 4544, 18176, 3) == 142 * 3 * 2 * 16384    # two bands per workgroup of the 128-column kernel: two slots each
+    assert ws(1, 96, 4544, 18176, 3) == 0                      # three bands, 64-column kernel: 3 x 284 groups fill the chip
     assert ws(1, 256, 4096, 4096, 3) == 0                      # fused tiled kernels
     assert ws(1, 2048, 4096, 14336, 3) == 4096 * 14336 * 2     # expanded weights
     assert ws(0, 32, 64, 64, 3) == 0
@@ -121,7 +122,9 @@ def test_every_unit_has_exactly_one_workgroup_and_collectors_come_last(shape, wi
     L.ttmi_test_stream_decomposition(*shape, wide, out)
     groups, kt, split, workgroups = (int(x) for x in out)
     batch, m, k, n = shape
-    assert kt == k // 32 and groups == batch * -(-m // 32) * -(-(n // 32) // (4 if wide else 2))
+    bands = -(-m // 32)
+    band_sets = -(-bands // 2) if wide and m > 32 else bands        # the 128-column kernel takes two bands per workgroup above 32 rows
+    assert kt == k // 32 and groups == batch * band_sets * -(-(n // 32) // (4 if wide else 2))
     assert split >= 1 and workgroups == groups * split
     assert split == 1 or kt // split >= 2                     # every wavefront of a shared output keeps work to do
     starts = [L.ttmi_test_range_start(kt, split, i) for i in range(min(workgroups, 600) + 1)]

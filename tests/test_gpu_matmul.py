@@ -365,6 +365,21 @@ def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch, layout):
     print(name, "pcc", pcc)
 
 
+@pytest.mark.parametrize("m", [64, 128 - 3])
+@pytest.mark.parametrize("name,k,n,fmt", [("falcon_h_to_4h", 4544, 18176, "bfp8_b"), ("falcon_4h_to_h", 18176, 4544, "bfp8_b"), ("mistral_gate", 4096, 14336, "bfp4_b")])
+def test_two_and_four_row_bands_full_size(oracle, name, m, k, n, fmt):
+    """64 and 125 rows on the decode shapes (the two-band form of the 128-column kernel: the weights once per 64 rows; 125 rows
+    leave the last band ragged), every output element against the float64 product with the oracle-unpacked weights."""
+    a_bits = workloads.activations_bf16(m, k, seed=84)
+    words = capi.pack_tensor(FMT[fmt], dev(workloads.weights_f32(k, n, seed=85)))
+    w_unpacked = oracle_unpacked(oracle, FMT[fmt], words, k, n)[0]
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, FMT[fmt], 1, 1, m, k, n)
+    check_on_gpu(c[0], a_bits, w_unpacked, k)
+    if m % 32 == 0:
+        tiles = capi.matmul_bfp(capi.tilize(bf16_dev(a_bits)), capi.TILE, words, FMT[fmt], 1, 1, m, k, n, c_layout=capi.TILE)
+        assert torch.equal(capi.untilize(tiles, (1, m, n)).view(torch.int16), c.view(torch.int16))
+
+
 @pytest.mark.parametrize("layout", [capi.ROW_MAJOR, capi.TILE])
 def test_prefill_shape_full_size_every_row(oracle, layout):
     """[2048,4096] x BFP8 [4096,14336]: all 2048 x 14336 outputs against the float64 product with the weights as the CPU

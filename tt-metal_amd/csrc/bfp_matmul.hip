@@ -43,6 +43,7 @@ struct MatmulDev {
     int drop_partial_sums;   // test only: producers keep their sums to themselves, so that the wait must give up
     uint32_t batch, b_batch, m, k, n;
     uint32_t mt, kt, nt, ngroups;
+    uint32_t mt_sets;        // 128-column kernel: sets of row bands that share a workgroup (mt, or ceil(mt / 2) in the two-band form)
     uint32_t groups;         // batch * mt * ngroups
     uint32_t workgroups;     // P
     uint32_t units;          // U = batch * mt * ngroups * kt
@@ -460,14 +461,19 @@ constexpr size_t WIDE_SLOT_BYTES = 32 * WIDE_COLS * sizeof(float);
 // NB = 2 is the gated form, C = act(A . B) * (A . B2) (silu(x w1) * (x w3) of a gated MLP in one launch): a unit is then
 // the same k-tile and column group of both weight matrices, which share the activations; every workgroup keeps two sets
 // of sums and hands over two slots.
-template <int W, int ACT, int NB>
+// MB = 2 is the two-band form for 33 to 127 rows: a unit is one k-tile and column group of the weights against two
+// 32-row bands of the activations, so that the weights are streamed once per 64 rows.  Either way a workgroup keeps
+// X = NB * MB sets of sums (one of NB, MB is 1).
+template <int W, int ACT, int NB, int MB>
 __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wide_kernel(const MatmulDev p) {
     using F = WideFmt<W>;
+    constexpr int X = NB * MB;
+    static_assert(X <= 2, "one of NB, MB is 1");
     constexpr int UNIT_BYTES = NB * F::unit_bytes;     // a stage holds the unit's tiles of every weight matrix
     constexpr int WAVE_LDS = WIDE_STAGES * UNIT_BYTES;
     constexpr int LDS_BYTES = WIDE_REDUCE_BYTES > WAVES * WAVE_LDS ? WIDE_REDUCE_BYTES : WAVES * WAVE_LDS;
     constexpr int NLOAD = F::loads;
-    constexpr int PER = NB * NLOAD + 2;                // vector-memory requests per unit
+    constexpr int PER = NB * NLOAD + 2 * MB;           // vector-memory requests per unit
     __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
 
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
@@ -486,7 +492,7 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     const uint32_t og = me / p.split, part = me - og * p.split;
     const uint32_t k_begin = (part * p.kt) / p.split, k_end = ((part + 1) * p.kt) / p.split;
     const uint32_t ng = og % p.ngroups, band = og / p.ngroups;
-    const uint32_t mt = band % p.mt, bb = band / p.mt;
+    const uint32_t mt = (band % p.mt_sets) * MB, bb = band / p.mt_sets;       // first row band of this workgroup
     const uint32_t nt0 = ng * WIDE_TILES;
     const uint32_t n_valid = min((uint32_t)WIDE_TILES, p.nt - nt0);
 
@@ -502,31 +508,35 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     const uint64_t w_step = (uint64_t)WAVES * p.nt * F::tile_bytes;
     // activations of one unit for this lane: row c32 of the band, k = kt*32 + 16s + 8kh .. + 7 for s = 0, 1;
     // rows past M read row M-1 and are never stored
-    const uint8_t *aptr;
+    // (a second band past the last one repeats the last one and is never stored)
+    const uint8_t *aptr[MB];
     uint32_t a_second, a_step;
-    if (p.a_tiled) {
-        aptr = p.a + (((uint64_t)bb * p.mt + mt) * p.kt + k_begin + wave) * 2048 + (c32 >> 4) * 1024 + (c32 & 15) * 32 + kh * 16;
-        a_second = 512; a_step = WAVES * 2048;
-    } else {
-        const uint32_t r0 = min(mt * 32 + c32, p.m - 1);
-        aptr = p.a + (((uint64_t)bb * p.m + r0) * p.k + (k_begin + wave) * 32 + kh * 8) * 2;
-        a_second = 32; a_step = WAVES * 64;
-    }
-
-    f32x16 acc[NB][4];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
+    for (int mb = 0; mb < MB; ++mb) {
+        const uint32_t band_mt = min(mt + mb, p.mt - 1);
+        if (p.a_tiled) {
+            aptr[mb] = p.a + (((uint64_t)bb * p.mt + band_mt) * p.kt + k_begin + wave) * 2048 + (c32 >> 4) * 1024 + (c32 & 15) * 32 + kh * 16;
+        } else {
+            const uint32_t r0 = min(band_mt * 32 + c32, p.m - 1);
+            aptr[mb] = p.a + (((uint64_t)bb * p.m + r0) * p.k + (k_begin + wave) * 32 + kh * 8) * 2;
+        }
+    }
+    if (p.a_tiled) { a_second = 512; a_step = WAVES * 2048; } else { a_second = 32; a_step = WAVES * 64; }
+
+    f32x16 acc[X][4];
+#pragma unroll
+    for (int x = 0; x < X; ++x)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) acc[nb][j][i] = 0.f;
+            for (int i = 0; i < 16; ++i) acc[x][j][i] = 0.f;
     // The ring registers are cleared by instructions the compiler cannot see through: entries it knows to be zero it
     // would keep in a shared constant register and copy loaded entries around at joins, while their loads are in flight.
-    u32x4 a_ring[WIDE_STAGES][2];
+    u32x4 a_ring[WIDE_STAGES][2 * MB];                  // [stage][2 * band + slab]
 #pragma unroll
     for (int s = 0; s < WIDE_STAGES; ++s)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < 2 * MB; ++h)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 uint32_t zero;
@@ -547,18 +557,22 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
                                                  16, 0, WEIGHTS_ONCE);
             wptr[nb] += w_step;
         }
-        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][0]) : "v"(aptr) : "memory");
-        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][1]) : "v"(aptr + a_second) : "memory");
-        aptr += a_step;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][2 * mb]) : "v"(aptr[mb]) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][2 * mb + 1]) : "v"(aptr[mb] + a_second) : "memory");
+            aptr[mb] += a_step;
+        }
     };
     auto work = [&](auto stage_tag, auto younger_tag, bool refill) __attribute__((always_inline)) {
         constexpr int S = decltype(stage_tag)::value;
         constexpr int YOUNGER = decltype(younger_tag)::value;
         if (YOUNGER >= 0) wait_vmcnt<(YOUNGER < 0 ? 0 : YOUNGER) * PER>();   // < 0: the caller has waited
-        asm volatile("" : "+v"(a_ring[S][0]), "+v"(a_ring[S][1]) :: "memory");
-        u32x4 a_now[2];
+        if constexpr (MB == 2) asm volatile("" : "+v"(a_ring[S][0]), "+v"(a_ring[S][1]), "+v"(a_ring[S][2 * MB - 2]), "+v"(a_ring[S][2 * MB - 1]) :: "memory");
+        else asm volatile("" : "+v"(a_ring[S][0]), "+v"(a_ring[S][1]) :: "memory");
+        u32x4 a_now[2 * MB];
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+        for (int s = 0; s < 2 * MB; ++s)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 uint32_t moved;
@@ -566,9 +580,9 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
                 a_now[s][e] = moved;
             }
         // hidden-one form (bfp_dequant.h): A.W = 2 (A.hi - A.lo); the subtraction is an MFMA with the negated activations
-        u32x4 a_neg[2];
+        u32x4 a_neg[2 * MB];
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+        for (int s = 0; s < 2 * MB; ++s)
 #pragma unroll
             for (int e = 0; e < 4; ++e) a_neg[s][e] = a_now[s][e] ^ 0x80008000u;
         // one weight matrix after the other; the stage is handed to the unit WIDE_STAGES ahead once its last LDS read has returned
@@ -583,14 +597,20 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
             bf16x8 hi[4], lo[4];
             slab_expand_hidden<W>(raw0, q, hi, lo);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[0]), hi[j], acc[nb][j], 0, 0, 0);
+            for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[0]), lo[j], acc[nb][j], 0, 0, 0);
+                for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb]), hi[j], acc[nb * MB + mb][j], 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[2 * mb]), lo[j], acc[nb * MB + mb][j], 0, 0, 0);
+            }
             slab_expand_hidden<W>(raw1, q, hi, lo);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[1]), hi[j], acc[nb][j], 0, 0, 0);
+            for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[1]), lo[j], acc[nb][j], 0, 0, 0);
+                for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb + 1]), hi[j], acc[nb * MB + mb][j], 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[2 * mb + 1]), lo[j], acc[nb * MB + mb][j], 0, 0, 0);
+            }
         });
     };
 
@@ -624,10 +644,10 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     // In two passes (operands j = 0, 1, then 2, 3; 32 KB each) every wavefront writes its accumulator registers as
     // float4 (acc[j][4q4 .. 4q4+3]); wavefront w then keeps q4 = w: rows 8w + 4kh + r (r = 0..3), columns 4*c32 + j.
     float4 *red = reinterpret_cast<float4 *>(lds);
-    float mine[NB][4][4];   // [weight matrix][r][j]
+    float mine[X][4][4];   // [set of sums][r][j]
 #pragma unroll
-    for (int pass = 0; pass < 2 * NB; ++pass) {
-        const int nb = pass >> 1;
+    for (int pass = 0; pass < 2 * X; ++pass) {
+        const int nb = pass >> 1;                         // the set of sums of this pass
         __syncthreads();
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj)
@@ -654,10 +674,11 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     // A chunk = 4 adjacent columns of one row = what one lane holds per r: chunk number (w * 4 + r) * 64 + lane, 1024
     // per output group.  Stores chunk `idx` of output group `group` (sums still carry the common factor; in the gated form
     // the activation applies to the first matrix's sums, which the second matrix's sums then multiply).
-    auto store_chunk = [&](uint32_t group, uint32_t idx, const float (&sums)[NB][4]) __attribute__((always_inline)) {
+    // `mb` is the row band inside the group (two-band form).
+    auto store_band = [&](uint32_t group, uint32_t idx, uint32_t mb, const float (&sums)[NB][4]) __attribute__((always_inline)) {
         const uint32_t lane_of = idx & 63, r_of = (idx >> 6) & 3, w_of = idx >> 8;
         const uint32_t c32_of = lane_of & 31, t_of = c32_of >> 3, fc_of = (c32_of >> 2) & 1, q_of = c32_of & 3;
-        const uint32_t band_of = group / p.ngroups, mt_of = band_of % p.mt, bb_of = band_of / p.mt;
+        const uint32_t band_of = group / p.ngroups, mt_of = (band_of % p.mt_sets) * MB + mb, bb_of = band_of / p.mt_sets;
         const uint32_t nt_of = (group % p.ngroups) * WIDE_TILES + t_of;
         const uint32_t row_in_band = w_of * 8 + (lane_of >> 5) * 4 + r_of, row = mt_of * 32 + row_in_band;
         if (nt_of >= p.nt || row >= p.m) return;
@@ -713,14 +734,29 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
         }
     };
 
+    // all sets of sums of a chunk: the two matrices of the gated form make one output, the two bands two
+    auto store_chunk = [&](uint32_t group, uint32_t idx, const float (&sums)[X][4]) __attribute__((always_inline)) {
+        if constexpr (MB == 1) {
+            store_band(group, idx, 0, sums);
+        } else {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                float one[NB][4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) one[0][j] = sums[mb][j];
+                store_band(group, idx, mb, one);
+            }
+        }
+    };
+
     if (p.split == 1) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            float sums[NB][4];
+            float sums[X][4];
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
+            for (int x = 0; x < X; ++x)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) sums[nb][j] = mine[nb][r][j];
+                for (int j = 0; j < 4; ++j) sums[x][j] = mine[x][r][j];
             store_chunk(og, (wave * 4 + r) * 64 + lane, sums);
         }
         return;
@@ -734,10 +770,10 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     // dispatched later, so they finish.
     float4 *const all_slots = reinterpret_cast<float4 *>(p.slots);
     if (computes) {
-        // slot (me, nb) = 1024 chunks from chunk (me * NB + nb) * 1024 on
+        // slot (me, x) = 1024 chunks from chunk (me * X + x) * 1024 on
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            float4 *slot = all_slots + (((uint64_t)me * NB + nb) * 16 + wave * 4) * 64 + lane;
+        for (int nb = 0; nb < X; ++nb) {
+            float4 *slot = all_slots + (((uint64_t)me * X + nb) * 16 + wave * 4) * 64 + lane;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 u32x4 v;
@@ -755,30 +791,30 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     for (uint32_t idx0 = lo; idx0 < hi; idx0 += 256) {
         const bool active = idx0 + threadIdx.x < hi;                       // idle lanes re-read the last chunk and drop it
         const uint32_t idx = active ? idx0 + threadIdx.x : hi - 1;
-        float4 *const at = all_slots + (uint64_t)target * p.split * NB * 1024 + idx;   // contributor c, matrix nb: at + (c * NB + nb) * 1024
+        float4 *const at = all_slots + (uint64_t)target * p.split * X * 1024 + idx;   // contributor c, set x: at + (c * X + x) * 1024
         uint32_t spins = 0;
         bool waiting;
         // workgroups with nothing else to do poll cheaply first (one contributor); then everything, checked word by word
         if (!computes) do {
-            u32x4 probe = slot_load_issue(at + (uint64_t)(p.split * NB - 1) * 1024);
+            u32x4 probe = slot_load_issue(at + (uint64_t)(p.split * X - 1) * 1024);
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(probe)::"memory");
             const bool missing = active && (probe[0] == SLOT_EMPTY || probe[1] == SLOT_EMPTY || probe[2] == SLOT_EMPTY || probe[3] == SLOT_EMPTY);
             waiting = __ballot(missing) != 0 && ++spins < p.spin_limit;
             if (waiting) __builtin_amdgcn_s_sleep(8);
         } while (waiting);
-        float sums[NB][4];
+        float sums[X][4];
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
+        for (int x = 0; x < X; ++x)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) sums[nb][j] = 0.f;
+            for (int j = 0; j < 4; ++j) sums[x][j] = 0.f;
         // N contributors at a time, N a compile-time constant: loads under a condition would have the compiler merge
         // loaded and unloaded registers (that is, copy them) while the loads are in flight
         auto collect = [&](auto count_tag, uint32_t c0) __attribute__((always_inline)) {
-            constexpr int N = decltype(count_tag)::value * NB;          // slots: those of a contributor lie side by side
+            constexpr int N = decltype(count_tag)::value * X;           // slots: those of a contributor lie side by side
             u32x4 got[N];
             do {
 #pragma unroll
-                for (int u = 0; u < N; ++u) got[u] = slot_load_issue(at + ((uint64_t)c0 * NB + u) * 1024);
+                for (int u = 0; u < N; ++u) got[u] = slot_load_issue(at + ((uint64_t)c0 * X + u) * 1024);
 #pragma unroll
                 for (int u = 0; u < N; ++u) asm volatile("s_waitcnt vmcnt(0)" : "+v"(got[u])::"memory");
                 bool missing = false;
@@ -794,8 +830,8 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
 #pragma unroll
             for (int u = 0; u < N; ++u) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) sums[u % NB][j] += __uint_as_float(got[u][j]);
-                if (active) slot_store(at + ((uint64_t)c0 * NB + u) * 1024, empty);      // ready for the next launch
+                for (int j = 0; j < 4; ++j) sums[u % X][j] += __uint_as_float(got[u][j]);
+                if (active) slot_store(at + ((uint64_t)c0 * X + u) * 1024, empty);       // ready for the next launch
             }
         };
         uint32_t c0 = 0;
@@ -817,14 +853,18 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
 // ---------------------------------------------------------------------------------------------------------
 // host side: decomposition, workspace, launch
 // ---------------------------------------------------------------------------------------------------------
-struct Decomposition { uint32_t mt, kt, nt, ngroups, workgroups, split; uint64_t groups, units; };
+struct Decomposition { uint32_t mt, mt_sets, kt, nt, ngroups, workgroups, split; uint64_t groups, units; };
+
+// two_bands: the 128-column kernel takes two 32-row bands per workgroup (33 to 127 rows, not gated)
+static bool two_bands(uint32_t m, bool wide, bool gated) { return wide && !gated && m > 32; }
 
 static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, bool wide, bool gated = false) {
     Decomposition d{};
     const uint32_t group_tiles = wide ? WIDE_TILES : GROUP_TILES;
     d.mt = (m + 31) / 32; d.kt = k / 32; d.nt = n / 32;
+    d.mt_sets = two_bands(m, wide, gated) ? (d.mt + 1) / 2 : d.mt;
     d.ngroups = (d.nt + group_tiles - 1) / group_tiles;
-    d.groups = (uint64_t)batch * d.mt * d.ngroups;
+    d.groups = (uint64_t)batch * d.mt_sets * d.ngroups;
     d.units = d.groups * d.kt;
     // Workgroups to aim for, every output's k range being cut into as many parts as get there (every wavefront keeping
     // >= 2 k-tiles).  64-column kernel: 256 CUs x 3 workgroups of 4 wavefronts when the output groups alone nearly get
@@ -844,9 +884,9 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     return d;
 }
 
-static size_t slot_bytes_needed(const Decomposition &d, bool wide, bool gated = false) {
+static size_t slot_bytes_needed(const Decomposition &d, bool wide, bool two_sets = false) {
     if (d.split == 1) return 0;                     // every output belongs to one workgroup: no slot is touched
-    return wide ? (size_t)d.workgroups * WIDE_SLOT_BYTES * (gated ? 2 : 1) : (size_t)2 * d.workgroups * SLOT_BYTES;
+    return wide ? (size_t)d.workgroups * WIDE_SLOT_BYTES * (two_sets ? 2 : 1) : (size_t)2 * d.workgroups * SLOT_BYTES;
 }
 
 static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
@@ -856,7 +896,7 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     const bool gated = x.b2 != nullptr;
     if (gated && !wide) return fail(TTMI_ERR_UNSUPPORTED, "matmul: the gated form runs on the 128-column kernel only");
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
-    p.mt = d.mt; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.groups = (uint32_t)d.groups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
+    p.mt = d.mt; p.mt_sets = d.mt_sets; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.groups = (uint32_t)d.groups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
     p.split = d.split;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE;
     p.c_f32 = x.c_dtype == TTMI_FLOAT32;
@@ -865,7 +905,8 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     if ((reinterpret_cast<uintptr_t>(x.a) | reinterpret_cast<uintptr_t>(x.b) | reinterpret_cast<uintptr_t>(x.b2) | reinterpret_cast<uintptr_t>(x.c)) & 15u)
         return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: a, b and c must be 16-byte aligned");
     if (d.units > 0x7fffffffull || d.groups * d.split > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");
-    const size_t need = slot_bytes_needed(d, wide, gated);
+    const bool bands2 = two_bands(x.m, wide, gated);
+    const size_t need = slot_bytes_needed(d, wide, gated || bands2);
     void *slots = nullptr;
     bool fill = false;
     size_t fill_bytes = need;
@@ -900,8 +941,9 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     p.spin_limit = knob_or(TTMI_KNOB_SPIN_LIMIT, SLOT_SPIN_LIMIT);
     p.drop_partial_sums = (int)knob_or(TTMI_KNOB_DROP_PARTIAL_SUMS, 0);
 #define TTMI_LAUNCH(W, ACT)                                                                                     \
-    if (wide && gated) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 2>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
-    else if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
+    if (wide && gated) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 2, 1>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
+    else if (wide && bands2) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 2>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
+    else if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 1>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
     else hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
 #define TTMI_LAUNCH_ACT(W)                                              \
     switch (x.activation) {                                             \
@@ -919,10 +961,12 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
 int matmul_bfp_stream(const MatmulArgs &x, hipStream_t st) { return launch_streaming(x, st, false); }
 int matmul_bfp_wide(const MatmulArgs &x, hipStream_t st) { return launch_streaming(x, st, true); }
 
-// Which kernel a shape goes to.  Up to 127 rows the weights are streamed once per 32-row band (HBM-bound): one band in
-// 128-column units, several bands in 64-column units (measured: 43 against 46 us for 64 rows of the Falcon shape).
-// Taller activations are MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows on (two or more
-// 256-row blocks share every weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
+// Which kernel a shape goes to.  Up to 127 rows the weights are streamed (HBM-bound): one 32-row band in 128-column units;
+// two or four bands in the two-band form of the same kernel, which streams the weights once per 64 rows (measured at 64
+// rows, TILE layout: 32.8 against 44.1 us for the Falcon h_to_4h shape, 29.8 against 41.4 us for 4h_to_h, no difference for
+// Mistral's shapes); three bands in 64-column units, once per band (the two-band form would compute a fourth band for
+// nothing: 57 against 53 us).  Taller activations are MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows
+// on (two or more 256-row blocks share every weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
 // The test entry point can force a kernel (TTMI_KNOB_MATMUL_KERNEL).
 enum class Kernel { Stream = 1, Wide = 2, Tile = 3, Expanded = 4 };
 static Kernel choose_kernel(uint32_t m) {
@@ -930,7 +974,7 @@ static Kernel choose_kernel(uint32_t m) {
     if (knob(TTMI_KNOB_MATMUL_KERNEL, &forced) && forced >= 1 && forced <= 4) return (Kernel)forced;
     if (m >= 512) return Kernel::Expanded;
     if (m >= 128) return Kernel::Tile;
-    return m <= 32 ? Kernel::Wide : Kernel::Stream;
+    return m <= 32 || ((m + 31) / 32) % 2 == 0 ? Kernel::Wide : Kernel::Stream;
 }
 
 size_t matmul_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
@@ -947,7 +991,7 @@ size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n
         default: break;
     }
     const bool wide = kernel == Kernel::Wide;
-    return slot_bytes_needed(decompose(batch, m, k, n, wide), wide);
+    return slot_bytes_needed(decompose(batch, m, k, n, wide), wide, two_bands(m, wide, false));
 }
 
 int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
