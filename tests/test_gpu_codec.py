@@ -95,6 +95,49 @@ def test_rounding_boundaries_bit_exact(oracle, fmt, exponents):
 
 
 @pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_whole_block_kernel_bit_exact(oracle, fmt):
+    """Tensors of at least 512 whole blocks (32 rows x 256 fp32 columns) take the straight-line pack kernel: ordinary rows by
+    float arithmetic on four codes at a time, wavefronts with any other row by the integer recipe.  Special values (NaN, Inf,
+    subnormals, +-0, rows that are not fixed points of pack/unpack/pack), ties / near-ties / saturation in every exponent
+    range, and a source with row and batch strides; every packed word against the oracle."""
+    shape = (2, 1, 1024, 2048)
+    cases = [workloads.normal_tensor(shape, seed=61), special_values(shape, seed=62)]
+    # mostly ordinary wavefronts with the odd element inside: -0, subnormals, the largest floats, and a NaN or Inf in a few rows
+    rng = np.random.default_rng(60)
+    sparse = workloads.normal_tensor(shape, seed=59).reshape(-1).view(np.uint32).copy()
+    pool = np.array([0x80000000, 0x00000001, 0x807FFFFF, 0x7F7FFFFF, 0xFF7FFFFF, 0x00800000, 0x3EFFFFFF, 0x00000000], dtype=np.uint32)
+    at = rng.random(sparse.size) < 0.02
+    sparse[at] = pool[rng.integers(0, pool.size, size=int(at.sum()))]
+    at = rng.random(sparse.size) < 1e-5
+    sparse[at] = np.array([0x7F800000, 0xFFC00001], dtype=np.uint32)[rng.integers(0, 2, size=int(at.sum()))]
+    cases.append(sparse.view(np.float32).reshape(shape))
+    cases += [rounding_boundaries(fmt, shape, 63 + k, e) for k, e in enumerate([(32, 33, 100, 127, 128, 200, 254), (31, 32, 127), (8, 20, 31, 40)])]
+    for x in cases:
+        want = oracle.from_torch_bfp_tiles(fmt, x)
+        assert np.array_equal(words_np(capi.pack_tensor(fmt, dev(x))), want)
+    x = cases[1]
+    big = np.full((2, 1024 + 3, 2048 + 64), np.float32(7.0))
+    big[:, :1024, :2048] = x.reshape(2, 1024, 2048)
+    d = dev(big)
+    out = torch.empty(capi.lib().ttmi_tiled_size_bytes(fmt, 2, 1024, 2048) // 4, dtype=torch.int32, device="cuda")
+    capi.check(capi.lib().ttmi_pack_rowmajor_as_bfp_tiles(fmt, d.data_ptr(), capi.FLOAT32, 2, 1024, 2048, 2048 + 64, (1024 + 3) * (2048 + 64), out.data_ptr(), None))
+    torch.cuda.synchronize()
+    assert np.array_equal(words_np(out), oracle.from_torch_bfp_tiles(fmt, x))
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_whole_block_kernel_bf16_source_bit_exact(oracle, fmt):
+    """The same kernel from a bf16 source (blocks of 32 rows x 512 columns): a stress mixture and the special patterns."""
+    shape = (1, 1, 4096, 2048)
+    n = int(np.prod(shape))
+    for x32 in (workloads.stress_mixture((1, 1, 1, n), seed=71).reshape(shape), special_values(shape, seed=72)):
+        bits = (x32.view(np.uint32) >> 16).astype(np.uint16)                   # any bf16 pattern will do: truncate
+        want = oracle.from_torch_bfp_tiles(fmt, workloads.bf16_bits_to_f32(bits))
+        got = capi.pack_tensor(fmt, dev(bits.view(np.int16)).view(torch.bfloat16))
+        assert np.array_equal(words_np(got), want)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
 @pytest.mark.parametrize("shape", [(1, 1, 64, 96), (2, 1, 5, 40), (1, 1, 32, 24)])
 def test_bf16_source_bit_exact(oracle, fmt, shape):
     bits = workloads.f32_to_bf16_bits_rne(workloads.stress_mixture((1, 1, 1, -(-int(np.prod(shape)) // 16) * 16), seed=23).reshape(-1)[: int(np.prod(shape))]).reshape(shape)

@@ -235,6 +235,120 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// pack of a row-major tensor whose blocks are all whole (h a multiple of 32, w a multiple of the block width, every lane
+// may use one 16-byte load): the same walk as pack_kernel<.., SRC_TENSOR, true, 0> in straight-line code.  Wavefront `wave`
+// reads rows 8 wave .. 8 wave + 7 of the block, one row (1 KiB) per load; lane = (tile, face column, quarter or half of the
+// face row), the same for all eight rows, so everything but the row is fixed per lane and the LDS addresses of the eight
+// items differ by constants.  Codes of ordinary rows (see pack_kernel) come from float arithmetic:
+//     floor(v + 1/2),  v = |x| * 2^(126+W-E)  (an exact product)   ==   trunc(fma(|x|, 2^(126+W-E), 1/2 - 2^-25))
+// for every 24-bit mantissa and every exponent gap (the fma rounds the exact sum once, to nearest even; with 1/2 itself the
+// single case v = 1/2 - 2^-25 would round up to 1), v + 1/2 < 2^W + 1/2, so a code exceeds 2^W - 1 only by being 2^W.
+// Signs, saturation and "no sign on a zero mantissa" are applied to the four codes of a dword at once.  Wavefronts with a row
+// that is not ordinary redo their eight items with the integer recipe.
+// ---------------------------------------------------------------------------------------------------------
+template <int W, int ELEM>
+__global__ __launch_bounds__(256) void pack_whole_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                         const CodecShape s) {
+    using F = Fmt<W>;
+    using I = Item<ELEM, 0>;
+    constexpr int TPB = I::TPB, EPL = I::EPL, LPR = I::LPR, ITS = 8;
+    constexpr int lane_bytes = EPL * (W + 1) / 8;               // 4, 8 (bfp8) or 2, 4 (bfp4)
+    constexpr uint32_t ONES = 0x01010101u, TOP = ONES << W, LOW = TOP - ONES;      // per byte: 2^W, 2^W - 1
+    __shared__ __attribute__((aligned(16))) uint8_t stage[TPB * F::tile_bytes];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t cg = blockIdx.x % s.col_groups;
+    const uint64_t rest = blockIdx.x / s.col_groups;
+    const uint32_t tr = (uint32_t)(rest % s.ht);
+    const uint64_t b = rest / s.ht;
+    const uint64_t tile0 = (b * s.ht + tr) * s.wt + (uint64_t)cg * TPB;
+    const uint8_t *p = src + (b * s.batch_stride + (uint64_t)(tr * 32 + wave * 8) * s.row_stride + (uint64_t)cg * TPB * 32) * ELEM + lane * 16;
+
+    uint4 raw[ITS];
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) raw[it] = *reinterpret_cast<const uint4 *>(p + (uint64_t)it * s.row_stride * ELEM);
+
+    const int t = lane / (2 * LPR), fc = (lane / LPR) & 1, q = lane % LPR;
+    const int face = (wave >> 1) * 2 + fc, i0 = (wave & 1) * 8;
+    uint8_t *tile = stage + t * F::tile_bytes;
+    uint8_t *row0 = tile + 64 + face * F::face_bytes + i0 * F::row_bytes + q * lane_bytes;
+
+    auto put = [&](int it, uint32_t lo, uint32_t hi) __attribute__((always_inline)) {
+        uint8_t *row = row0 + it * F::row_bytes;
+        if (lane_bytes == 2) *reinterpret_cast<uint16_t *>(row) = (uint16_t)lo;
+        else if (lane_bytes == 4) *reinterpret_cast<uint32_t *>(row) = lo;
+        else *reinterpret_cast<uint2 *>(row) = make_uint2(lo, hi);
+    };
+    // four codes, one per byte (m <= 2^W each), with the sign bytes of their elements (sign in bit 7): saturate, put the
+    // sign on every code whose mantissa is not zero
+    auto finish = [&](uint32_t m4, uint32_t sign4) __attribute__((always_inline)) -> uint32_t {
+        m4 -= (m4 & TOP) >> W;                                   // 2^W -> 2^W - 1
+        const uint32_t nonzero = m4 + LOW;                       // bit W of a byte set iff its code is not zero
+        return (((W == 7 ? sign4 : sign4 >> 4) & nonzero) & TOP) | m4;
+    };
+    // bfp4: the low nibbles of four bytes -> 16 bits
+    auto nibbles = [&](uint32_t c4) __attribute__((always_inline)) -> uint32_t {
+        const uint32_t pairs = c4 | (c4 >> 4);                   // bytes 0 and 2 hold a pair each
+        return __builtin_amdgcn_perm(0u, pairs, 0x0c0c0200u);
+    };
+
+    uint32_t exps[2] = {0u, 0u};
+    bool odd = false;
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) {
+        uint32_t bits[EPL];
+        expand<ELEM>(raw[it], bits);
+        uint32_t top = 0;                                        // largest |x| of the lane, as bits shifted up by one
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) { const uint32_t a = bits[e] << 1; top = a > top ? a : top; }
+        top = row_max<LPR>(top);
+        const uint32_t shared = top >> 24;
+        odd |= (shared < 32u && top != 0u) || shared == 255u;
+        exps[it >> 2] |= shared << (8 * (it & 3));
+        const float scale = shared < 32u ? 0.f : __uint_as_float((253u + (uint32_t)W - shared) << 23);
+        uint32_t m4[EPL / 4], sign4[EPL / 4];
+#pragma unroll
+        for (int g = 0; g < EPL / 4; ++g) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                m |= (uint32_t)__builtin_fmaf(fabsf(__uint_as_float(bits[4 * g + e])), scale, 0.5f - 0x1p-25f) << (8 * e);
+            m4[g] = m;
+            if (ELEM == 4) sign4[g] = __builtin_amdgcn_perm(raw[it].y, raw[it].x, 0x0c0c0703u) | __builtin_amdgcn_perm(raw[it].w, raw[it].z, 0x07030c0cu);
+            else sign4[g] = g == 0 ? __builtin_amdgcn_perm(raw[it].y, raw[it].x, 0x07050301u) : __builtin_amdgcn_perm(raw[it].w, raw[it].z, 0x07050301u);
+        }
+        if (W == 7) put(it, finish(m4[0], sign4[0]), EPL == 8 ? finish(m4[EPL / 4 - 1], sign4[EPL / 4 - 1]) : 0u);
+        else if (EPL == 4) put(it, nibbles(finish(m4[0], sign4[0])), 0u);
+        else put(it, nibbles(finish(m4[0], sign4[0])) | (nibbles(finish(m4[EPL / 4 - 1], sign4[EPL / 4 - 1])) << 16), 0u);
+    }
+    if (q == 0) *reinterpret_cast<uint2 *>(tile + face * 16 + i0) = make_uint2(exps[0], exps[1]);
+
+    if (__ballot(odd) != 0) {                                    // the integer recipe, as in pack_kernel
+#pragma unroll
+        for (int it = 0; it < ITS; ++it) {
+            uint32_t bits[EPL];
+            expand<ELEM>(raw[it], bits);
+            const uint32_t shared = (exps[it >> 2] >> (8 * (it & 3))) & 0xffu;
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                uint32_t code = to_code<W>(bits[e], shared);
+                if (shared < (uint32_t)W && (code & ((1u << W) - 1u)) == (1u << ((W - 1 - shared) & 31u))) code = 0;
+                const int sh = (W + 1) * e;
+                if (sh < 32) lo |= code << sh; else hi |= code << (sh - 32);
+            }
+            put(it, lo, hi);
+        }
+    }
+    __syncthreads();
+    constexpr uint32_t n16 = TPB * (F::tile_bytes / 16);
+    uint4 *out = reinterpret_cast<uint4 *>(dst + tile0 * F::tile_bytes);
+    const uint4 *in = reinterpret_cast<const uint4 *>(stage);
+#pragma unroll
+    for (uint32_t k = threadIdx.x; k < n16; k += 256) out[k] = in[k];
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // unpack: the inverse walk.  ELEM is the destination element size (4 = fp32, 2 = bf16).
 // ---------------------------------------------------------------------------------------------------------
 template <int W, int ELEM, int MODE, bool ALIGNED, int SHRINK = 0>
@@ -613,6 +727,19 @@ int codec_pack_tensor(int fmt, const void *src, int elem, uint32_t batch, uint32
     if (int rc = tensor_shape(s, batch, h, w, row_stride, batch_stride, elem, blocks, &shrink)) return rc;
     const size_t per16 = 16 / elem;
     const bool al = aligned16(src) && w % per16 == 0 && row_stride % per16 == 0 && batch_stride % per16 == 0;
+    // every block whole: the straight-line kernel (the bounds of every load and store are those of the tensor itself)
+    const bool whole = al && shrink == 0 && h % 32 == 0 && w % (32 * (32 / elem)) == 0;
+    if (whole) {
+        const dim3 grid((uint32_t)blocks), wg(256);
+        if (fmt == TTMI_BFLOAT8_B) {
+            if (elem == 4) hipLaunchKernelGGL((pack_whole_kernel<7, 4>), grid, wg, 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+            else hipLaunchKernelGGL((pack_whole_kernel<7, 2>), grid, wg, 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+        } else {
+            if (elem == 4) hipLaunchKernelGGL((pack_whole_kernel<3, 4>), grid, wg, 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+            else hipLaunchKernelGGL((pack_whole_kernel<3, 2>), grid, wg, 0, st, (const uint8_t *)src, (uint8_t *)dst, s);
+        }
+        return check_launch("pack_whole_kernel");
+    }
     if (fmt == TTMI_BFLOAT8_B) {
         if (elem == 4) launch_pack_tensor<7, 4>(shrink, al, src, dst, s, (uint32_t)blocks, st);
         else launch_pack_tensor<7, 2>(shrink, al, src, dst, s, (uint32_t)blocks, st);
