@@ -294,3 +294,33 @@ def test_known_answers_follow_from_the_reference_text():
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     assert mod.strip_docs(mod.as_file(mod.derive())) == mod.strip_docs(KNOWN)
+
+
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_float_route_of_the_pack_kernels_equals_the_element_converter(oracle, fmt):
+    """The GPU packers compute the code of an element of an ordinary row (32 <= E < 255, elements normal or zero) as
+    min(trunc(fma(|x|, 2^(126+W-E), 1/2 - 2^-25)), 2^W - 1).  The fma is one rounding (to nearest even) of the exact sum,
+    which float64 holds exactly for the gaps tested here.  Mantissas on, next to and between every rounding boundary, all-ones
+    mantissas and random ones, at every exponent gap; with 1/2 itself in place of 1/2 - 2^-25 one mantissa per format fails."""
+    w = W[fmt]
+    conv = oracle.lib().oracle_convert_u32_to_bfp
+    rng = np.random.default_rng(11)
+    c = float(np.float32(0.5) - np.float32(2.0 ** -25))
+    failures_with_half = 0
+    for gap in range(0, 26):
+        own = 100
+        shared = own + gap
+        step = 1 << min(23, 23 - w + gap)                       # mantissa units per code step at this gap
+        near = []
+        for k in range(0, (1 << 24) // step + 1):
+            base = k * step + step // 2                          # a tie, in units of the 24-bit mantissa
+            near += [base - 2, base - 1, base, base + 1, base + 2]
+        m24 = np.array(sorted({m for m in near if (1 << 23) <= m < (1 << 24)} | {(1 << 24) - 1, (1 << 24) - 2, 1 << 23}), dtype=np.int64)
+        m24 = np.concatenate([m24, rng.integers(1 << 23, 1 << 24, size=2000)])
+        v = m24.astype(np.float64) * 2.0 ** (w - 24 - gap)      # |x| * 2^(126+W-E), exact
+        got = np.minimum(np.trunc((v + c).astype(np.float32)), (1 << w) - 1).astype(np.int64)
+        half = np.minimum(np.trunc((v + 0.5).astype(np.float32)), (1 << w) - 1).astype(np.int64)
+        want = np.array([conv(int((own << 23) | (m & 0x7FFFFF)), shared, fmt) for m in m24.tolist()], dtype=np.int64)
+        assert np.array_equal(got, want), (gap, m24[got != want][:4])
+        failures_with_half += int((half != want).sum())
+    assert failures_with_half == 1

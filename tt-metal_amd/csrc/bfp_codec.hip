@@ -93,6 +93,42 @@ template <int ELEM> __device__ __forceinline__ void expand(const uint4 raw, uint
     }
 }
 
+// Codes of a lane's 16 source bytes in an ordinary face row (shared exponent 32 <= E < 255, every element a normal float or
+// zero; or a row of nothing but zeros), lowest element in the lowest bits of lo (bfp8 from bf16: elements 4..7 in hi).
+// The packers' recipe (shift the 24-bit mantissa down by the exponent gap, add half, shift again) is
+//     floor(v + 1/2),  v = |x| * 2^(126+W-E)  (an exact product)   ==   trunc(fma(|x|, 2^(126+W-E), 1/2 - 2^-25))
+// for every 24-bit mantissa and every exponent gap: the fma rounds the exact sum once, to nearest even, which never crosses
+// an integer (with 1/2 itself the single case v = 1/2 - 2^-25 would round up to 1).  v + 1/2 < 2^W + 1/2, so a code exceeds
+// 2^W - 1 only by being 2^W.  Saturation, the sign (bit 7 of the element's top byte) and "no sign on a zero mantissa" are
+// applied to four codes, one per byte, at a time.
+template <int W, int ELEM> __device__ __forceinline__ void ordinary_codes(const uint4 raw, uint32_t shared, uint32_t &lo, uint32_t &hi) {
+    constexpr int EPL = 16 / ELEM;
+    constexpr uint32_t ONES = 0x01010101u, TOP = ONES << W, LOW = TOP - ONES;       // per byte: 2^W, 2^W - 1
+    uint32_t bits[EPL];
+    expand<ELEM>(raw, bits);
+    const float scale = shared < 32u ? 0.f : __uint_as_float((253u + (uint32_t)W - shared) << 23);
+    uint32_t c4[EPL / 4];
+#pragma unroll
+    for (int g = 0; g < EPL / 4; ++g) {
+        uint32_t m4 = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            m4 |= (uint32_t)__builtin_fmaf(fabsf(__uint_as_float(bits[4 * g + e])), scale, 0.5f - 0x1p-25f) << (8 * e);
+        uint32_t sign4;
+        if (ELEM == 4) sign4 = __builtin_amdgcn_perm(raw.y, raw.x, 0x0c0c0703u) | __builtin_amdgcn_perm(raw.w, raw.z, 0x07030c0cu);
+        else sign4 = g == 0 ? __builtin_amdgcn_perm(raw.y, raw.x, 0x07050301u) : __builtin_amdgcn_perm(raw.w, raw.z, 0x07050301u);
+        m4 -= (m4 & TOP) >> W;                                   // 2^W -> 2^W - 1
+        const uint32_t nonzero = m4 + LOW;                       // bit W of a byte set iff its code is not zero
+        c4[g] = (((W == 7 ? sign4 : sign4 >> 4) & nonzero) & TOP) | m4;
+        if (W == 3) {                                            // the low nibbles of the four bytes -> 16 bits
+            const uint32_t pairs = c4[g] | (c4[g] >> 4);         // bytes 0 and 2 hold a pair each
+            c4[g] = __builtin_amdgcn_perm(0u, pairs, 0x0c0c0200u);
+        }
+    }
+    if (W == 7) { lo = c4[0]; hi = c4[EPL / 4 - 1]; }
+    else { lo = EPL == 4 ? c4[0] : (c4[0] | (c4[EPL / 4 - 1] << 16)); hi = 0u; }
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // pack: MODE selects how the source is addressed; ALIGNED means every lane may use one 16-byte load.
 // ---------------------------------------------------------------------------------------------------------
@@ -155,12 +191,10 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
 
     // Shared exponents of the wavefront's eight face-row pieces first, and with them one question for the whole wavefront:
     // is every row ordinary?  A row is ordinary if its exponent is 32 <= E < 255 (all elements normal floats or zero; no
-    // Inf or NaN), or if it holds nothing but zeros.  For such rows the packer's integer recipe (shift the 24-bit mantissa
-    // down by the exponent gap, add half, shift again) equals floor(|x| * 2^(126+W-E) + 1/2), and |x| * 2^(127+W-E) is an
-    // exact float product: scale, truncate to an integer, add one, halve.  Everything else (non-zero values below 2^-95,
-    // where the reference ORs a hidden one into subnormals and from_torch's double pass zeroes single-bit codes; Inf; NaN)
-    // sends the wavefront through the integer recipe.  One ballot per wavefront: per-item ballots and the branches behind
-    // them cost 2 to 4 us of 18 for a 4096 x 4096 tensor.
+    // Inf or NaN), or if it holds nothing but zeros: ordinary_codes then gives the packers' codes by float arithmetic.
+    // Everything else (non-zero values below 2^-95, where the reference ORs a hidden one into subnormals and from_torch's
+    // double pass zeroes single-bit codes; Inf; NaN) sends the wavefront through the integer recipe.  One ballot per
+    // wavefront: per-item ballots and the branches behind them cost 2 to 4 us of 18 for a 4096 x 4096 tensor.
     uint32_t shared_of[ITS];
     bool odd = false;
 #pragma unroll
@@ -190,20 +224,9 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
 #pragma unroll
         for (int it = 0; it < ITS; ++it) {
             const I at(MODE, wave, it, lane);
-            uint32_t bits[EPL];
-            expand<ELEM>(raw[it], bits);
-            const uint32_t shared = shared_of[it];
-            const float scale2 = shared < 32u ? 0.f : __uint_as_float((254u + (uint32_t)W - shared) << 23);
-            uint32_t lo = 0, hi = 0;
-#pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                const uint32_t twice = (uint32_t)(fabsf(__uint_as_float(bits[e])) * scale2);     // exact product, truncated
-                const uint32_t m = min((twice + 1u) >> 1, (1u << W) - 1u);
-                const uint32_t code = m ? (((bits[e] >> 31) << W) | m) : 0u;
-                const int sh = (W + 1) * e;
-                if (sh < 32) lo |= code << sh; else hi |= code << (sh - 32);
-            }
-            put(at, shared, lo, hi);
+            uint32_t lo, hi;
+            ordinary_codes<W, ELEM>(raw[it], shared_of[it], lo, hi);
+            put(at, shared_of[it], lo, hi);
         }
     } else {
 #pragma unroll
@@ -238,13 +261,9 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint8_t *__restrict__ s
 // pack of a row-major tensor whose blocks are all whole (h a multiple of 32, w a multiple of the block width, every lane
 // may use one 16-byte load): the same walk as pack_kernel<.., SRC_TENSOR, true, 0> in straight-line code.  Wavefront `wave`
 // reads rows 8 wave .. 8 wave + 7 of the block, one row (1 KiB) per load; lane = (tile, face column, quarter or half of the
-// face row), the same for all eight rows, so everything but the row is fixed per lane and the LDS addresses of the eight
-// items differ by constants.  Codes of ordinary rows (see pack_kernel) come from float arithmetic:
-//     floor(v + 1/2),  v = |x| * 2^(126+W-E)  (an exact product)   ==   trunc(fma(|x|, 2^(126+W-E), 1/2 - 2^-25))
-// for every 24-bit mantissa and every exponent gap (the fma rounds the exact sum once, to nearest even; with 1/2 itself the
-// single case v = 1/2 - 2^-25 would round up to 1), v + 1/2 < 2^W + 1/2, so a code exceeds 2^W - 1 only by being 2^W.
-// Signs, saturation and "no sign on a zero mantissa" are applied to the four codes of a dword at once.  Wavefronts with a row
-// that is not ordinary redo their eight items with the integer recipe.
+// face row), the same for all eight rows, so everything but the row is fixed per lane, the LDS addresses of the eight
+// items differ by constants and the eight exponent bytes of a lane are one 8-byte store.  An item is processed as soon as
+// its load has landed; a wavefront with a row that is not ordinary redoes its eight items with the integer recipe.
 // ---------------------------------------------------------------------------------------------------------
 template <int W, int ELEM>
 __global__ __launch_bounds__(256) void pack_whole_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
@@ -253,7 +272,6 @@ __global__ __launch_bounds__(256) void pack_whole_kernel(const uint8_t *__restri
     using I = Item<ELEM, 0>;
     constexpr int TPB = I::TPB, EPL = I::EPL, LPR = I::LPR, ITS = 8;
     constexpr int lane_bytes = EPL * (W + 1) / 8;               // 4, 8 (bfp8) or 2, 4 (bfp4)
-    constexpr uint32_t ONES = 0x01010101u, TOP = ONES << W, LOW = TOP - ONES;      // per byte: 2^W, 2^W - 1
     __shared__ __attribute__((aligned(16))) uint8_t stage[TPB * F::tile_bytes];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -279,19 +297,6 @@ __global__ __launch_bounds__(256) void pack_whole_kernel(const uint8_t *__restri
         else if (lane_bytes == 4) *reinterpret_cast<uint32_t *>(row) = lo;
         else *reinterpret_cast<uint2 *>(row) = make_uint2(lo, hi);
     };
-    // four codes, one per byte (m <= 2^W each), with the sign bytes of their elements (sign in bit 7): saturate, put the
-    // sign on every code whose mantissa is not zero
-    auto finish = [&](uint32_t m4, uint32_t sign4) __attribute__((always_inline)) -> uint32_t {
-        m4 -= (m4 & TOP) >> W;                                   // 2^W -> 2^W - 1
-        const uint32_t nonzero = m4 + LOW;                       // bit W of a byte set iff its code is not zero
-        return (((W == 7 ? sign4 : sign4 >> 4) & nonzero) & TOP) | m4;
-    };
-    // bfp4: the low nibbles of four bytes -> 16 bits
-    auto nibbles = [&](uint32_t c4) __attribute__((always_inline)) -> uint32_t {
-        const uint32_t pairs = c4 | (c4 >> 4);                   // bytes 0 and 2 hold a pair each
-        return __builtin_amdgcn_perm(0u, pairs, 0x0c0c0200u);
-    };
-
     uint32_t exps[2] = {0u, 0u};
     bool odd = false;
 #pragma unroll
@@ -305,21 +310,9 @@ __global__ __launch_bounds__(256) void pack_whole_kernel(const uint8_t *__restri
         const uint32_t shared = top >> 24;
         odd |= (shared < 32u && top != 0u) || shared == 255u;
         exps[it >> 2] |= shared << (8 * (it & 3));
-        const float scale = shared < 32u ? 0.f : __uint_as_float((253u + (uint32_t)W - shared) << 23);
-        uint32_t m4[EPL / 4], sign4[EPL / 4];
-#pragma unroll
-        for (int g = 0; g < EPL / 4; ++g) {
-            uint32_t m = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                m |= (uint32_t)__builtin_fmaf(fabsf(__uint_as_float(bits[4 * g + e])), scale, 0.5f - 0x1p-25f) << (8 * e);
-            m4[g] = m;
-            if (ELEM == 4) sign4[g] = __builtin_amdgcn_perm(raw[it].y, raw[it].x, 0x0c0c0703u) | __builtin_amdgcn_perm(raw[it].w, raw[it].z, 0x07030c0cu);
-            else sign4[g] = g == 0 ? __builtin_amdgcn_perm(raw[it].y, raw[it].x, 0x07050301u) : __builtin_amdgcn_perm(raw[it].w, raw[it].z, 0x07050301u);
-        }
-        if (W == 7) put(it, finish(m4[0], sign4[0]), EPL == 8 ? finish(m4[EPL / 4 - 1], sign4[EPL / 4 - 1]) : 0u);
-        else if (EPL == 4) put(it, nibbles(finish(m4[0], sign4[0])), 0u);
-        else put(it, nibbles(finish(m4[0], sign4[0])) | (nibbles(finish(m4[EPL / 4 - 1], sign4[EPL / 4 - 1])) << 16), 0u);
+        uint32_t lo, hi;
+        ordinary_codes<W, ELEM>(raw[it], shared, lo, hi);
+        put(it, lo, hi);
     }
     if (q == 0) *reinterpret_cast<uint2 *>(tile + face * 16 + i0) = make_uint2(exps[0], exps[1]);
 
