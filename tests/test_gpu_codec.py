@@ -185,6 +185,30 @@ def test_unpack_foreign_codes_every_code_and_exponent(oracle, fmt):
     assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("fmt", [BFP8, BFP4])
+def test_whole_block_unpack_kernel(oracle, fmt):
+    """Tensors of at least 512 whole blocks take the straight-line unpack kernel.  (a) Words the packers write for the
+    special patterns: most wavefronts hold a row the integer route exists for (E < W with mantissa bits, E >= 248).
+    (b) Tiles of random bytes with exponents W + 8 <= E < 248: every wavefront on the float route, with codes no packer
+    writes (rows that are not normalised; sign-only codes, which come out as +0 in the to_torch sequence).  fp32 and bf16
+    destinations against the oracle's to_torch sequence."""
+    shapes = {torch.float32: (2, 1, 1024, 2048), torch.bfloat16: (1, 1, 4096, 2048)}
+    w = 7 if fmt == BFP8 else 3
+    rng = np.random.default_rng(81)
+    for dtype, shape in shapes.items():
+        n_tiles = int(np.prod(shape)) // 1024
+        tiles = rng.integers(0, 256, size=(n_tiles, capi.TILE_BYTES[fmt]), dtype=np.uint8)
+        tiles[:, :64] = rng.integers(w + 8, 248, size=(n_tiles, 64), dtype=np.uint8)
+        for words in (oracle.from_torch_bfp_tiles(fmt, special_values(shape, seed=82)), tiles.reshape(-1).view(np.uint32)):
+            want = oracle.to_torch_bfp_tiles(fmt, words, shape)
+            got = capi.unpack_tensor(fmt, dev(words.view(np.int32)), shape, dtype=dtype)
+            if dtype == torch.float32:
+                assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+            else:
+                assert not (want.view(np.uint32) & 0xFFFF).any()
+                assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), (want.view(np.uint32) >> 16).astype(np.uint16))
+
+
 def test_known_answers_on_gpu():
     for case in KNOWN["edge_single_value_rows"]["cases"]:
         row = np.zeros(1024, dtype=np.uint32)

@@ -443,6 +443,91 @@ __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// unpack into a row-major tensor whose blocks are all whole: the walk of pack_whole_kernel backwards, in straight-line code.
+// A lane's eight face rows (rows 8 wave .. 8 wave + 7 of the block, same tile, face column and piece of the row) have their
+// exponents in eight consecutive bytes and their codes a constant number of bytes apart.  The decision "is every row of the
+// wavefront ordinary" (see unpack_kernel) is taken once, from the eight exponents and code words; ordinary rows are
+//     fma(mantissa, +-2^(E - 126 - W), +0.0)
+// (the mantissa converted from its byte or bit field, the sign moved onto the power of two; the +0.0 of the to_torch
+// sequence is the fma's addend: a sign-only code comes out as -0 + 0 = +0), other wavefronts take the integer route.
+// ---------------------------------------------------------------------------------------------------------
+template <int W, int ELEM>
+__global__ __launch_bounds__(256) void unpack_whole_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                           const CodecShape s) {
+    using F = Fmt<W>;
+    using I = Item<ELEM, 0>;
+    constexpr int TPB = I::TPB, EPL = I::EPL, LPR = I::LPR, ITS = 8;
+    constexpr int lane_bytes = EPL * (W + 1) / 8;               // 4, 8 (bfp8) or 2, 4 (bfp4)
+    __shared__ __attribute__((aligned(16))) uint8_t stage[TPB * F::tile_bytes];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t cg = blockIdx.x % s.col_groups;
+    const uint64_t rest = blockIdx.x / s.col_groups;
+    const uint32_t tr = (uint32_t)(rest % s.ht);
+    const uint64_t b = rest / s.ht;
+    const uint64_t tile0 = (b * s.ht + tr) * s.wt + (uint64_t)cg * TPB;
+    {
+        constexpr uint32_t n16 = TPB * (F::tile_bytes / 16);
+        const uint4 *in = reinterpret_cast<const uint4 *>(src + tile0 * F::tile_bytes);
+        uint4 *out = reinterpret_cast<uint4 *>(stage);
+#pragma unroll
+        for (uint32_t k = threadIdx.x; k < n16; k += 256) out[k] = in[k];
+    }
+    __syncthreads();
+
+    const int t = lane / (2 * LPR), fc = (lane / LPR) & 1, q = lane % LPR;
+    const int face = (wave >> 1) * 2 + fc, i0 = (wave & 1) * 8;
+    const uint8_t *tile = stage + t * F::tile_bytes;
+    const uint8_t *row0 = tile + 64 + face * F::face_bytes + i0 * F::row_bytes + q * lane_bytes;
+    const uint2 exps = *reinterpret_cast<const uint2 *>(tile + face * 16 + i0);
+    uint32_t lo[ITS], hi[ITS];
+    bool odd = false;
+    constexpr uint32_t all_mantissas = W == 7 ? 0x7f7f7f7fu : 0x77777777u;
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) {
+        const uint8_t *row = row0 + it * F::row_bytes;
+        hi[it] = 0;
+        if (lane_bytes == 2) lo[it] = *reinterpret_cast<const uint16_t *>(row);
+        else if (lane_bytes == 4) lo[it] = *reinterpret_cast<const uint32_t *>(row);
+        else { const uint2 v = *reinterpret_cast<const uint2 *>(row); lo[it] = v.x; hi[it] = v.y; }
+        const uint32_t shared = ((it < 4 ? exps.x : exps.y) >> (8 * (it & 3))) & 0xffu;
+        odd |= (shared < (uint32_t)W && ((lo[it] | hi[it]) & all_mantissas) != 0) || shared >= 248u;
+    }
+    const bool odd_rows = __ballot(odd) != 0;
+    uint8_t *p = dst + (b * s.batch_stride + (uint64_t)(tr * 32 + wave * 8) * s.row_stride + (uint64_t)cg * TPB * 32) * ELEM + lane * 16;
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) {
+        const uint32_t shared = ((it < 4 ? exps.x : exps.y) >> (8 * (it & 3))) & 0xffu;
+        uint32_t bits[EPL];
+        if (!odd_rows) {
+            const uint32_t two_to = shared < (uint32_t)W ? 0u : (shared - (uint32_t)W + 1u) << 23;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const int sh = (W + 1) * e;
+                const uint32_t word = sh < 32 ? lo[it] : hi[it];
+                const int at = sh & 31;                                               // the code's lowest bit in its word
+                const float mantissa = (float)((word >> at) & ((1u << W) - 1u));
+                const uint32_t sign = at + W == 31 ? word : word << (31 - W - at);    // the sign bit moved to bit 31
+                bits[e] = __float_as_uint(__builtin_fmaf(mantissa, __uint_as_float((sign & 0x80000000u) | two_to), 0.0f));
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const int sh = (W + 1) * e;
+                const uint32_t field = sh < 32 ? (lo[it] >> sh) : (hi[it] >> (sh - 32));
+                bits[e] = from_code<W>(field & ((2u << W) - 1u), shared);
+                if ((bits[e] & 0x7fffffffu) == 0) bits[e] = 0;
+            }
+        }
+        uint4 v;
+        if (ELEM == 4) v = make_uint4(bits[0], bits[1], bits[2], bits[3]);
+        else v = make_uint4((bits[0] >> 16) | (bits[1 % EPL] & 0xffff0000u), (bits[2 % EPL] >> 16) | (bits[3 % EPL] & 0xffff0000u),
+                            (bits[4 % EPL] >> 16) | (bits[5 % EPL] & 0xffff0000u), (bits[6 % EPL] >> 16) | (bits[7 % EPL] & 0xffff0000u));
+        *reinterpret_cast<uint4 *>(p + (uint64_t)it * s.row_stride * ELEM) = v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // tilize / untilize: pure permutation with zero padding (TO_TILES) or cropping.
 // ---------------------------------------------------------------------------------------------------------
 template <int ELEM, bool TO_TILES, bool ALIGNED>
@@ -753,6 +838,19 @@ int codec_unpack_tensor(int fmt, const uint32_t *words, uint32_t batch, uint32_t
     if (int rc = tensor_shape(s, batch, h, w, w, (size_t)h * w, elem, blocks, &shrink)) return rc;
     const size_t per16 = 16 / elem;
     const bool al = aligned16(dst) && w % per16 == 0;
+    // every block whole: the straight-line kernel (the bounds of every load and store are those of the tensor itself)
+    const bool whole = al && shrink == 0 && h % 32 == 0 && w % (32 * (32 / elem)) == 0;
+    if (whole) {
+        const dim3 grid((uint32_t)blocks), wg(256);
+        if (fmt == TTMI_BFLOAT8_B) {
+            if (elem == 4) hipLaunchKernelGGL((unpack_whole_kernel<7, 4>), grid, wg, 0, st, (const uint8_t *)words, (uint8_t *)dst, s);
+            else hipLaunchKernelGGL((unpack_whole_kernel<7, 2>), grid, wg, 0, st, (const uint8_t *)words, (uint8_t *)dst, s);
+        } else {
+            if (elem == 4) hipLaunchKernelGGL((unpack_whole_kernel<3, 4>), grid, wg, 0, st, (const uint8_t *)words, (uint8_t *)dst, s);
+            else hipLaunchKernelGGL((unpack_whole_kernel<3, 2>), grid, wg, 0, st, (const uint8_t *)words, (uint8_t *)dst, s);
+        }
+        return check_launch("unpack_whole_kernel");
+    }
     if (fmt == TTMI_BFLOAT8_B) {
         if (elem == 4) launch_unpack_tensor<7, 4>(shrink, al, words, dst, s, (uint32_t)blocks, st);
         else launch_unpack_tensor<7, 2>(shrink, al, words, dst, s, (uint32_t)blocks, st);
