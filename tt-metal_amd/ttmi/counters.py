@@ -64,11 +64,11 @@ def leg_kernels():
         out = (u32 * 4)()
         L.ttmi_test_stream_decomposition(batch or 1, m, k, n, 1, out)
         split, workgroups = int(out[2]), int(out[3])
-        legs[name] = [(f"matmul_wide_kernel<{7 if fmt == 'bfp8_b' else 3}, 0>", workgroups + (split if split > 1 else 0))]
+        legs[name] = [(f"matmul_wide_kernel<{7 if fmt == 'bfp8_b' else 3}, 0, 1, 1>", workgroups + (split if split > 1 else 0))]
     legs["prefill_ff1"] = [("expand_kernel<7>", None), ("matmul_expanded_kernel<0>", None)]
     legs["bert_bmm"] = [("matmul_tall_kernel<7, 0", None)]
-    legs["pack_bfp4_4k_pack"] = [("pack_kernel<3,", None)]
-    legs["pack_bfp4_4k_unpack"] = [("unpack_kernel<3,", None)]
+    legs["pack_bfp4_4k_pack"] = [("pack_whole_kernel<3,", None)]
+    legs["pack_bfp4_4k_unpack"] = [("unpack_whole_kernel<3,", None)]
     legs["pack_bfp8_1k_pack"] = [("pack_kernel<7,", None)]
     legs["pack_bfp8_1k_unpack"] = [("unpack_kernel<7,", None)]
     return legs
