@@ -112,3 +112,20 @@ def test_gated_mistral_mlp_shape_full_size(oracle):
     # the three launches round to bf16 three times (2^-9 relative each), the fused one once
     worst = float(((fused.float() - three.float()).abs() / (three.float().abs() + 1e-3)).max())
     assert worst <= 2.0 ** -6, worst
+
+
+@pytest.mark.parametrize("out_fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("m,k,n", [(32, 64, 128), (32, 2048, 256), (32, 4096, 96)])
+def test_gated_block_float_output(oracle, out_fmt, m, k, n):
+    """Output dtype BFLOAT8_B / BFLOAT4_B of the gated launch (TILE layout): the words that packing its bf16 output gives
+    (ttmi_typecast_tiles, itself pinned against the oracle's packer), stored directly and through the hand-over of partial
+    sums, with a column group that is not full."""
+    a_tiles = capi.tilize(bf16_dev(workloads.activations_bf16(m, k, seed=340)))
+    gate_words, _ = pack_weights(oracle, workloads.weights_f32(k, n, seed=341), BFP4)
+    up_words, _ = pack_weights(oracle, workloads.weights_f32(k, n, seed=342), BFP4)
+    dense = capi.matmul_bfp_gated(a_tiles, capi.TILE, gate_words, up_words, BFP4, 1, 1, m, k, n, c_layout=capi.TILE)
+    want = capi.typecast_tiles(dense, capi.BFLOAT16, out_fmt)
+    got = capi.matmul_bfp_gated(a_tiles, capi.TILE, gate_words, up_words, BFP4, 1, 1, m, k, n, c_layout=capi.TILE, out_bfp=out_fmt)
+    assert torch.equal(got, want)
+    host = oracle.pack_fp32_vec_as_bfp_tiles(out_fmt, dense.float().cpu().numpy().reshape(-1), False)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), host)

@@ -233,19 +233,22 @@ def matmul_bf16(a, a_layout: int, b_tiles, batch: int, b_batch: int, m: int, k: 
 
 
 def matmul_bfp_gated(a, a_layout: int, gate_words, up_words, b_fmt: int, batch: int, b_batch: int, m: int, k: int, n: int, *,
-                     bias=None, activation: int = ACT_SILU, c_layout: int = ROW_MAJOR, out_dtype=None, workspace=None):
+                     bias=None, activation: int = ACT_SILU, c_layout: int = ROW_MAJOR, out_dtype=None, workspace=None, out_bfp=None):
     """act(a . gate + bias) * (a . up) in one launch (ttmi_matmul_bfp_gated); arguments as for matmul_bfp."""
     import torch
 
     out_dtype = out_dtype or torch.bfloat16
     mp = padded(m) if c_layout == TILE else m
-    c = torch.empty(batch * mp * n, dtype=out_dtype, device=a.device)
+    if out_bfp is not None:
+        c = torch.empty(lib().ttmi_tiled_size_bytes(out_bfp, batch, m, n) // 4, dtype=torch.int32, device=a.device)
+    else:
+        c = torch.empty(batch * mp * n, dtype=out_dtype, device=a.device)
     ws_ptr, ws_bytes = None, 0
     if workspace is not None:
         ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
     check(lib().ttmi_matmul_bfp_gated(
         _dev(a), a_layout, _dev(gate_words), _dev(up_words), b_fmt, batch, b_batch, m, k, n,
-        _dev(bias) if bias is not None else None, activation, _dev(c), c_layout, _torch_dtype_code(c),
+        _dev(bias) if bias is not None else None, activation, _dev(c), c_layout, out_bfp if out_bfp is not None else _torch_dtype_code(c),
         ws_ptr, ws_bytes, _stream()))
     if c_layout == ROW_MAJOR:
         return c.view(batch, m, n)
