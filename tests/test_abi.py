@@ -109,6 +109,35 @@ SHAPES = [(1, 32, 4544, 18176), (1, 32, 18176, 4544), (1, 32, 4096, 6144), (1, 3
           (1, 32, 4096, 14336), (3, 24, 768, 160), (2, 40, 1024, 288), (1, 8, 32, 32), (1, 32, 64, 4096), (5, 100, 96, 2080)]
 
 
+def test_kernel_choice_by_shape():
+    """Which kernel a GEMM goes to: one band streams in 128-column units, unless its 64-column groups are one workgroup per CU
+    (200 to 256 of them) with at most 256 KiB of weights each and the output is not block-float — then the 64-column kernel
+    takes it with one workgroup per group and nothing shared; two and four bands in the two-band form, three in 64-column
+    units; 128 to 511 rows tiled, from 512 rows expanded."""
+    from ttmi import capi
+
+    L = _test_entries()
+    u32 = ctypes.c_uint32
+    L.ttmi_test_kernel_choice.restype = ctypes.c_int
+    L.ttmi_test_kernel_choice.argtypes = [u32, u32, u32, u32, ctypes.c_int, ctypes.c_int]
+    STREAM, WIDE, TILE, EXPANDED = 1, 2, 3, 4
+    B8, B4, BF16 = capi.BFLOAT8_B, capi.BFLOAT4_B, capi.BFLOAT16
+    cases = [((1, 32, 4544, 18176, B8, BF16), WIDE), ((1, 32, 18176, 4544, B8, BF16), WIDE), ((1, 32, 4096, 4096, B8, BF16), WIDE),
+             ((1, 32, 4096, 14336, B4, BF16), STREAM), ((1, 32, 4096, 14336, B4, B8), WIDE), ((1, 32, 4096, 14336, B8, BF16), WIDE),
+             ((1, 32, 4096, 16384, B4, BF16), STREAM), ((1, 32, 4096, 16448, B4, BF16), WIDE), ((1, 32, 4096, 12736, B4, BF16), WIDE),
+             ((1, 32, 14336, 4096, B4, BF16), WIDE), ((2, 20, 1024, 7168, B8, BF16), STREAM), ((1, 64, 4096, 14336, B4, BF16), WIDE),
+             ((1, 96, 4096, 4096, B8, BF16), STREAM), ((1, 128, 4096, 4096, B8, BF16), TILE), ((1, 2048, 4096, 14336, B8, BF16), EXPANDED)]
+    for args, want in cases:
+        assert L.ttmi_test_kernel_choice(*args) == want, args
+    # the one-round form: one workgroup per group, no partial sums, no workspace
+    out = (u32 * 4)()
+    L.ttmi_test_stream_decomposition(1, 32, 4096, 14336, 0, out)
+    assert [int(x) for x in out] == [224, 128, 1, 224]
+    # the workspace query covers the 128-column kernel, which the same shape takes with a block-float output
+    L.ttmi_test_stream_decomposition(1, 32, 4096, 14336, 1, out)
+    assert L.ttmi_matmul_bfp_workspace_bytes(1, 32, 4096, 14336, B4) == int(out[3]) * 16384
+
+
 @pytest.mark.parametrize("wide", [0, 1])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_every_unit_has_exactly_one_workgroup_and_collectors_come_last(shape, wide):

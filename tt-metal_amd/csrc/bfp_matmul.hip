@@ -21,6 +21,7 @@
 //              many as fill the chip.  Outputs whose k range is shared between workgroups are finished by the
 //              workgroup that owns the last part (see the kernel).
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <stdint.h>
 #include <mutex>
 #include <type_traits>
@@ -858,6 +859,10 @@ struct Decomposition { uint32_t mt, mt_sets, kt, nt, ngroups, workgroups, split;
 // two_bands: the 128-column kernel takes two 32-row bands per workgroup (33 to 127 rows, not gated)
 static bool two_bands(uint32_t m, bool wide, bool gated) { return wide && !gated && m > 32; }
 
+// 64-column kernel: between 200 and 256 output groups are one workgroup per CU, each with its whole k range: nothing is
+// handed over (with fewer groups too many CUs idle, with more a second round begins).
+static bool one_round_of_groups(uint64_t groups) { return groups >= 200 && groups <= 256; }
+
 static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, bool wide, bool gated = false) {
     Decomposition d{};
     const uint32_t group_tiles = wide ? WIDE_TILES : GROUP_TILES;
@@ -876,6 +881,8 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     const bool few = d.groups < 100 || gated;
     const uint64_t resident = knob_or(TTMI_KNOB_MATMUL_WORKGROUPS, wide ? (few ? 256 : 256 * WIDE_WGS_PER_CU) : d.groups >= 256 ? 768 : 512);
     uint64_t parts = d.groups >= resident ? 1 : wide && !few ? resident / (d.groups + 1) : resident / d.groups;
+    uint32_t asked;
+    if (!wide && one_round_of_groups(d.groups) && !knob(TTMI_KNOB_MATMUL_WORKGROUPS, &asked)) parts = 1;
     if (parts == 0) parts = 1;
     const uint64_t most = d.kt / (2 * WAVES) ? d.kt / (2 * WAVES) : 1;
     if (parts > most) parts = most;
@@ -969,11 +976,20 @@ int matmul_bfp_wide(const MatmulArgs &x, hipStream_t st) { return launch_streami
 // on (two or more 256-row blocks share every weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
 // The test entry point can force a kernel (TTMI_KNOB_MATMUL_KERNEL).
 enum class Kernel { Stream = 1, Wide = 2, Tile = 3, Expanded = 4 };
-static Kernel choose_kernel(uint32_t m) {
+static Kernel choose_kernel(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt, bool c_bfp) {
     uint32_t forced;
     if (knob(TTMI_KNOB_MATMUL_KERNEL, &forced) && forced >= 1 && forced <= 4) return (Kernel)forced;
     if (m >= 512) return Kernel::Expanded;
     if (m >= 128) return Kernel::Tile;
+    // One band whose 64-column groups are one workgroup per CU, with at most 256 KiB of weights each: the 64-column kernel,
+    // which then shares no output and has nothing to hand over.  Measured against the 128-column kernel, same box, M = 32:
+    // [4096, 14336] BFP4_B (Mistral's gate / up, 147 KB per group) 14.8 against 16.1 us, [4096, 16384] BFP4_B 14.5 against
+    // 18.6, [2048, 15360] BFP4_B 9.2 against 10.8, [4096, 12800] BFP8_B (278 KB) 17.8 either way, [8192, 14336] BFP8_B
+    // (557 KB) 30.2 against 28.5: the longer the k range, the less the hand-over matters and the more the 64-column
+    // kernel's extra instruction work per byte.  It writes no block-float output.
+    const uint64_t group_weights = (uint64_t)(k / 32) * GROUP_TILES * (b_fmt == TTMI_BFLOAT4_B ? 576u : 1088u);
+    if (m <= 32 && !c_bfp && group_weights <= 256u * 1024u && one_round_of_groups((uint64_t)batch * ((n / 32 + GROUP_TILES - 1) / GROUP_TILES)))
+        return Kernel::Stream;
     return m <= 32 || ((m + 31) / 32) % 2 == 0 ? Kernel::Wide : Kernel::Stream;
 }
 
@@ -982,24 +998,27 @@ size_t matmul_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint
     return slot_bytes_needed(decompose(batch, m, k, n, true, true), true, true);
 }
 
-size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int) {
+size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt) {
     if (!batch || !m || !k || !n) return 0;
-    const Kernel kernel = choose_kernel(m);
+    const Kernel kernel = choose_kernel(batch, m, k, n, b_fmt, false);
     switch (kernel) {
         case Kernel::Expanded: return matmul_expanded_workspace_bytes(batch, k, n);   // as if every slice had weights of its own
         case Kernel::Tile: return 0;
         default: break;
     }
     const bool wide = kernel == Kernel::Wide;
-    return slot_bytes_needed(decompose(batch, m, k, n, wide), wide, two_bands(m, wide, false));
+    const size_t need = slot_bytes_needed(decompose(batch, m, k, n, wide), wide, two_bands(m, wide, false));
+    // one band in the 64-column kernel: with a block-float output the same shape goes to the 128-column kernel
+    if (!wide && m <= 32) return std::max(need, slot_bytes_needed(decompose(batch, m, k, n, true), true, false));
+    return need;
 }
 
 int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
     // what an earlier launch on this device has reported (a wait for partial sums that gave up) surfaces here
     if (!x.no_alloc || error_word_if_exists(nullptr, nullptr))
         if (int rc = ttmi_device_status()) return rc;
-    const Kernel kernel = choose_kernel(x.m);
     const bool c_bfp = x.c_dtype == TTMI_BFLOAT8_B || x.c_dtype == TTMI_BFLOAT4_B;
+    const Kernel kernel = choose_kernel(x.batch, x.m, x.k, x.n, x.b_fmt, c_bfp);
     if (c_bfp && kernel != Kernel::Wide) {
         // Only the 128-column kernel packs in its epilogue.  The others write bf16 tiles into a buffer of the library (one
         // per stream) and one typecast pass packs them: the same bits, one more launch.
@@ -1108,6 +1127,10 @@ __attribute__((visibility("default"))) void ttmi_test_stream_decomposition(uint3
                                                                            uint32_t out[4]) {
     const ttmi::Decomposition d = ttmi::decompose(batch, m, k, n, wide != 0);
     out[0] = (uint32_t)d.groups; out[1] = d.kt; out[2] = d.split; out[3] = d.workgroups;
+}
+// which kernel a shape goes to: 1 = 64-column streaming kernel, 2 = 128-column streaming kernel, 3 = tiled, 4 = expanded
+__attribute__((visibility("default"))) int ttmi_test_kernel_choice(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt, int c_dtype) {
+    return (int)ttmi::choose_kernel(batch, m, k, n, b_fmt, c_dtype == TTMI_BFLOAT8_B || c_dtype == TTMI_BFLOAT4_B);
 }
 __attribute__((visibility("default"))) void ttmi_test_wide_layout(int mantissa_bits, int lane, uint32_t out[16]) {
     if (mantissa_bits == 7) wide_layout_of<7>(lane, out); else wide_layout_of<3>(lane, out);

@@ -60,11 +60,18 @@ def leg_kernels():
     L.ttmi_test_stream_decomposition.restype = None
     L.ttmi_test_stream_decomposition.argtypes = [u32, u32, u32, u32, ctypes.c_int, ctypes.POINTER(u32)]
     legs = {}
+    L.ttmi_test_kernel_choice.restype = ctypes.c_int
+    L.ttmi_test_kernel_choice.argtypes = [u32, u32, u32, u32, ctypes.c_int, ctypes.c_int]
     for name, m, k, n, fmt, batch in workloads.DECODE_FALCON + workloads.DECODE_MISTRAL:
         out = (u32 * 4)()
-        L.ttmi_test_stream_decomposition(batch or 1, m, k, n, 1, out)
+        wide = L.ttmi_test_kernel_choice(batch or 1, m, k, n, capi.BFLOAT8_B if fmt == "bfp8_b" else capi.BFLOAT4_B, capi.BFLOAT16) == 2
+        L.ttmi_test_stream_decomposition(batch or 1, m, k, n, int(wide), out)
         split, workgroups = int(out[2]), int(out[3])
-        legs[name] = [(f"matmul_wide_kernel<{7 if fmt == 'bfp8_b' else 3}, 0, 1, 1>", workgroups + (split if split > 1 else 0))]
+        w = 7 if fmt == "bfp8_b" else 3
+        if wide:
+            legs[name] = [(f"matmul_wide_kernel<{w}, 0, 1, 1>", workgroups + (split if split > 1 else 0))]
+        else:
+            legs[name] = [(f"matmul_stream_kernel<{w}, 0>", workgroups)]
     legs["prefill_ff1"] = [("expand_kernel<7>", None), ("matmul_expanded_kernel<0>", None)]
     legs["bert_bmm"] = [("matmul_tall_kernel<7, 0", None)]
     legs["pack_bfp4_4k_pack"] = [("pack_whole_kernel<3,", None)]
