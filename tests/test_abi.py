@@ -111,7 +111,7 @@ SHAPES = [(1, 32, 4544, 18176), (1, 32, 18176, 4544), (1, 32, 4096, 6144), (1, 3
 
 def test_kernel_choice_by_shape():
     """Which kernel a GEMM goes to: one band streams in 128-column units, unless its 64-column groups are one workgroup per CU
-    (200 to 256 of them) with at most 256 KiB of weights each and the output is not block-float — then the 64-column kernel
+    (200 to 256 of them) of at most 192 KiB of BFP4_B weights each and the output is not block-float — then the 64-column kernel
     takes it with one workgroup per group and nothing shared; two and four bands in the two-band form, three in 64-column
     units; 128 to 511 rows tiled, from 512 rows expanded."""
     from ttmi import capi
@@ -125,7 +125,7 @@ def test_kernel_choice_by_shape():
     cases = [((1, 32, 4544, 18176, B8, BF16), WIDE), ((1, 32, 18176, 4544, B8, BF16), WIDE), ((1, 32, 4096, 4096, B8, BF16), WIDE),
              ((1, 32, 4096, 14336, B4, BF16), STREAM), ((1, 32, 4096, 14336, B4, B8), WIDE), ((1, 32, 4096, 14336, B8, BF16), WIDE),
              ((1, 32, 4096, 16384, B4, BF16), STREAM), ((1, 32, 4096, 16448, B4, BF16), WIDE), ((1, 32, 4096, 12736, B4, BF16), WIDE),
-             ((1, 32, 14336, 4096, B4, BF16), WIDE), ((2, 20, 1024, 7168, B8, BF16), STREAM), ((1, 64, 4096, 14336, B4, BF16), WIDE),
+             ((1, 32, 14336, 4096, B4, BF16), WIDE), ((2, 20, 1024, 7168, B8, BF16), WIDE), ((2, 20, 1024, 7168, B4, BF16), STREAM), ((1, 32, 8192, 14336, B4, BF16), WIDE), ((1, 64, 4096, 14336, B4, BF16), WIDE),
              ((1, 96, 4096, 4096, B8, BF16), STREAM), ((1, 128, 4096, 4096, B8, BF16), TILE), ((1, 2048, 4096, 14336, B8, BF16), EXPANDED)]
     for args, want in cases:
         assert L.ttmi_test_kernel_choice(*args) == want, args

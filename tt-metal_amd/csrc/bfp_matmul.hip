@@ -981,14 +981,17 @@ static Kernel choose_kernel(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, 
     if (knob(TTMI_KNOB_MATMUL_KERNEL, &forced) && forced >= 1 && forced <= 4) return (Kernel)forced;
     if (m >= 512) return Kernel::Expanded;
     if (m >= 128) return Kernel::Tile;
-    // One band whose 64-column groups are one workgroup per CU, with at most 256 KiB of weights each: the 64-column kernel,
-    // which then shares no output and has nothing to hand over.  Measured against the 128-column kernel, same box, M = 32:
-    // [4096, 14336] BFP4_B (Mistral's gate / up, 147 KB per group) 14.8 against 16.1 us, [4096, 16384] BFP4_B 14.5 against
-    // 18.6, [2048, 15360] BFP4_B 9.2 against 10.8, [4096, 12800] BFP8_B (278 KB) 17.8 either way, [8192, 14336] BFP8_B
-    // (557 KB) 30.2 against 28.5: the longer the k range, the less the hand-over matters and the more the 64-column
-    // kernel's extra instruction work per byte.  It writes no block-float output.
-    const uint64_t group_weights = (uint64_t)(k / 32) * GROUP_TILES * (b_fmt == TTMI_BFLOAT4_B ? 576u : 1088u);
-    if (m <= 32 && !c_bfp && group_weights <= 256u * 1024u && one_round_of_groups((uint64_t)batch * ((n / 32 + GROUP_TILES - 1) / GROUP_TILES)))
+    // One band of BFP4_B weights whose 64-column groups are one workgroup per CU, with at most 192 KiB of weights each:
+    // the 64-column kernel, which then shares no output and has nothing to hand over.  Measured against the 128-column
+    // kernel, same box, M = 32, weights rotated through more than the Infinity Cache holds: [4096, 14336] BFP4_B (Mistral's
+    // gate / up, 147 KB per group) 15.0 against 15.3 us, [4096, 16384] BFP4_B 15.2 against 18.7, [2048, 15360] BFP4_B 9.7
+    // against 10.8; but [8192, 14336] BFP4_B (295 KB) 25.3 against 23.0, and BFP8_B loses at every size ([2048, 14336]
+    // 12.3 against 11.7, [4096, 12800] 18.0 against 17.7, [8192, 14336] 30.0 against 28.4): the longer the k range, the
+    // less the hand-over matters and the more the 64-column kernel's extra instruction work per byte.  It writes no
+    // block-float output.
+    const uint64_t group_weights = (uint64_t)(k / 32) * GROUP_TILES * 576u;
+    if (m <= 32 && !c_bfp && b_fmt == TTMI_BFLOAT4_B && group_weights <= 192u * 1024u &&
+        one_round_of_groups((uint64_t)batch * ((n / 32 + GROUP_TILES - 1) / GROUP_TILES)))
         return Kernel::Stream;
     return m <= 32 || ((m + 31) / 32) % 2 == 0 ? Kernel::Wide : Kernel::Stream;
 }
