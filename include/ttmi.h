@@ -150,7 +150,7 @@ TTMI_API size_t ttmi_matmul_bfp_workspace_bytes(uint32_t batch, uint32_t m, uint
  *            TTMI_BFLOAT4_B with c_layout TTMI_TILE (output_dtype of tt::operations::primary::matmul, bmm_op.hpp:318-346):
  *            packed tiles of the bf16-rounded result with the host packers' arithmetic (what ttmi_typecast_tiles gives for
  *            the bf16 output) — packed in the epilogue of the decode kernel (up to 32 rows), by one more launch otherwise
- *   workspace NULL (the library keeps a per-device buffer of its own, allocated on first use) or at least
+ *   workspace NULL (the library keeps a buffer of its own per device and stream, allocated on first use) or at least
  *            ttmi_matmul_bfp_workspace_bytes() bytes of device memory, 256-byte aligned.  Up to 127 rows it holds
  *            partial sums of workgroups that share an output (a few MB); from 512 rows on the weights expanded to
  *            bf16 (2 bytes per weight; the size query assumes every batch slice has weights of its own, a call with
