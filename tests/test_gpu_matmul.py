@@ -442,7 +442,7 @@ def assemble_tiles(fmt, exps, codes):
     return np.ascontiguousarray(out).reshape(-1).view(np.uint32)
 
 
-EDGE_KERNELS = [("wide", 32, None), ("stream", 64, None), ("tile", 256, 128), ("tile", 256, 256), ("tile", 256, 4), ("tile", 384, 384), ("expanded", 512, None)]
+EDGE_KERNELS = [("wide", 32, None), ("wide", 64, None), ("stream", 64, None), ("tile", 256, 128), ("tile", 256, 256), ("tile", 256, 4), ("tile", 384, 384), ("expanded", 512, None)]
 
 
 @pytest.mark.parametrize("kernel,m,block", EDGE_KERNELS)
@@ -452,8 +452,9 @@ def test_rows_at_the_ends_of_the_exponent_range(oracle, kernel, m, block, fmt, k
       E = 0     (fp32 subnormal sources)  the row is read with the scale of E = 1, the IEEE convention for a zero exponent
                 field; the same in every kernel
       E = 247   the largest exponent every kernel takes exactly
-      E = 254   exact in the streaming kernels (M < 128), whose operands carry no common factor; in the tiled and expanding
-                kernels the operand, mantissa x 2^(E - 127), overflows for mantissas >= 2: those columns come out non-finite
+      E = 254   exact in the streaming kernels (M < 128) where they take the weights in hidden-one form; in the tiled and
+                expanding kernels, and in the two-band form of the 128-column kernel for BFLOAT4_B (single exact operands),
+                the operand, mantissa x 2^(E - 127), overflows for mantissas >= 2: those columns come out non-finite
       E = 255   (Inf / NaN sources) the 16 columns that share the exponent are non-finite, all others are untouched
     Expected values are formed here from codes and exponents directly: sign x mantissa x 2^(max(E, 1) - 127 - (W - 1))."""
     knobs("kernel", kernel)
@@ -482,7 +483,7 @@ def test_rows_at_the_ends_of_the_exponent_range(oracle, kernel, m, block, fmt, k
     bound = 2.0 ** -22 * np.abs(ref) + 2.0 * k * 2.0 ** -24 * (np.abs(a64) @ (np.abs(w64) + np.exp2((e_eff - 127).astype(np.float64)))) + 1e-37
     poisoned = np.zeros(n, dtype=bool)
     poisoned[48:64] = True                                   # E = 255
-    if kernel in ("tile", "expanded"):
+    if kernel in ("tile", "expanded") or (kernel == "wide" and m > 32 and fmt == BFP4):
         poisoned |= (codes[77] & ((1 << w_bits) - 1)) >= 2   # E = 254: mantissa x 2^127 overflows
     assert not np.isfinite(c[:, poisoned]).any()
     ok = ~poisoned
@@ -627,20 +628,22 @@ def test_bf16_weights(batch, b_batch, m, k, n):
 
 
 @pytest.mark.parametrize("fmt", [BFP8, BFP4])
-@pytest.mark.parametrize("kernel", ["wide", "stream", "tile", "expanded"])
+@pytest.mark.parametrize("kernel", ["wide", "wide two bands", "stream", "tile", "expanded"])
 def test_face_rows_with_outliers(oracle, fmt, kernel, knobs):
     """Weights whose face rows mix magnitudes over 40 binades (the stress mixture, x 50): for the kernels that multiply by
     the expanded weights the error stays within the fp32 accumulation bound on |A| . |W|; the streaming kernels add and
     subtract the face row's power of two with every weight (hi - lo), so their accumulation error is relative to that
     power of two - at most 2^-16 of the row's own quantisation step per product - and an output next to an outlier can
     leave the |W| bound while the sum over all outputs is as accurate as before (relative rms error below 1e-6)."""
-    m, k, n = 32, 256, 384
+    m, k, n = (64 if kernel == "wide two bands" else 32), 256, 384
     w = np.ascontiguousarray(workloads.stress_mixture((1, 1, k, n), seed=3)[0, 0] * 50.0)
     words, w_ref = pack_weights(oracle, w, fmt)
     a_bits = workloads.activations_bf16(m, k, seed=4)
     a = workloads.bf16_bits_to_f32(a_bits)
-    knobs("kernel", kernel)
+    knobs("kernel", kernel.split()[0])
     c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n, out_dtype=torch.float32)[0].cpu().numpy()
-    check_against_reference(c, a, w_ref, k, bf16_out=False, face_row_scale=kernel in ("wide", "stream"))
+    # hidden-one form: the 64-column kernel, the 128-column kernel with one band, and with two bands of BFLOAT8_B weights
+    hidden = kernel in ("wide", "stream") or (kernel == "wide two bands" and fmt == BFP8)
+    check_against_reference(c, a, w_ref, k, bf16_out=False, face_row_scale=hidden)
     ref = a.astype(np.float64) @ w_ref.astype(np.float64)
     assert np.sqrt(((c - ref) ** 2).mean() / (ref ** 2).mean()) < 1e-6

@@ -221,6 +221,46 @@ __device__ __forceinline__ void wait_slabs(SlabRaw &a, SlabRaw &b) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.e01), "+v"(a.w01), "+v"(a.w23), "+v"(a.w45), "+v"(a.w67),
                                           "+v"(b.e01), "+v"(b.w01), "+v"(b.w23), "+v"(b.w45), "+v"(b.w67)::"memory");
 }
+// BFLOAT4_B: exact expansion into single operands through the scaled fp8-to-bf16 conversion.  A 3-bit mantissa 0..7 is an
+// e4m3 value (bytes 00 38 40 44 48 4A 4C 4E), and v_cvt_scalef32_pk_bf16_fp8 turns two of them into bf16 values times a power
+// of two, here 2^(max(E, 1) - 127): the operand holds mantissa x 2^(max(E, 1) - 127) = 4 x the weight (Wfmt<3>::unscale takes
+// the 4 out of the sums), exactly.  About 2.75 vector-ALU instructions per weight, and one matrix instruction per operand
+// where the hidden-one form below needs two, and the sums see nothing but products with the weights.  Edge rows as in the
+// tiled kernels: E = 0 is read as E = 1; E = 254 overflows
+// for mantissas >= 2; E = 255 makes the 16 columns that share the exponent non-finite.
+__device__ __forceinline__ void slab_expand_bfp4(const SlabRaw &r, int q, bf16x8 (&bop)[4]) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const uint32_t words[8] = {r.w01[0], r.w01[1], r.w23[0], r.w23[1], r.w45[0], r.w45[1], r.w67[0], r.w67[1]};
+    uint32_t lo[8], hi[8];         // (columns 0, 1) and (columns 2, 3) of row jj as bf16 pairs
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+        const uint32_t e = (r.e01[jj >> 2] >> (8 * (jj & 3))) & 0xffu;
+        const float scale = __uint_as_float((e > 1u ? e : 1u) << 23);
+        uint32_t v = (words[jj] >> (16 * (q & 1))) & 0xffffu;
+        v = (v | (v << 8)) & 0x00ff00ffu;
+        v = (v | (v << 4)) & 0x0f0f0f0fu;                                   // one code per byte
+        const uint32_t fp8 = ((v << 4) & 0x80808080u) | __builtin_amdgcn_perm(0x4E4C4A48u, 0x44403800u, v & 0x07070707u);
+        lo[jj] = __builtin_bit_cast(uint32_t, (bf16x2_t)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(fp8, scale, false));
+        hi[jj] = __builtin_bit_cast(uint32_t, (bf16x2_t)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(fp8, scale, true));
+    }
+    uint32_t packed[4][4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        packed[0][p] = __builtin_amdgcn_perm(lo[2 * p + 1], lo[2 * p], 0x05040100u);
+        packed[1][p] = __builtin_amdgcn_perm(lo[2 * p + 1], lo[2 * p], 0x07060302u);
+        packed[2][p] = __builtin_amdgcn_perm(hi[2 * p + 1], hi[2 * p], 0x05040100u);
+        packed[3][p] = __builtin_amdgcn_perm(hi[2 * p + 1], hi[2 * p], 0x07060302u);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bop[j] = __builtin_bit_cast(bf16x8, make_uint4(packed[j][0], packed[j][1], packed[j][2], packed[j][3]));
+}
+
+// Which form the 128-column kernel feeds the matrix cores: BFLOAT4_B weights as single exact operands where a workgroup
+// multiplies them with two 32-row bands (the conversion is shared by the bands and the matrix instructions are what such a
+// launch waits for: 22.0 against 23.6 us for [64, 4096] x [4096, 14336]); the hidden-one form below everywhere else (one
+// band: 14.5 against 15.3 us for the same weights, 14.8 against 15.5 us for [14336, 4096]).
+template <int W, int BANDS> constexpr bool single_operand() { return W == 3 && BANDS == 2; }
+
 // Expansion without arithmetic ("hidden-one form"), for kernels that are bound by vector-ALU issue rather than by the
 // matrix pipe.  A code (sign s, mantissa m of W bits) under the shared exponent E of its face row is written into a bf16 as
 //      hi[15] = s, hi[14:7] = E, hi[6:7-W] = m          value  +-(1 + m / 2^W) * 2^(E - 127)
@@ -236,6 +276,8 @@ __device__ __forceinline__ void wait_slabs(SlabRaw &a, SlabRaw &b) {
 // E = 255 (Inf / NaN sources) makes the sums of the 16 columns that share the exponent non-finite; every other exponent,
 // 254 included, is exact.
 constexpr float hidden_unscale = 2.0f;
+// what the sums of a streaming kernel are multiplied by
+template <int W, int BANDS> constexpr float decode_unscale() { return single_operand<W, BANDS>() ? Wfmt<W>::unscale : hidden_unscale; }
 
 // exponent field of k rows (2p, 2p + 1), one in each half of a word
 __device__ __forceinline__ uint32_t hidden_pair_field(const u32x2 e01, int p) {

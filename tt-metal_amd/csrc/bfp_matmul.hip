@@ -595,22 +595,36 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
             wide_slab_read<W, AT + 32, AT + F::slab_bytes>(exp_at, mant_at, raw1);
             wait_slabs(raw0, raw1);
             if (nb == NB - 1 && refill) fetch(stage_tag);
-            bf16x8 hi[4], lo[4];
-            slab_expand_hidden<W>(raw0, q, hi, lo);
+            if constexpr (single_operand<W, MB>()) {
+                bf16x8 bop[4];
+                slab_expand_bfp4(raw0, q, bop);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
+                for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb]), hi[j], acc[nb * MB + mb][j], 0, 0, 0);
+                    for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb]), bop[j], acc[nb * MB + mb][j], 0, 0, 0);
+                slab_expand_bfp4(raw1, q, bop);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[2 * mb]), lo[j], acc[nb * MB + mb][j], 0, 0, 0);
-            }
-            slab_expand_hidden<W>(raw1, q, hi, lo);
+                for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
+                    for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb + 1]), bop[j], acc[nb * MB + mb][j], 0, 0, 0);
+            } else {
+                bf16x8 hi[4], lo[4];
+                slab_expand_hidden<W>(raw0, q, hi, lo);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb + 1]), hi[j], acc[nb * MB + mb][j], 0, 0, 0);
+                for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[2 * mb + 1]), lo[j], acc[nb * MB + mb][j], 0, 0, 0);
+                    for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb]), hi[j], acc[nb * MB + mb][j], 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[2 * mb]), lo[j], acc[nb * MB + mb][j], 0, 0, 0);
+                }
+                slab_expand_hidden<W>(raw1, q, hi, lo);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb + 1]), hi[j], acc[nb * MB + mb][j], 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_neg[2 * mb + 1]), lo[j], acc[nb * MB + mb][j], 0, 0, 0);
+                }
             }
         });
     };
@@ -687,10 +701,10 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
         float v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            float x = sums[0][j] * hidden_unscale;
+            float x = sums[0][j] * decode_unscale<W, MB>();
             if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
             v[j] = apply_activation<ACT>(x);
-            if (NB == 2) v[j] *= sums[NB - 1][j] * hidden_unscale;
+            if (NB == 2) v[j] *= sums[NB - 1][j] * decode_unscale<W, MB>();
         }
         if (p.c_bfp) {
             // Block-float output (TILE layout): the sums are rounded to bf16 as for a bf16 output and packed with the host
