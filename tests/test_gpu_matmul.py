@@ -453,8 +453,8 @@ def test_rows_at_the_ends_of_the_exponent_range(oracle, kernel, m, block, fmt, k
                 field; the same in every kernel
       E = 247   the largest exponent every kernel takes exactly
       E = 254   exact in the streaming kernels (M < 128) where they take the weights in hidden-one form; in the tiled and
-                expanding kernels, and in the two-band form of the 128-column kernel for BFLOAT4_B (single exact operands),
-                the operand, mantissa x 2^(E - 127), overflows for mantissas >= 2: those columns come out non-finite
+                expanding kernels, and in the two-band form of the 128-column kernel (single exact operands), the operand,
+                mantissa x 2^(E - 127), overflows for mantissas >= 2: those columns come out non-finite
       E = 255   (Inf / NaN sources) the 16 columns that share the exponent are non-finite, all others are untouched
     Expected values are formed here from codes and exponents directly: sign x mantissa x 2^(max(E, 1) - 127 - (W - 1))."""
     knobs("kernel", kernel)
@@ -483,7 +483,7 @@ def test_rows_at_the_ends_of_the_exponent_range(oracle, kernel, m, block, fmt, k
     bound = 2.0 ** -22 * np.abs(ref) + 2.0 * k * 2.0 ** -24 * (np.abs(a64) @ (np.abs(w64) + np.exp2((e_eff - 127).astype(np.float64)))) + 1e-37
     poisoned = np.zeros(n, dtype=bool)
     poisoned[48:64] = True                                   # E = 255
-    if kernel in ("tile", "expanded") or (kernel == "wide" and m > 32 and fmt == BFP4):
+    if kernel in ("tile", "expanded") or (kernel == "wide" and m > 32):
         poisoned |= (codes[77] & ((1 << w_bits) - 1)) >= 2   # E = 254: mantissa x 2^127 overflows
     assert not np.isfinite(c[:, poisoned]).any()
     ok = ~poisoned
@@ -642,8 +642,7 @@ def test_face_rows_with_outliers(oracle, fmt, kernel, knobs):
     a = workloads.bf16_bits_to_f32(a_bits)
     knobs("kernel", kernel.split()[0])
     c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n, out_dtype=torch.float32)[0].cpu().numpy()
-    # hidden-one form: the 64-column kernel, the 128-column kernel with one band, and with two bands of BFLOAT8_B weights
-    hidden = kernel in ("wide", "stream") or (kernel == "wide two bands" and fmt == BFP8)
-    check_against_reference(c, a, w_ref, k, bf16_out=False, face_row_scale=hidden)
+    # hidden-one form: the 64-column kernel and the 128-column kernel with one band
+    check_against_reference(c, a, w_ref, k, bf16_out=False, face_row_scale=kernel in ("wide", "stream"))
     ref = a.astype(np.float64) @ w_ref.astype(np.float64)
     assert np.sqrt(((c - ref) ** 2).mean() / (ref ** 2).mean()) < 1e-6

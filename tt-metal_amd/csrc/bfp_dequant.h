@@ -255,11 +255,24 @@ __device__ __forceinline__ void slab_expand_bfp4(const SlabRaw &r, int q, bf16x8
     for (int j = 0; j < 4; ++j) bop[j] = __builtin_bit_cast(bf16x8, make_uint4(packed[j][0], packed[j][1], packed[j][2], packed[j][3]));
 }
 
-// Which form the 128-column kernel feeds the matrix cores: BFLOAT4_B weights as single exact operands where a workgroup
-// multiplies them with two 32-row bands (the conversion is shared by the bands and the matrix instructions are what such a
-// launch waits for: 22.0 against 23.6 us for [64, 4096] x [4096, 14336]); the hidden-one form below everywhere else (one
-// band: 14.5 against 15.3 us for the same weights, 14.8 against 15.5 us for [14336, 4096]).
-template <int W, int BANDS> constexpr bool single_operand() { return W == 3 && BANDS == 2; }
+// Which form the 128-column kernel feeds the matrix cores: single exact operands where a workgroup multiplies the weights
+// with two 32-row bands (the expansion is shared by the bands and the matrix instructions are what such a launch waits for:
+// BFLOAT4_B 22.0 against 23.6 us for [64, 4096] x [4096, 14336], BFLOAT8_B 32.0 against 33.3 us for [64, 4544] x
+// [4544, 18176]); the hidden-one form below with one band (BFLOAT4_B 14.5 against 15.3 us for [32, 4096] x [4096, 14336];
+// BFLOAT8_B 23.1 against 24.9 us for the Falcon shape).
+template <int W, int BANDS> constexpr bool single_operand() { return BANDS == 2; }
+// BFLOAT8_B the same way: convert, multiply by the row's power of two, keep the upper halves (weights_operand8)
+__device__ __forceinline__ void slab_expand_bfp8(const SlabRaw &r, bf16x8 (&bop)[4]) {
+    const uint32_t words[8] = {r.w01[0], r.w01[1], r.w23[0], r.w23[1], r.w45[0], r.w45[1], r.w67[0], r.w67[1]};
+    float scale[8];
+    uint32_t mags[8];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) { scale[jj] = row_scale((r.e01[jj >> 2] >> (8 * (jj & 3))) & 0xffu); mags[jj] = words[jj] & 0x7f7f7f7fu; }
+    bop[0] = weights_operand8<0>(words, mags, scale);
+    bop[1] = weights_operand8<1>(words, mags, scale);
+    bop[2] = weights_operand8<2>(words, mags, scale);
+    bop[3] = weights_operand8<3>(words, mags, scale);
+}
 
 // Expansion without arithmetic ("hidden-one form"), for kernels that are bound by vector-ALU issue rather than by the
 // matrix pipe.  A code (sign s, mantissa m of W bits) under the shared exponent E of its face row is written into a bf16 as

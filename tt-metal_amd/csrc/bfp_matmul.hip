@@ -597,12 +597,12 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
             if (nb == NB - 1 && refill) fetch(stage_tag);
             if constexpr (single_operand<W, MB>()) {
                 bf16x8 bop[4];
-                slab_expand_bfp4(raw0, q, bop);
+                if constexpr (W == 3) slab_expand_bfp4(raw0, q, bop); else slab_expand_bfp8(raw0, bop);
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) acc[nb * MB + mb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a_now[2 * mb]), bop[j], acc[nb * MB + mb][j], 0, 0, 0);
-                slab_expand_bfp4(raw1, q, bop);
+                if constexpr (W == 3) slab_expand_bfp4(raw1, q, bop); else slab_expand_bfp8(raw1, bop);
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
