@@ -75,6 +75,15 @@ def test_argument_validation_returns_errors_without_launching():
     assert L.ttmi_matmul_bfp(one, 0, one, 3, 4, 2, 32, 32, 64, None, 0, one, 0, 0, None, 0, None) == 1
     assert L.ttmi_matmul_bfp(one, 1, one, 3, 1, 1, 7, 32, 64, None, 0, one, 0, 0, None, 0, None) == 1
     assert L.ttmi_matmul_bfp(one, 0, one, 2, 1, 1, 32, 32, 64, None, 0, one, 0, 0, None, 0, None) == 1
+    # dense weight dtypes (BFLOAT16 = 0, FLOAT32 = 1) pass only through ttmi_matmul_bf16: every other matmul entry point would
+    # decode them as packed tiles, so each refuses them before anything is launched
+    for dense in (0, 1):
+        assert L.ttmi_matmul_bfp(one, 0, one, dense, 1, 1, 32, 32, 64, None, 0, one, 0, 0, None, 0, None) == 1
+        assert b"weight dtype" in L.ttmi_last_error()
+        assert L.ttmi_matmul_bfp_static(one, 0, one, dense, 1, 1, 32, 32, 64, None, 0, one, 0, 0, None) == 1
+        assert b"weight dtype" in L.ttmi_last_error()
+        assert L.ttmi_matmul_bfp_gated(one, 0, one, one, dense, 1, 1, 32, 32, 64, None, 0, one, 0, 0, None, 0, None) == 1
+        assert b"weight dtype" in L.ttmi_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch):

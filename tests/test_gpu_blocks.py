@@ -191,6 +191,33 @@ def test_mistral_mlp_block(oracle, device, seq, dim, hidden_dim, name):
     assert pcc(got, want) >= (0.99 if name == "bfloat8_b" else 0.95)   # 3-bit mantissas: the quantisation itself costs that much
 
 
+@pytest.mark.parametrize("seq,dim,hidden_dim,name", [(32, 128, 352, "bfloat8_b"), (32, 4096, 14336, "bfloat4_b")])
+def test_gated_linear_is_linear_linear_mul_in_one_launch(oracle, device, seq, dim, hidden_dim, name):
+    """ttnn.experimental.gated_linear(x, w1, w3) against what a gated MLP issues on the reference's surface: ttnn.linear(x, w1,
+    activation="silu"), ttnn.linear(x, w3), ttnn.mul.  The fused launch multiplies the two fp32 sums and rounds once, the three
+    ops round each factor to bf16 first: equal within two bf16 roundings, and both within the quantised model's PCC."""
+    import ttnn
+
+    dtype = getattr(ttnn, name)
+    torch.manual_seed(2)
+    gate, up = torch.randn(hidden_dim, dim) * 0.02, torch.randn(hidden_dim, dim) * 0.02
+    x = torch.randn(1, 1, seq, dim).to(torch.bfloat16)
+    tx = ttnn.from_torch(x, dtype=ttnn.bfloat16, layout=ttnn.TILE_LAYOUT, device=device)
+    w1, w3 = (weight_on_device(ttnn, device, w, dtype) for w in (gate, up))
+    fused = ttnn.experimental.gated_linear(tx, w1, w3, activation="silu")
+    assert tuple(fused.shape) == (1, 1, seq, hidden_dim) and fused.dtype == ttnn.bfloat16 and fused.layout == ttnn.TILE_LAYOUT
+    three = ttnn.mul(ttnn.linear(tx, w1, activation="silu"), ttnn.linear(tx, w3))
+    got, ops = ttnn.to_torch(fused)[0, 0].double(), ttnn.to_torch(three)[0, 0].double()
+    xd = x[0, 0].double()
+    want = torch.nn.functional.silu(xd @ quantised(oracle, dtype, gate.t())) * (xd @ quantised(oracle, dtype, up.t()))
+    assert pcc(got, want) >= 0.9999 and pcc(ops, want) >= 0.9999
+    assert torch.all((got - ops).abs() <= 2.0 ** -6 * want.abs() + 1e-6)
+    with pytest.raises(RuntimeError, match="same dtype and shape"):
+        ttnn.experimental.gated_linear(tx, w1, weight_on_device(ttnn, device, up[:32], dtype))
+    with pytest.raises(RuntimeError, match="is not supported as activation"):
+        ttnn.experimental.gated_linear(tx, w1, w3, activation="tanh")
+
+
 # ---- device-resident dtype changes ------------------------------------------------------------------------------------
 @pytest.mark.parametrize("name", ["bfloat8_b", "bfloat4_b"])
 def test_to_layout_with_dtype_and_clone(oracle, device, name):

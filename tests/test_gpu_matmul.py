@@ -523,6 +523,31 @@ def test_a_wait_that_gives_up_is_reported_and_leaves_later_calls_correct(oracle,
     check_against_reference(again.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
 
 
+def test_a_wait_that_gives_up_is_raised_where_the_result_is_read(oracle, knobs):
+    """The same forced give-up through the TT-NN surface: the matmul returns (its kernels run to their end), and the call that
+    brings the bad result to the host — ttnn.to_torch, ttnn.from_device, Tensor.cpu — raises instead of handing it over."""
+    import ttnn
+
+    m, k, n = 32, 2048, 256
+    torch.manual_seed(7)
+    device = ttnn.open_device(0)
+    x = torch.randn(1, 1, m, k).to(torch.bfloat16)
+    tx = ttnn.from_torch(x, dtype=ttnn.bfloat16, layout=ttnn.TILE_LAYOUT, device=device)
+    tw = ttnn.from_torch(torch.randn(1, 1, k, n) * 0.02, dtype=ttnn.bfloat8_b, layout=ttnn.TILE_LAYOUT, device=device)
+    knobs("kernel", "wide")
+    good = ttnn.to_torch(ttnn.matmul(tx, tw))
+    for read in (ttnn.to_torch, ttnn.from_device, lambda t: t.cpu()):
+        knobs("drop_partial_sums", 1)
+        knobs("spin_limit", 3)
+        bad = ttnn.matmul(tx, tw)
+        torch.cuda.synchronize()
+        knobs("drop_partial_sums", 0)
+        knobs("spin_limit", 1 << 20)
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            read(bad)
+        assert torch.equal(ttnn.to_torch(ttnn.matmul(tx, tw)), good)        # reported once; the slots are refilled
+
+
 def test_library_scratch_is_per_stream(oracle):
     """Without a caller workspace every stream gets slots of its own, so decode GEMMs issued on two streams at once do not
     share partial sums (the same two calls on one stream share a buffer and run in order)."""

@@ -211,3 +211,26 @@ def test_tt_lib_matmul_and_bmm(device):
         ttl.tensor.matmul(ta.cpu(), tw)
     out2 = ttl.operations.primary.matmul(ta, tw)
     assert torch.equal(out2.cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch(), out.cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch())
+
+
+@pytest.mark.parametrize("m", [32, 64, 96, 160, 544])        # every GEMM kernel: one band, two bands, three bands, tiled, expanded
+def test_untilize_out_gives_the_tile_result_row_major(device, m):
+    """bmm_op.cpp:1069: with untilize_out the output tensor is ROW_MAJOR; :536-538, :865-867: bfloat16 only.  The values are
+    those of the TILE output, untilized, bit for bit."""
+    import tt_lib as ttl
+
+    torch.manual_seed(5)
+    a = torch.randn((1, 2, m, 256), dtype=torch.bfloat16)
+    w = torch.randn((1, 1, 256, 192), dtype=torch.float32)
+    ta = ttl.tensor.Tensor(a, ttl.tensor.DataType.BFLOAT16).to(ttl.tensor.Layout.TILE).to(device)
+    tw = ttl.tensor.Tensor(w, ttl.tensor.DataType.BFLOAT8_B).to(ttl.tensor.Layout.TILE).to(device)
+    tiles = ttl.tensor.matmul(ta, tw)
+    for rows in (ttl.tensor.matmul(ta, tw, untilize_out=True), ttl.operations.primary.matmul(ta, tw, untilize_out=True)):
+        assert rows.get_layout() == ttl.tensor.Layout.ROW_MAJOR and tuple(rows.get_legacy_shape()) == (1, 2, m, 192)
+        assert rows.get_dtype() == ttl.tensor.DataType.BFLOAT16
+        assert torch.equal(rows.cpu().to_torch().view(torch.int16), tiles.cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch().view(torch.int16))
+    twb = ttl.tensor.Tensor(torch.randn((1, 2, 256, 192)), ttl.tensor.DataType.BFLOAT8_B).to(ttl.tensor.Layout.TILE).to(device)
+    rows = ttl.tensor.bmm(ta, twb, untilize_out=True)
+    assert torch.equal(rows.cpu().to_torch().view(torch.int16), ttl.tensor.bmm(ta, twb).cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch().view(torch.int16))
+    with pytest.raises(RuntimeError, match="output_dtype == DataType::BFLOAT16"):
+        ttl.operations.primary.matmul(ta, tw, output_dtype=ttl.tensor.DataType.BFLOAT8_B, untilize_out=True)

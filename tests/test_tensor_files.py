@@ -86,3 +86,13 @@ def test_errors(tmp_path):
     (tmp_path / "cut.bin").write_bytes(data[:-8])
     with pytest.raises(RuntimeError, match="ends inside"):
         ttnn.load_tensor(tmp_path / "cut.bin")
+    # a header whose element count is not what its shape says (a stale or truncated cache file): refused before any kernel
+    # could index the buffer by the shape
+    (tmp_path / "count.bin").write_bytes(data[:192] + struct.pack("<Q", 8) + data[200:232])
+    with pytest.raises(RuntimeError, match="the header counts 8 elements"):
+        ttnn.load_tensor(tmp_path / "count.bin")
+    header = bytearray(data[:200])
+    header[48 + 8:48 + 16] = struct.pack("<Q", 9)            # Padding::pad_dimensions_[0].back = 9 on a dimension of 4
+    (tmp_path / "pad.bin").write_bytes(bytes(header) + data[200:])
+    with pytest.raises(RuntimeError, match="exceeds the dimension"):
+        ttnn.load_tensor(tmp_path / "pad.bin")

@@ -87,7 +87,20 @@ def _host_tile_tensor(shape, dtype=tt_lib.tensor.DataType.BFLOAT16):
     n = 1
     for s in shape:
         n *= s
-    return tt_lib.tensor.Tensor(None, _raw=(torch.zeros(n, dtype=torch.bfloat16), tuple(shape), tuple(shape), dtype, tt_lib.tensor.Layout.TILE, None))
+    nbytes = {tt_lib.tensor.DataType.BFLOAT16: 2 * n, tt_lib.tensor.DataType.BFLOAT8_B: n // 1024 * 1088, tt_lib.tensor.DataType.BFLOAT4_B: n // 1024 * 576}[dtype]
+    return tt_lib.tensor.Tensor(None, _raw=(torch.zeros(nbytes, dtype=torch.uint8), tuple(shape), tuple(shape), dtype, tt_lib.tensor.Layout.TILE, None))
+
+
+def test_a_buffer_that_does_not_hold_its_shape_is_refused():
+    """Kernels index a buffer by the tensor's shape: a raw buffer of another size never becomes a Tensor."""
+    tile = tt_lib.tensor.Layout.TILE
+    with pytest.raises(RuntimeError, match="the buffer holds 2048 bytes"):
+        tt_lib.tensor.Tensor(None, _raw=(torch.zeros(2048, dtype=torch.uint8), (1, 1, 32, 64), (1, 1, 32, 64), tt_lib.tensor.DataType.BFLOAT16, tile, None))
+    with pytest.raises(RuntimeError, match="whole tiles"):
+        tt_lib.tensor.Tensor(None, _raw=(torch.zeros(544, dtype=torch.uint8), (1, 1, 16, 32), (1, 1, 16, 32), tt_lib.tensor.DataType.BFLOAT8_B,
+                                         tt_lib.tensor.Layout.ROW_MAJOR, None))
+    with pytest.raises(RuntimeError, match="larger without padding"):
+        tt_lib.tensor.Tensor(None, _raw=(torch.zeros(2048, dtype=torch.uint8), (1, 1, 64, 32), (1, 1, 32, 32), tt_lib.tensor.DataType.BFLOAT16, tile, None))
 
 
 def test_elementwise_argument_checks_need_no_gpu():

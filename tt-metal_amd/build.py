@@ -38,31 +38,37 @@ def _stale(target: str, deps) -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
+def _compile(src: str, verbose: bool) -> None:
+    path = os.path.join(CSRC, src)
+    obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
+    if src in ISA_CHECKED:
+        # the device assembly of this file is inspected before the object is built (see check_isa.py)
+        asm = os.path.join(LIB_DIR, src.replace(".hip", ".s"))
+        cmd = [HIPCC] + FLAGS + ["-S", "--cuda-device-only", path, "-o", asm]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True)
+        import check_isa
+        if getattr(check_isa, ISA_CHECKED[src])(asm):
+            if os.path.exists(obj):
+                os.remove(obj)
+            raise RuntimeError(f"{src}: the compiler moved registers of hand-scheduled loads; see check_isa.py")
+        os.remove(asm)
+    cmd = [HIPCC] + FLAGS + ["-c", path, "-o", obj]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+
+
 def build(force: bool = False, verbose: bool = False) -> str:
+    from concurrent.futures import ThreadPoolExecutor
+
     os.makedirs(LIB_DIR, exist_ok=True)
-    objs = []
-    for src in SOURCES:
-        path = os.path.join(CSRC, src)
-        obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
-        if force or _stale(obj, [path] + HEADERS):
-            if src in ISA_CHECKED:
-                # the device assembly of this file is inspected before the object is built (see check_isa.py)
-                asm = os.path.join(LIB_DIR, src.replace(".hip", ".s"))
-                cmd = [HIPCC] + FLAGS + ["-S", "--cuda-device-only", path, "-o", asm]
-                if verbose:
-                    print(" ".join(cmd), flush=True)
-                subprocess.run(cmd, check=True)
-                import check_isa
-                if getattr(check_isa, ISA_CHECKED[src])(asm):
-                    if os.path.exists(obj):
-                        os.remove(obj)
-                    raise RuntimeError(f"{src}: the compiler moved registers of hand-scheduled loads; see check_isa.py")
-                os.remove(asm)
-            cmd = [HIPCC] + FLAGS + ["-c", path, "-o", obj]
-            if verbose:
-                print(" ".join(cmd), flush=True)
-            subprocess.run(cmd, check=True)
-        objs.append(obj)
+    objs = [os.path.join(LIB_DIR, src.replace(".hip", ".o")) for src in SOURCES]
+    stale = [src for src, obj in zip(SOURCES, objs) if force or _stale(obj, [os.path.join(CSRC, src)] + HEADERS)]
+    # the translation units are independent: compile those that are out of date side by side
+    with ThreadPoolExecutor(max_workers=min(4, max(1, len(stale)))) as pool:
+        list(pool.map(lambda src: _compile(src, verbose), stale))
     if force or _stale(LIB, objs):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
         if verbose:

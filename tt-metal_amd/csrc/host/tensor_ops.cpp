@@ -67,6 +67,9 @@ void copy(Buffer &dst, const Buffer &src, size_t nbytes) {
     const hipMemcpyKind kind = dst.device < 0 ? hipMemcpyDeviceToHost : src.device < 0 ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice;
     hip_check(hipMemcpyAsync(dst.data, src.data, nbytes, kind, st), "hipMemcpyAsync");
     hip_check(hipStreamSynchronize(st), "hipStreamSynchronize");
+    // Data that leaves the device is where a user first looks at a result: whatever a kernel has reported by now (a bounded
+    // wait that gave up) is raised here, not at the next launch.
+    if (kind == hipMemcpyDeviceToHost) check(ttmi_device_status());
 }
 
 Buffer moved_to(const Buffer &src, int device) {
@@ -154,6 +157,24 @@ Buffer window(DataType dtype, const Buffer &src, const Dims &src_shape, const Di
     return out;
 }
 
+// Kernels index a buffer by the tensor's shape: a tensor whose buffer does not hold exactly what its shape, dtype and layout
+// say (a truncated or stale cache file, a raw buffer of the wrong size) is refused before any of them can run.
+void check_consistent(const Tensor &t, const std::string &what) {
+    if (!element_bytes(t.dtype) && !is_block_float(t.dtype)) raise(what + ": unsupported DataType " + std::to_string((int)t.dtype));
+    if (t.layout != Layout::ROW_MAJOR && t.layout != Layout::TILE) raise(what + ": unsupported Layout " + std::to_string((int)t.layout));
+    for (size_t i = 0; i < t.shape.size(); ++i)
+        if (t.shape[i] > t.padded[i]) raise(what + ": dimension " + std::to_string(i) + " is larger without padding (" + std::to_string(t.shape[i]) + ") than with it (" + std::to_string(t.padded[i]) + ")");
+    const uint64_t volume = product(t.padded);
+    if (is_block_float(t.dtype) && volume % 1024) raise(what + ": a block-float tensor holds whole tiles, " + std::to_string(volume) + " elements are not");
+    if (t.layout == Layout::TILE && !t.padded.empty()) {
+        const size_t r = t.padded.size();
+        if (t.padded[r - 1] % 32 || (r > 1 && t.padded[r - 2] % 32)) raise(what + ": the last two dimensions of a TILE tensor must be multiples of 32");
+    }
+    const size_t expected = storage_bytes(t.dtype, t.layout, t.padded);
+    if (t.buffer.nbytes != expected)
+        raise(what + ": the buffer holds " + std::to_string(t.buffer.nbytes) + " bytes, shape " + list_of(t.padded) + " of " + name_of(t.dtype) + " needs " + std::to_string(expected));
+}
+
 void require_rank4(const Dims &d, const char *what) {
     if (d.size() != 4) raise(std::string(what) + ": shapes must have rank 4");
 }
@@ -219,6 +240,7 @@ Tensor wrap(Buffer buffer, const Dims &shape, const Dims &padded, DataType dtype
     Tensor t;
     t.buffer = std::move(buffer);
     t.shape = shape; t.padded = padded; t.dtype = dtype; t.layout = layout;
+    check_consistent(t, "Tensor");
     return t;
 }
 
@@ -375,7 +397,7 @@ Tensor device_unpad(const Tensor &t, const Dims &start, const Dims &end) {
 // matmul
 // ---------------------------------------------------------------------------------------------------------------------------
 Tensor matmul(const Tensor &a, const Tensor &b, bool bcast_batch, const Tensor *bias, int activation, std::optional<DataType> output_dtype,
-              const std::string &op) {
+              const std::string &op, bool untilize_out) {
     const std::pair<const Tensor *, const char *> operands[2] = {{&a, "input_tensor_a"}, {&b, "input_tensor_b"}};
     for (const auto &[t, name] : operands) {
         if (!t->on_device()) raise("TT_FATAL: Operands to " + op + " need to be on device! (" + name + ")");
@@ -400,6 +422,8 @@ Tensor matmul(const Tensor &a, const Tensor &b, bool bcast_batch, const Tensor *
     const DataType out_dtype = output_dtype ? *output_dtype : a.dtype;      // bmm_op.hpp:388: the output takes input a's dtype
     if (out_dtype != DataType::BFLOAT16 && !is_block_float(out_dtype))
         raise(op + ": output dtype " + name_of(out_dtype) + " is not supported (BFLOAT16, BFLOAT8_B, BFLOAT4_B)");
+    if (untilize_out && out_dtype != DataType::BFLOAT16)                                                // bmm_op.cpp:536-538, 865-867
+        raise("TT_FATAL: this->output_dtype == DataType::BFLOAT16 (untilize_out writes a ROW_MAJOR output, which a block-float tensor cannot be)");
     const int device = a.buffer.device;
     DeviceGuard guard(device);
     Buffer bias_row;
@@ -426,18 +450,58 @@ Tensor matmul(const Tensor &a, const Tensor &b, bool bcast_batch, const Tensor *
     // library (the host packers' arithmetic on the bf16-rounded sums: parity with the Tensix packer unpinned)
     Buffer a_tiles = is_block_float(a.dtype) ? typecast_tiles(a.buffer, a.dtype, DataType::BFLOAT16, a_elements, device) : a.buffer;
     const bool packed_out = is_block_float(out_dtype);
+    const int c_layout = untilize_out ? TTMI_ROW_MAJOR : TTMI_TILE;                                     // bmm_op.cpp:1069
     Buffer c = allocate(packed_out ? storage_bytes(out_dtype, Layout::TILE, {batch_a, m, n}) : c_elements * 2, device);
     if (b.dtype == DataType::BFLOAT16)      // two bf16 operands: not the tuned path (the weights are re-laid-out on every call), but the same surface
         check(ttmi_matmul_bf16(a_tiles.data, TTMI_TILE, b.buffer.data, batch_a, batch_b, m, k, n, bias ? bias_row.data : nullptr, activation, c.data,
-                               TTMI_TILE, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0, stream_of(device)));
+                               c_layout, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0, stream_of(device)));
     else
         check(ttmi_matmul_bfp(a_tiles.data, TTMI_TILE, (const uint32_t *)b.buffer.data, (int)b.dtype, batch_a, batch_b, m, k, n,
-                              bias ? bias_row.data : nullptr, activation, c.data, TTMI_TILE, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0,
+                              bias ? bias_row.data : nullptr, activation, c.data, c_layout, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0,
                               stream_of(device)));
     Tensor out;
     out.buffer = std::move(c);
     out.shape.assign(a.shape.begin(), a.shape.end() - 1);
     out.shape.push_back(b.shape.back());
+    out.padded.assign(pa.begin(), pa.end() - 1);
+    out.padded.push_back(n);
+    out.dtype = out_dtype;
+    out.layout = untilize_out ? Layout::ROW_MAJOR : Layout::TILE;     // the padded rows and columns stay part of the row-major output
+    return out;
+}
+
+// silu(x w1) * (x w3) of a gated MLP (models/demos/mistral7b/tt/mistral_mlp.py:43-82 issues it as linear(activation), linear,
+// mul) as ONE launch: both weight matrices stream through the same workgroups and share the activation loads.
+Tensor matmul_gated(const Tensor &a, const Tensor &b_gate, const Tensor &b_up, int activation, std::optional<DataType> output_dtype,
+                    const std::string &op) {
+    const std::pair<const Tensor *, const char *> operands[3] = {{&a, "input_tensor_a"}, {&b_gate, "input_tensor_b"}, {&b_up, "input_tensor_c"}};
+    for (const auto &[t, name] : operands) {
+        if (!t->on_device()) raise("TT_FATAL: Operands to " + op + " need to be on device! (" + name + ")");
+        if (t->layout != Layout::TILE) raise("TT_FATAL: Inputs to " + op + " must be tilized (" + name + ")");
+    }
+    if (a.dtype != DataType::BFLOAT16) raise(std::string("TT_FATAL: Unsupported data format for input a: ") + name_of(a.dtype));
+    if (!is_block_float(b_gate.dtype) || b_up.dtype != b_gate.dtype || b_up.padded != b_gate.padded)
+        raise("TT_FATAL: " + op + ": the two weight tensors must be block-float tensors of the same dtype and shape");
+    const Dims &pa = a.padded, &pb = b_gate.padded;
+    if (pa.size() < 2 || pb.size() < 2 || pa.size() > 4 || pb.size() > 4) raise("TT_FATAL: " + op + " supports ranks 2 to 4");
+    if (product(pb, 0, pb.size() - 2) != 1) raise("TT_FATAL: " + op + " expects input tensors of shapes BCMK*11KN=BCMN");
+    if (pa.back() != pb[pb.size() - 2])
+        raise("TT_FATAL: The width of the first tensor must be equal to the height of the second tensor (a.shape[-1] = " + std::to_string(pa.back()) +
+              ", b.shape[-2] = " + std::to_string(pb[pb.size() - 2]) + ")");
+    const DataType out_dtype = output_dtype ? *output_dtype : a.dtype;
+    if (out_dtype != DataType::BFLOAT16 && !is_block_float(out_dtype))
+        raise(op + ": output dtype " + name_of(out_dtype) + " is not supported (BFLOAT16, BFLOAT8_B, BFLOAT4_B)");
+    const uint32_t batch = (uint32_t)product(pa, 0, pa.size() - 2), m = pa[pa.size() - 2], k = pa.back(), n = pb.back();
+    const int device = a.buffer.device;
+    DeviceGuard guard(device);
+    const bool packed_out = is_block_float(out_dtype);
+    Buffer c = allocate(packed_out ? storage_bytes(out_dtype, Layout::TILE, {batch, m, n}) : (size_t)batch * m * n * 2, device);
+    check(ttmi_matmul_bfp_gated(a.buffer.data, TTMI_TILE, (const uint32_t *)b_gate.buffer.data, (const uint32_t *)b_up.buffer.data, (int)b_gate.dtype, batch, 1,
+                                m, k, n, nullptr, activation, c.data, TTMI_TILE, (int)out_dtype, nullptr, 0, stream_of(device)));
+    Tensor out;
+    out.buffer = std::move(c);
+    out.shape.assign(a.shape.begin(), a.shape.end() - 1);
+    out.shape.push_back(b_gate.shape.back());
     out.padded.assign(pa.begin(), pa.end() - 1);
     out.padded.push_back(n);
     out.dtype = out_dtype;
@@ -475,7 +539,7 @@ Tensor ttnn_matmul(const std::string &operation_name, const Tensor &a, const Ten
     const uint64_t batch_b = product(b.padded, 0, b.padded.size() - 2);
     if (batch_b != 1 && activation) raise("Cannot use activation with batched input b");              // matmul.py:215-216
     if (bias) ttnn_validate(operation_name, *bias);
-    return matmul(a, b, batch_b == 1, bias, act, dtype, operation_name);
+    return matmul(a, b, batch_b == 1, bias, act, dtype, operation_name, false);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -716,14 +780,26 @@ Tensor load_tensor(const std::string &file_name) {
     Tensor t;
     t.dtype = dtype; t.layout = (Layout)h.layout;
     for (size_t i = 0; i < h.rank; ++i) {
+        if (h.pad[i].front > h.dimensions[i] || h.pad[i].back > h.dimensions[i] - h.pad[i].front) {
+            std::fclose(f);
+            raise("\"" + file_name + "\": the padding of dimension " + std::to_string(i) + " exceeds the dimension");
+        }
         t.padded.push_back(h.dimensions[i]);
         t.shape.push_back((uint32_t)(h.dimensions[i] - h.pad[i].front - h.pad[i].back));
+    }
+    // the count must be what the shape says: everything downstream indexes the buffer by the shape
+    const size_t expected = storage_bytes(dtype, t.layout, t.padded);
+    if (h.count > expected / file_element_bytes(dtype) || (size_t)h.count * file_element_bytes(dtype) != expected) {
+        std::fclose(f);
+        raise("\"" + file_name + "\": the header counts " + std::to_string(h.count) + " elements, shape " + list_of(t.padded) + " of " + name_of(dtype) + " needs " +
+              std::to_string(expected / file_element_bytes(dtype)));
     }
     const size_t bytes = (size_t)h.count * file_element_bytes(dtype);
     t.buffer = allocate(bytes, -1);
     const bool ok = bytes == 0 || std::fread(t.buffer.data, bytes, 1, f) == 1;
     std::fclose(f);
     if (!ok) raise("\"" + file_name + "\" ends inside the tensor data");
+    check_consistent(t, "\"" + file_name + "\"");
     return t;
 }
 

@@ -71,8 +71,12 @@ Tensor unpad_from_tile(const Tensor &t, const Dims &output_shape);              
 Tensor device_unpad(const Tensor &t, const Dims &start, const Dims &end);                              // unpad_op.cpp:95-125
 
 // ---- matmul family (bmm_op.cpp:518-539, 828-1049) ---------------------------------------------------------------------------
+// untilize_out: the output is a ROW_MAJOR bf16 tensor of the padded shape instead of a TILE one (bmm_op.cpp:1069; :536-538, :865-867)
 Tensor matmul(const Tensor &a, const Tensor &b, bool bcast_batch, const Tensor *bias, int activation, std::optional<DataType> output_dtype,
-              const std::string &op);
+              const std::string &op, bool untilize_out = false);
+// act(a . b_gate) * (a . b_up) in one launch (ttmi_matmul_bfp_gated): what a gated MLP issues as linear(activation), linear, mul
+Tensor matmul_gated(const Tensor &a, const Tensor &b_gate, const Tensor &b_up, int activation, std::optional<DataType> output_dtype,
+                    const std::string &op);
 // ttnn.matmul / ttnn.linear (ttnn/cpp/ttnn/operations/matmul.hpp:39-62, ttnn/ttnn/operations/matmul.py:200-220)
 Tensor ttnn_matmul(const std::string &operation_name, const Tensor &a, const Tensor &b, const Tensor *bias,
                    const std::optional<std::string> &activation, std::optional<DataType> dtype);

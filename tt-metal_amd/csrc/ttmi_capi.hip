@@ -26,8 +26,8 @@ int check_launch(const char *what) { return check_hip(hipGetLastError(), what); 
 static bool is_bfp(int fmt) { return fmt == TTMI_BFLOAT8_B || fmt == TTMI_BFLOAT4_B; }
 
 int validate_matmul(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch, uint32_t m, uint32_t k,
-                    uint32_t n, int activation, const void *c, int c_layout, int c_dtype) {
-    if (!is_bfp(b_fmt) && b_fmt != TTMI_BFLOAT16) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: weight dtype must be BFLOAT8_B or BFLOAT4_B, got %d", b_fmt);
+                    uint32_t n, int activation, const void *c, int c_layout, int c_dtype, bool allow_bf16_weights) {
+    if (!is_bfp(b_fmt) && !(allow_bf16_weights && b_fmt == TTMI_BFLOAT16)) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: weight dtype must be BFLOAT8_B or BFLOAT4_B, got %d", b_fmt);
     if (!a || !b || !c) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: null pointer");
     if (batch == 0 || m == 0 || k == 0 || n == 0) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: empty dimension");
     // tt_eager/tt_dnn/op_library/bmm/multi_core_reuse_mcast_1d_optimized/...cpp:1207-1210: tile-multiple shapes
@@ -152,7 +152,7 @@ size_t ttmi_matmul_bf16_workspace_bytes(uint32_t b_batch, uint32_t k, uint32_t n
 int ttmi_matmul_bf16(const void *a, int a_layout, const void *b, uint32_t batch, uint32_t b_batch, uint32_t m, uint32_t k, uint32_t n,
                      const void *bias, int activation, void *c, int c_layout, int c_dtype, void *workspace, size_t workspace_bytes,
                      void *stream) {
-    if (int rc = validate_matmul(a, a_layout, (const uint32_t *)b, TTMI_BFLOAT16, batch, b_batch, m, k, n, activation, c, c_layout, c_dtype)) return rc;
+    if (int rc = validate_matmul(a, a_layout, (const uint32_t *)b, TTMI_BFLOAT16, batch, b_batch, m, k, n, activation, c, c_layout, c_dtype, true)) return rc;
     MatmulArgs args{a, a_layout, (const uint32_t *)b, TTMI_BFLOAT16, batch, b_batch, m, k, n, bias, activation, c, c_layout, c_dtype, workspace, workspace_bytes};
     return matmul_bf16(args, (hipStream_t)stream);
 }
@@ -160,7 +160,6 @@ int ttmi_matmul_bf16(const void *a, int a_layout, const void *b, uint32_t batch,
 int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch,
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
                     int c_dtype, void *workspace, size_t workspace_bytes, void *stream) {
-    if (!is_bfp(b_fmt)) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: weight dtype must be BFLOAT8_B or BFLOAT4_B, got %d", b_fmt);
     if (int rc = validate_matmul(a, a_layout, b, b_fmt, batch, b_batch, m, k, n, activation, c, c_layout, c_dtype)) return rc;
     MatmulArgs args{a, a_layout, b, b_fmt, batch, b_batch, m, k, n, bias, activation, c, c_layout, c_dtype, workspace, workspace_bytes};
     return matmul_bfp(args, (hipStream_t)stream);

@@ -66,9 +66,10 @@ struct MatmulArgs {
     bool no_alloc = false;          // the call may not allocate: `workspace` is all the scratch there is, its last 256 bytes stand
                                     // in for the error word when the device has none yet
 };
-// the argument checks of ttmi_matmul_bfp (everything but the workspace)
+// the argument checks of the matmul entry points (everything but the workspace); dense bf16 weights pass only where the
+// caller says so (ttmi_matmul_bf16): every other entry point decodes `b` as packed block-float tiles
 int validate_matmul(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch, uint32_t m, uint32_t k,
-                    uint32_t n, int activation, const void *c, int c_layout, int c_dtype);
+                    uint32_t n, int activation, const void *c, int c_layout, int c_dtype, bool allow_bf16_weights = false);
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
 int matmul_bfp(const MatmulArgs &args, hipStream_t st);         // streaming kernel (decode shapes) or the tiled one
 int matmul_bfp_stream(const MatmulArgs &args, hipStream_t st);

@@ -59,6 +59,12 @@ std::optional<host::DataType> optional_dtype(const py::object &dtype) {
     if (dtype.is_none()) return std::nullopt;
     return (host::DataType)py::cast<int>(dtype);
 }
+// Runs a host-layer operation (launches, synchronising copies) with the GIL released; the Runtime callbacks re-acquire it.
+// Arguments are converted from Python before, the result is converted after.
+template <typename F> auto unlocked(F &&f) {
+    py::gil_scoped_release release;
+    return f();
+}
 const host::Tensor *optional_tensor(const py::object &t) { return t.is_none() ? nullptr : &py::cast<const host::Tensor &>(t); }
 
 void bind_tensor_layer(py::module_ &m) {
@@ -76,7 +82,9 @@ void bind_tensor_layer(py::module_ &m) {
     m.def("set_runtime",
           [](py::function allocate, py::function stream, py::function gpu_available) {
               host::Runtime rt;
+              // the operations below run with the GIL released; the callbacks are Python and take it back for their own duration
               rt.allocate = [allocate](size_t nbytes, int device) {
+                  py::gil_scoped_acquire gil;
                   py::object storage = allocate(nbytes, device);                  // flat uint8 tensor on that device (-1: host)
                   host::Buffer b;
                   b.data = reinterpret_cast<void *>(py::cast<uintptr_t>(storage.attr("data_ptr")()));
@@ -85,8 +93,8 @@ void bind_tensor_layer(py::module_ &m) {
                   b.owner = keep_alive(std::move(storage));
                   return b;
               };
-              rt.stream = [stream](int device) { return reinterpret_cast<void *>(py::cast<uintptr_t>(stream(device))); };
-              rt.gpu_available = [gpu_available]() { return py::cast<bool>(gpu_available()); };
+              rt.stream = [stream](int device) { py::gil_scoped_acquire gil; return reinterpret_cast<void *>(py::cast<uintptr_t>(stream(device))); };
+              rt.gpu_available = [gpu_available]() { py::gil_scoped_acquire gil; return py::cast<bool>(gpu_available()); };
               host::set_runtime(std::move(rt));
               // the callbacks are Python objects: they go before the interpreter does
               static bool registered = false;
@@ -105,29 +113,43 @@ void bind_tensor_layer(py::module_ &m) {
               return host::wrap(std::move(b), shape, padded, (host::DataType)dtype, (host::Layout)layout);
           },
           "a Tensor over memory that a Python object owns");
-    m.def("from_host", [](uintptr_t data, host::Dims shape, int dtype) { return host::from_host(reinterpret_cast<const void *>(data), shape, (host::DataType)dtype); },
+    m.def("from_host", [](uintptr_t data, host::Dims shape, int dtype) { return unlocked([&] { return host::from_host(reinterpret_cast<const void *>(data), shape, (host::DataType)dtype); }); },
           "tt_lib.tensor.Tensor(torch_tensor, data_type), tt_lib_bindings_tensor_pytensor.cpp:26-167");
-    m.def("to_layout", [](const host::Tensor &t, int layout) { return host::to_layout(t, (host::Layout)layout); });
-    m.def("to_device", &host::to_device);
-    m.def("to_host", &host::to_host);
+    const auto no_gil = py::call_guard<py::gil_scoped_release>();
+    m.def("to_layout", [](const host::Tensor &t, int layout) { return host::to_layout(t, (host::Layout)layout); }, no_gil);
+    m.def("to_device", &host::to_device, no_gil);
+    m.def("to_host", &host::to_host, no_gil);
     m.def("reshape", &host::reshape);
-    m.def("to_torch", &host::to_torch);
-    m.def("pad", &host::pad);
-    m.def("unpad", &host::unpad);
-    m.def("pad_to_tile", &host::pad_to_tile);
-    m.def("unpad_from_tile", &host::unpad_from_tile);
-    m.def("device_unpad", &host::device_unpad);
+    m.def("to_torch", &host::to_torch, no_gil);
+    m.def("pad", &host::pad, no_gil);
+    m.def("unpad", &host::unpad, no_gil);
+    m.def("pad_to_tile", &host::pad_to_tile, no_gil);
+    m.def("unpad_from_tile", &host::unpad_from_tile, no_gil);
+    m.def("device_unpad", &host::device_unpad, no_gil);
     m.def("matmul",
           [](const host::Tensor &a, const host::Tensor &b, bool bcast_batch, const py::object &bias, int activation, const py::object &output_dtype,
-             const std::string &op) { return host::matmul(a, b, bcast_batch, optional_tensor(bias), activation, optional_dtype(output_dtype), op); },
+             const std::string &op, bool untilize_out) {
+              const host::Tensor *bias_tensor = optional_tensor(bias);
+              const std::optional<host::DataType> dtype = optional_dtype(output_dtype);
+              return unlocked([&] { return host::matmul(a, b, bcast_batch, bias_tensor, activation, dtype, op, untilize_out); });
+          },
           py::arg("a"), py::arg("b"), py::arg("bcast_batch"), py::arg("bias") = py::none(), py::arg("activation") = 0, py::arg("output_dtype") = py::none(),
-          py::arg("op") = "matmul", "tt::operations::primary::matmul, tt_eager/tt_dnn/op_library/bmm/bmm_op.cpp:828-1049");
+          py::arg("op") = "matmul", py::arg("untilize_out") = false, "tt::operations::primary::matmul, tt_eager/tt_dnn/op_library/bmm/bmm_op.cpp:828-1049");
+    m.def("matmul_gated",
+          [](const host::Tensor &a, const host::Tensor &b_gate, const host::Tensor &b_up, int activation, const py::object &output_dtype, const std::string &op) {
+              const std::optional<host::DataType> dtype = optional_dtype(output_dtype);
+              return unlocked([&] { return host::matmul_gated(a, b_gate, b_up, activation, dtype, op); });
+          },
+          py::arg("a"), py::arg("b_gate"), py::arg("b_up"), py::arg("activation") = 0, py::arg("output_dtype") = py::none(), py::arg("op") = "gated_linear",
+          "act(a . b_gate) * (a . b_up) in one launch: linear(activation) + linear + mul of a gated MLP (models/demos/mistral7b/tt/mistral_mlp.py:43-82)");
     m.def("ttnn_matmul",
           [](const std::string &name, const host::Tensor &a, const host::Tensor &b, const py::object &bias, const py::object &activation,
              const py::object &dtype) {
               std::optional<std::string> act;
               if (!activation.is_none()) act = py::cast<std::string>(py::str(activation));
-              return host::ttnn_matmul(name, a, b, optional_tensor(bias), act, optional_dtype(dtype));
+              const host::Tensor *bias_tensor = optional_tensor(bias);
+              const std::optional<host::DataType> out_dtype = optional_dtype(dtype);
+              return unlocked([&] { return host::ttnn_matmul(name, a, b, bias_tensor, act, out_dtype); });
           },
           py::arg("operation_name"), py::arg("a"), py::arg("b"), py::arg("bias") = py::none(), py::arg("activation") = py::none(), py::arg("dtype") = py::none(),
           "ttnn.matmul / ttnn.linear, ttnn/cpp/ttnn/operations/matmul.hpp:44-214");
@@ -137,21 +159,27 @@ void bind_tensor_layer(py::module_ &m) {
         return host::activation_code(act);
     });
     m.def("eltwise",
-          [](int op, const host::Tensor &a, const py::object &b, float scalar, const std::string &name) { return host::eltwise(op, a, optional_tensor(b), scalar, name); },
+          [](int op, const host::Tensor &a, const py::object &b, float scalar, const std::string &name) {
+              const host::Tensor *other = optional_tensor(b);
+              return unlocked([&] { return host::eltwise(op, a, other, scalar, name); });
+          },
           py::arg("op"), py::arg("a"), py::arg("b") = py::none(), py::arg("scalar") = 0.0f, py::arg("name") = "eltwise");
-    m.def("typecast", [](const host::Tensor &t, int dtype) { return host::typecast(t, (host::DataType)dtype); });
-    m.def("clone", [](const host::Tensor &t, const py::object &dtype) { return host::clone(t, optional_dtype(dtype)); });
-    m.def("tilize", [](const host::Tensor &t, const py::object &dtype) { return host::tilize(t, optional_dtype(dtype)); });
+    m.def("typecast", [](const host::Tensor &t, int dtype) { return host::typecast(t, (host::DataType)dtype); }, no_gil);
+    m.def("clone", [](const host::Tensor &t, const py::object &dtype) { const auto d = optional_dtype(dtype); return unlocked([&] { return host::clone(t, d); }); });
+    m.def("tilize", [](const host::Tensor &t, const py::object &dtype) { const auto d = optional_dtype(dtype); return unlocked([&] { return host::tilize(t, d); }); });
     m.def("ttnn_from_torch_block_float",
           [](uintptr_t data, int src_dtype, host::Dims shape, int dtype, int device) {
-              return host::ttnn_from_torch_block_float(reinterpret_cast<const void *>(data), (host::DataType)src_dtype, shape, (host::DataType)dtype, device);
+              return unlocked([&] { return host::ttnn_from_torch_block_float(reinterpret_cast<const void *>(data), (host::DataType)src_dtype, shape, (host::DataType)dtype, device); });
           },
           "ttnn.from_torch(dtype=bfloat8_b|bfloat4_b, layout=TILE_LAYOUT), ttnn/ttnn/operations/core.py:245-311, as one fused kernel");
-    m.def("ttnn_to_torch", &host::ttnn_to_torch);
-    m.def("ttnn_to_layout", [](const host::Tensor &t, int layout, const py::object &dtype) { return host::ttnn_to_layout(t, (host::Layout)layout, optional_dtype(dtype)); });
-    m.def("ttnn_getitem_prefix", &host::ttnn_getitem_prefix);
-    m.def("dump_tensor", &host::dump_tensor);
-    m.def("load_tensor", &host::load_tensor);
+    m.def("ttnn_to_torch", &host::ttnn_to_torch, no_gil);
+    m.def("ttnn_to_layout", [](const host::Tensor &t, int layout, const py::object &dtype) {
+        const auto d = optional_dtype(dtype);
+        return unlocked([&] { return host::ttnn_to_layout(t, (host::Layout)layout, d); });
+    });
+    m.def("ttnn_getitem_prefix", &host::ttnn_getitem_prefix, no_gil);
+    m.def("dump_tensor", &host::dump_tensor, no_gil);
+    m.def("load_tensor", &host::load_tensor, no_gil);
 }
 
 PYBIND11_MODULE(_ttmi, m) {

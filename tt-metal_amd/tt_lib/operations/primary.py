@@ -12,7 +12,8 @@ def matmul(input_tensor_a, input_tensor_b, bias=None, program_config=None, outpu
            compute_kernel_config=None, untilize_out=False, *, activation=None):
     """Mixed dtype (bf16 activations x block-float weights) is legal here (bmm_op.cpp:839).  program_config and
     compute_kernel_config describe Tensix grids and fidelity phases and are accepted and ignored; a fused activation
-    carried by the program config (`fused_activation`) is honoured."""
+    carried by the program config (`fused_activation`) is honoured, and so is untilize_out (a ROW_MAJOR bfloat16 output:
+    bmm_op.cpp:1069, checks at :536-538 and :865-867)."""
     fused = activation if activation is not None else getattr(program_config, "fused_activation", None)
     if isinstance(fused, (tuple, list)):
         fused = fused[0]
@@ -24,4 +25,4 @@ def matmul(input_tensor_a, input_tensor_b, bias=None, program_config=None, outpu
     for extent in tuple(input_tensor_b.shape.with_tile_padding())[:-2]:
         batch_b *= extent
     return _t._matmul(input_tensor_a, input_tensor_b, bcast_batch=batch_b == 1, bias=bias, activation=_ACT[fused],
-                      output_dtype=output_dtype, op="primary.matmul")
+                      output_dtype=output_dtype, op="primary.matmul", untilize_out=untilize_out)

@@ -299,19 +299,20 @@ def _handle_or_none(t):
 def matmul(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None, kernel_config=None,
            untilize_out: bool = False) -> Tensor:
     """tt_lib.tensor.matmul: [B, C, M, K] x [1, 1, K, N] (tt_lib_bindings_tensor_custom_bmm_ops.cpp:50-65, bmm_op.hpp:388)."""
-    return _matmul(input_a, input_b, bcast_batch=True, op="matmul")
+    return _matmul(input_a, input_b, bcast_batch=True, op="matmul", untilize_out=untilize_out)
 
 
 def bmm(input_a: Tensor, input_b: Tensor, output_mem_config: Optional[MemoryConfig] = None, kernel_config=None,
         untilize_out: bool = False) -> Tensor:
     """tt_lib.tensor.bmm: [B, C, M, K] x [B, C, K, N] (tt_lib_bindings_tensor_custom_bmm_ops.cpp:66-81, bmm_op.hpp:425)."""
-    return _matmul(input_a, input_b, bcast_batch=False, op="bmm")
+    return _matmul(input_a, input_b, bcast_batch=False, op="bmm", untilize_out=untilize_out)
 
 
 def _matmul(a: Tensor, b: Tensor, *, bcast_batch: bool, bias: Optional[Tensor] = None, activation: int = capi.ACT_NONE,
-            output_dtype: Optional[DataType] = None, op: str = "matmul") -> Tensor:
-    """Shared body of matmul / bmm / primary.matmul: validation (bmm_op.cpp:518-539,828-1049) and dispatch are in the C++ layer."""
-    return _wrap(_m().matmul(a._t, b._t, bcast_batch, _handle_or_none(bias), int(activation), _opt(output_dtype), op))
+            output_dtype: Optional[DataType] = None, op: str = "matmul", untilize_out: bool = False) -> Tensor:
+    """Shared body of matmul / bmm / primary.matmul: validation (bmm_op.cpp:518-539,828-1049) and dispatch are in the C++ layer.
+    untilize_out: the output is ROW_MAJOR instead of TILE (bmm_op.cpp:1069), bfloat16 only (bmm_op.cpp:536-538, 865-867)."""
+    return _wrap(_m().matmul(a._t, b._t, bcast_batch, _handle_or_none(bias), int(activation), _opt(output_dtype), op, bool(untilize_out)))
 
 
 def unpad(input_tensor: Tensor, output_tensor_start, output_tensor_end, output_mem_config: Optional[MemoryConfig] = None) -> Tensor:

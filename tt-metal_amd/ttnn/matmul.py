@@ -27,3 +27,16 @@ def linear(input_tensor_a: Tensor, input_tensor_b: Tensor, *, bias: Optional[Ten
            use_1d_systolic_array: Optional[bool] = None, compute_kernel_config=None) -> Tensor:
     """act(A @ B + bias): bias row-broadcast, activation in {None, "relu", "gelu", "silu"}, fused into the GEMM epilogue."""
     return _run("ttnn.linear", input_tensor_a, input_tensor_b, bias, activation, dtype)
+
+
+def gated_linear(input_tensor_a: Tensor, gate_weight: Tensor, up_weight: Tensor, *, activation: Optional[str] = "silu",
+                 memory_config=None, dtype: Optional[DataType] = None, core_grid=None, compute_kernel_config=None) -> Tensor:
+    """act(A @ W_gate) * (A @ W_up) in ONE launch.  No counterpart in tt-metal, whose gated MLPs issue
+    ``ttnn.linear(x, w1, activation="silu")``, ``ttnn.linear(x, w3)`` and ``ttnn.mul``
+    (models/demos/mistral7b/tt/mistral_mlp.py:43-82); exported as ``ttnn.experimental.gated_linear``.  Both weight tensors are
+    block-float, of one dtype and shape, and stream through the same workgroups, which share the activation loads."""
+    for t, name in ((input_tensor_a, "input_tensor_a"), (gate_weight, "gate_weight"), (up_weight, "up_weight")):
+        if not isinstance(t, Tensor):
+            raise RuntimeError(f"ttnn.experimental.gated_linear: {name} must be a ttnn.Tensor")
+    act = _m().activation_code(activation)
+    return _wrap(_m().matmul_gated(input_tensor_a._t, gate_weight._t, up_weight._t, act, _opt(dtype), "ttnn.experimental.gated_linear"))
