@@ -22,14 +22,14 @@ def oracle():
 
 
 # knobs of libttmi's test entry point (tt-metal_amd/csrc/ttmi_internal.h: TTMI_KNOB_*)
-KNOB = {"kernel": 0, "workgroups": 1, "block": 2, "spin_limit": 3, "drop_partial_sums": 4}
+KNOB = {"kernel": 0, "workgroups": 1, "block": 2, "spin_limit": 3, "drop_partial_sums": 4, "xcds": 5}
 KERNEL_CODE = {"stream": 1, "wide": 2, "tile": 3, "expanded": 4}
 
 
 @pytest.fixture
 def knobs():
     """knobs(name, value) on the library's test entry point (name: kernel = stream | wide | tile | expanded, workgroups,
-    block = 256 | 128 | 4 | 384, spin_limit, drop_partial_sums); everything set is cleared again after the test."""
+    block = 256 | 128 | 4 | 384, spin_limit, drop_partial_sums, xcds = 1 | 8); everything set is cleared again after the test."""
     import ctypes
 
     from ttmi import capi

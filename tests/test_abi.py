@@ -156,6 +156,8 @@ def test_every_unit_has_exactly_one_workgroup_and_collectors_come_last(shape, wi
     dispatched first and therefore finish without waiting for anybody is an assumption about the hardware's dispatcher,
     not a guarantee of the programming model; the bounded wait and the error word cover the case that it fails.)"""
     L = _test_entries()
+    L.ttmi_test_wide_workgroup_number.restype = ctypes.c_uint32
+    L.ttmi_test_wide_workgroup_number.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
     out = (ctypes.c_uint32 * 4)()
     L.ttmi_test_stream_decomposition(*shape, wide, out)
     groups, kt, split, workgroups = (int(x) for x in out)
@@ -180,6 +182,20 @@ def test_every_unit_has_exactly_one_workgroup_and_collectors_come_last(shape, wi
             contributors = range(g * split, (g + 1) * split)
             collectors = range((g + 1) * split, (g + 2) * split) if wide else [contributors[-1]]
             assert min(collectors) >= max(contributors) and (not wide or min(collectors) > max(contributors))
+    if split > 1 and wide:
+        # The same kernel with the output groups dealt out to 8 XCDs (hardware index b -> XCD b % 8 + c, number b / 8 there):
+        # the launch has one more round of `split` workgroups per XCD; every (group, part) has exactly one workgroup, all
+        # contributors and collectors of a group share b % 8, i.e. an XCD, and the collectors (the group 8 further on) still
+        # have the higher hardware indices.
+        grid = 8 * (-(-groups // 8) + 1) * split
+        number = [L.ttmi_test_wide_workgroup_number(b, split) for b in range(grid)]
+        assert sorted(number) == list(range(grid))
+        where = {n: b for b, n in enumerate(number)}
+        for g in range(min(groups, 60)):
+            contributors = [where[g * split + part] for part in range(split)]
+            collectors = [where[(g + 8) * split + part] for part in range(split)]
+            assert len({b % 8 for b in contributors + collectors}) == 1
+            assert min(collectors) > max(contributors)
 
 
 def test_library_scratch_grows_geometrically_and_is_never_shrunk():

@@ -158,6 +158,27 @@ def test_any_number_of_workgroups_gives_the_same_bits(oracle, workgroups, m, kno
     check_against_reference(c.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
 
 
+@pytest.mark.parametrize("m,k,n,fmt", [(32, 4544, 18176, BFP8), (32, 4096, 6144, BFP8), (64, 2048, 1024, BFP4), (24, 1024, 288, BFP8)])
+def test_shared_outputs_inside_one_xcd_or_anywhere_give_the_same_bits(oracle, m, k, n, fmt, knobs):
+    """Where consecutive workgroups are known to go to consecutive XCDs, the 128-column kernel places the workgroups that
+    share an output in one XCD and hands partial sums over through that XCD's L2 (plain stores); otherwise through
+    device-scope stores.  The sums are added in the same order either way: the same bits."""
+    a_bits = workloads.activations_bf16(m, k, seed=75)
+    words, w_unpacked = pack_weights(oracle, workloads.weights_f32(k, n, seed=76), fmt)
+    a = bf16_dev(a_bits)
+    knobs("kernel", "wide")
+    placed = [capi.matmul_bfp(a, capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n).clone() for _ in range(3)]
+    knobs("xcds", 1)
+    anywhere = capi.matmul_bfp(a, capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n).clone()
+    knobs("xcds", 8)
+    placed.append(capi.matmul_bfp(a, capi.ROW_MAJOR, words, fmt, 1, 1, m, k, n).clone())
+    torch.cuda.synchronize()
+    capi.device_status()
+    for c in placed:
+        assert torch.equal(c.view(torch.int16), anywhere.view(torch.int16))
+    check_against_reference(anywhere.float().cpu().numpy()[0], workloads.bf16_bits_to_f32(a_bits), w_unpacked, k)
+
+
 def test_caller_workspace(oracle):
     m, k, n = 32, 2048, 256
     a_bits = workloads.activations_bf16(m, k, seed=73)

@@ -49,6 +49,7 @@ struct MatmulDev {
     uint32_t workgroups;     // P
     uint32_t units;          // U = batch * mt * ngroups * kt
     uint32_t split;          // k ranges per output group (>= 1)
+    uint32_t xcds;           // 128-column kernel: 8 when workgroups b and b + 8 are known to run on one XCD (the workgroups that share an output are then placed there), else 1
     int a_tiled, c_tiled, c_f32;
     int c_bfp;               // 128-column kernel only: 0, or the mantissa bits (7 | 3) of a block-float output in TILE layout
 };
@@ -88,6 +89,14 @@ __device__ __forceinline__ void slot_store(float4 *to, const u32x4 v) {
     // inserts the wait states for stores of its own, here the s_nop does it.
     asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(to), "v"(v) : "memory");
 }
+// The same for a reader in the writer's own XCD: the vector L1 writes through, so a plain store puts the data into the
+// XCD's L2, which all its CUs share, and a device-scope load (slot_load_issue) finds it there.  Measured with two
+// workgroups passing a word back and forth: 0.52 us per round trip against 0.78 us with device-scope stores (0.84 us
+// between XCDs); loads of any narrower scope are served from the reader's vector L1 when a line is read a second time.
+__device__ __forceinline__ void slot_store_same_xcd(float4 *to, const u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(to), "v"(v) : "memory");
+}
+
 __device__ __forceinline__ u32x4 slot_load_issue(const float4 *from) {
     u32x4 v;
     asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(from) : "memory");
@@ -465,6 +474,13 @@ constexpr size_t WIDE_SLOT_BYTES = 32 * WIDE_COLS * sizeof(float);
 // MB = 2 is the two-band form for 33 to 127 rows: a unit is one k-tile and column group of the weights against two
 // 32-row bands of the activations, so that the weights are streamed once per 64 rows.  Either way a workgroup keeps
 // X = NB * MB sets of sums (one of NB, MB is 1).
+// 128-column kernel with the output groups dealt out to 8 XCDs: the number (group * split + part) of the workgroup with
+// hardware index b, which runs on XCD (b + c) % 8 and is number b / 8 there: group (b / 8 / split) * 8 + b % 8
+__host__ __device__ __forceinline__ uint32_t wide_workgroup_number(uint32_t b, uint32_t split) {
+    const uint32_t in_xcd = b >> 3, local_group = in_xcd / split;
+    return (local_group * 8 + (b & 7)) * split + (in_xcd - local_group * split);
+}
+
 template <int W, int ACT, int NB, int MB>
 __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wide_kernel(const MatmulDev p) {
     using F = WideFmt<W>;
@@ -489,7 +505,15 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     const uint32_t mant_at = lds_base + wave * WAVE_LDS + wide_mant_at<W>(t_of_lane, fc, q, kh);
 
     // ---- this workgroup's output group and k range ---------------------------------------------------------
-    const uint32_t me = blockIdx.x;
+    // Output groups are dealt out to the XCDs in turn and the workgroups of a group are consecutive inside their XCD: the
+    // hardware's dispatcher hands consecutive workgroups of a launch to consecutive XCDs, so workgroups b and b + 8 run on
+    // the same one (whichever it is: the first workgroup's XCD differs from queue to queue) and the partial sums of an
+    // output never leave the L2 of one XCD.  Were the placement ever different, a collector would not see sums that sit in
+    // another XCD's L2: its bounded wait gives up and the launch is reported, it does not return wrong sums.  `me` numbers
+    // the workgroups group by group; slots and waits below are told in terms of it.
+    const bool in_xcds = p.xcds == 8;
+    const uint32_t me = in_xcds ? wide_workgroup_number(blockIdx.x, p.split) : blockIdx.x;
+    const uint32_t before = in_xcds ? 8 : 1;           // the output group that this workgroup's group collects lies this far back
     const uint32_t og = me / p.split, part = me - og * p.split;
     const uint32_t k_begin = (part * p.kt) / p.split, k_end = ((part + 1) * p.kt) / p.split;
     const uint32_t ng = og % p.ngroups, band = og / p.ngroups;
@@ -777,8 +801,8 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
         return;
     }
     // Outputs shared between `split` workgroups.  Every workgroup publishes its 1024 chunks in its slot; the sums of
-    // output group g are then formed by the `split` workgroups of group g + 1 (after the last group: by `split`
-    // workgroups launched for nothing else), workgroup j of them taking chunks [1024 j / split, 1024 (j + 1) / split)
+    // output group g are then formed by the `split` workgroups of the next group of the same XCD (g + 8; g + 1 where
+    // placement is unknown; after the last group: by `split` workgroups launched for nothing else), workgroup j of them taking chunks [1024 j / split, 1024 (j + 1) / split)
     // from every contributor, in contributor order (so the result does not depend on timing), storing them and putting
     // SLOT_EMPTY back.  The work of collecting is spread evenly, every chunk is read by exactly one thread, and
     // whoever waits, waits for workgroups of lower index only: they were dispatched earlier and wait for nobody
@@ -794,12 +818,13 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
                 u32x4 v;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) v[j] = not_empty(__float_as_uint(mine[nb][r][j]));
-                if (!p.drop_partial_sums) slot_store(slot + r * 64, v);
+                if (p.drop_partial_sums) continue;
+                if (in_xcds) slot_store_same_xcd(slot + r * 64, v); else slot_store(slot + r * 64, v);
             }
         }
     }
-    if (og == 0) return;
-    const uint32_t target = og - 1;
+    if (og < before || og - before >= p.groups) return;
+    const uint32_t target = og - before;
     // ranges of whole lane quads: the four chunks of a face row (16 columns) stay with four neighbouring threads
     const uint32_t lo = ((part * 256u) / p.split) * 4u, hi = (((part + 1) * 256u) / p.split) * 4u;
     const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
@@ -846,7 +871,7 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
             for (int u = 0; u < N; ++u) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) sums[u % X][j] += __uint_as_float(got[u][j]);
-                if (active) slot_store(at + ((uint64_t)c0 * X + u) * 1024, empty);       // ready for the next launch
+                if (active) { if (in_xcds) slot_store_same_xcd(at + ((uint64_t)c0 * X + u) * 1024, empty); else slot_store(at + ((uint64_t)c0 * X + u) * 1024, empty); }       // ready for the next launch
             }
         };
         uint32_t c0 = 0;
@@ -910,6 +935,41 @@ static size_t slot_bytes_needed(const Decomposition &d, bool wide, bool two_sets
     return wide ? (size_t)d.workgroups * WIDE_SLOT_BYTES * (two_sets ? 2 : 1) : (size_t)2 * d.workgroups * SLOT_BYTES;
 }
 
+// Where consecutive workgroups run.  The 128-column kernel keeps the workgroups that share an output in one XCD, which
+// relies on consecutive workgroups going to consecutive XCDs, eight of them: workgroup b to XCD (b + c) % 8 with some c
+// that is the same for the whole launch (observed on MI355X from the null stream, from other streams, back to back,
+// beside a kernel on another stream and in graph replays; c depends on the queue).  A probe launch reads the XCC_ID
+// register of 64 workgroups once per device; any other answer — another part, a partitioned one — selects the
+// device-scope hand-over, which assumes nothing about placement.
+static __device__ uint32_t placement_probe[64];
+__global__ void placement_probe_kernel(uint32_t *out) {
+    uint32_t xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    if (threadIdx.x == 0) out[blockIdx.x] = xcc & 0xfu;
+}
+static std::mutex g_placement_guard;
+static uint32_t g_xcds[64];       // per device, 0 = not asked yet
+
+static int device_xcds(uint32_t *xcds) {
+    int dev = 0;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (dev < 0 || dev >= 64) return fail(TTMI_ERR_UNSUPPORTED, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_placement_guard);
+    if (!g_xcds[dev]) {
+        uint32_t *probe = nullptr;
+        if (int rc = check_hip(hipGetSymbolAddress((void **)&probe, HIP_SYMBOL(placement_probe)), "hipGetSymbolAddress(placement_probe)")) return rc;
+        hipLaunchKernelGGL(placement_probe_kernel, dim3(64), dim3(64), 0, nullptr, probe);
+        if (int rc = check_launch("placement_probe_kernel")) return rc;
+        uint32_t seen[64];
+        if (int rc = check_hip(hipMemcpy(seen, probe, sizeof(seen), hipMemcpyDeviceToHost), "hipMemcpy(placement_probe)")) return rc;
+        bool round_robin = true;
+        for (uint32_t b = 0; b < 64; ++b) round_robin = round_robin && seen[b] == (seen[0] + b) % 8;
+        g_xcds[dev] = round_robin ? 8 : 1;
+    }
+    *xcds = g_xcds[dev];
+    return TTMI_OK;
+}
+
 static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     const Decomposition d = decompose(x.batch, x.m, x.k, x.n, wide, x.b2 != nullptr);
     MatmulDev p{};
@@ -961,10 +1021,18 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     }
     p.spin_limit = knob_or(TTMI_KNOB_SPIN_LIMIT, SLOT_SPIN_LIMIT);
     p.drop_partial_sums = (int)knob_or(TTMI_KNOB_DROP_PARTIAL_SUMS, 0);
+    // 128-column kernel with shared outputs: one more round of `split` workgroups per XCD collects the XCD's last groups
+    p.xcds = 1;
+    if (wide && d.split > 1 && p.error)
+        if (int rc = device_xcds(&p.xcds)) return rc;
+    // dealing the groups out to 8 XCDs leaves some XCDs a group short when their number is no multiple of 8: only where that costs little
+    if (p.xcds == 8 && (((uint32_t)d.groups + 7) / 8) * 8 * 32 > (uint32_t)d.groups * 33) p.xcds = 1;
+    p.xcds = knob_or(TTMI_KNOB_XCDS, p.xcds) == 8 ? p.xcds : 1;      // a test can ask for the placement-agnostic form
+    const uint32_t wide_grid = d.split == 1 ? d.workgroups : p.xcds == 8 ? 8 * (((uint32_t)d.groups + 7) / 8 + 1) * d.split : d.workgroups + d.split;
 #define TTMI_LAUNCH(W, ACT)                                                                                     \
-    if (wide && gated) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 2, 1>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
-    else if (wide && bands2) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 2>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
-    else if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 1>), dim3(d.workgroups + (d.split > 1 ? d.split : 0)), dim3(256), 0, st, p); \
+    if (wide && gated) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 2, 1>), dim3(wide_grid), dim3(256), 0, st, p); \
+    else if (wide && bands2) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 2>), dim3(wide_grid), dim3(256), 0, st, p); \
+    else if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 1>), dim3(wide_grid), dim3(256), 0, st, p); \
     else hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
 #define TTMI_LAUNCH_ACT(W)                                              \
     switch (x.activation) {                                             \
@@ -1153,5 +1221,7 @@ __attribute__((visibility("default"))) void ttmi_test_wide_layout(int mantissa_b
     if (mantissa_bits == 7) wide_layout_of<7>(lane, out); else wide_layout_of<3>(lane, out);
 }
 __attribute__((visibility("default"))) uint32_t ttmi_test_range_start(uint32_t kt, uint32_t split, uint32_t i) { return ttmi::range_start(kt, split, i); }
+// 128-column kernel, output groups dealt out to 8 XCDs: group * split + part of the workgroup with hardware index b
+__attribute__((visibility("default"))) uint32_t ttmi_test_wide_workgroup_number(uint32_t b, uint32_t split) { return ttmi::wide_workgroup_number(b, split); }
 __attribute__((visibility("default"))) uint32_t ttmi_test_workgroup_of(uint32_t kt, uint32_t split, uint32_t unit) { return ttmi::workgroup_of(kt, split, unit); }
 }

@@ -32,7 +32,8 @@ enum {
     TTMI_KNOB_MATMUL_BLOCK = 2,       // block form of the tiled kernels: 256, 128 (eight wavefronts), 4 (128 rows, four wavefronts), 384
     TTMI_KNOB_SPIN_LIMIT = 3,         // polls before a bounded wait gives up
     TTMI_KNOB_DROP_PARTIAL_SUMS = 4,  // producers do not publish their partial sums (so that a wait must give up)
-    TTMI_KNOB_COUNT = 5
+    TTMI_KNOB_XCDS = 5,               // 1: the 128-column kernel assumes nothing about where workgroups run (device-scope hand-over)
+    TTMI_KNOB_COUNT = 6
 };
 bool knob(int which, uint32_t *value);
 uint32_t knob_or(int which, uint32_t fallback);
