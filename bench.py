@@ -291,6 +291,28 @@ def main():
             legs.append(leg)
         return legs, (runs, keep)
 
+    def measured_ceilings():
+        """What this box delivers to kernels that do no arithmetic, with kernels the box already has and the same rotation over
+        more than the Infinity Cache holds: a read-only pass (torch.sum), a copy (torch.mul(src, 1.0, out=dst)) and an empty
+        launch, timed as every leg is.  A roofline fraction can then be read against 8 TB/s and against what the part gives."""
+        n = 128 << 20                                   # 512 MiB of fp32 per buffer
+        bufs = [torch.ones(n, dtype=torch.float32, device="cuda") for _ in range(3)]
+        out = torch.empty(n, dtype=torch.float32, device="cuda")
+        ms_read = time_loop(lambda i: torch.sum(bufs[i % 3]), 12, 3)
+        ms_copy = time_loop(lambda i: torch.mul(bufs[i % 3], 1.0, out=out), 12, 3)
+        # the decode GEMM's own size: 88 MB read per launch, rotated the same way
+        k = 22 << 20
+        ms_read_88mb = time_loop(lambda i: torch.sum(bufs[i % 3][(i % 5) * k:(i % 5 + 1) * k]), 30, 5)
+        del bufs, out
+        torch.cuda.empty_cache()
+        tiny = torch.zeros(64, dtype=torch.float32, device="cuda")
+        ms_launch = time_loop(lambda i: tiny.add_(1.0), 200, 20)
+        return {"measured_read_gbs": round(n * 4 / (ms_read * 1e-3) / 1e9, 1), "measured_copy_gbs": round(2 * n * 4 / (ms_copy * 1e-3) / 1e9, 1),
+                "measured_read_88mb_us": round(ms_read_88mb * 1e3, 2), "measured_read_88mb_gbs": round(k * 4 / (ms_read_88mb * 1e-3) / 1e9, 1),
+                "launch_floor_us": round(ms_launch * 1e3, 2),
+                "how": "torch.sum over 512 MiB (3 buffers rotated), torch.mul(src, 1.0, out=dst) over 512 MiB + 512 MiB, torch.sum over 88 MB slices, "
+                       "a 64-element add_ back to back; HIP events on the launching stream"}
+
     if args.counter_calibration:
         src = torch.ones(64 << 20, dtype=torch.float32, device="cuda")
         dst = torch.empty_like(src)
@@ -447,13 +469,16 @@ def main():
     for leg in (l for wl in order for l in results[wl]):
         leg["roofline"]["traffic"] = measured_traffic.get(leg["workload"])
 
+    note("measured ceilings")
+    ceilings = measured_ceilings()
     line = {
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(total_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic",
         "config": {"workload": WORKLOAD_NAMES[args.workload], "parts": [l["workload"] for l in prim],
                    "note": "weights rotate over distinct copies (>512 MiB) so the Infinity Cache cannot serve them"},
-        "roofline": dict(dominant["roofline"], kernel=dominant["workload"]),
+        "roofline": dict(dominant["roofline"], kernel=dominant["workload"], **{k: v for k, v in ceilings.items() if k != "how"}),
+        "measured_ceilings": ceilings,
         "cpu_baseline": cpu,
         "legs": [l for wl in order for l in results[wl]],
     }

@@ -22,6 +22,7 @@
 //              workgroup that owns the last part (see the kernel).
 #include <hip/hip_runtime.h>
 #include <algorithm>
+#include <cmath>
 #include <stdint.h>
 #include <mutex>
 #include <type_traits>
@@ -1061,8 +1062,28 @@ enum class Kernel { Stream = 1, Wide = 2, Tile = 3, Expanded = 4 };
 static Kernel choose_kernel(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt, bool c_bfp) {
     uint32_t forced;
     if (knob(TTMI_KNOB_MATMUL_KERNEL, &forced) && forced >= 1 && forced <= 4) return (Kernel)forced;
-    if (m >= 512) return Kernel::Expanded;
-    if (m >= 128) return Kernel::Tile;
+    if (m >= 128) {
+        // Tall activations are MFMA-bound when the output has enough blocks for the chip: a 128 x 256 or 256 x 256 block per
+        // workgroup takes about 0.75 us per k-tile, and a GEMM with few columns leaves most CUs without one.  Streaming the
+        // weights once per 64 rows (the two-band form of the 128-column kernel, which cuts the k range to fill the chip)
+        // is then faster, up to surprisingly many rows.  Measured, BFLOAT8_B, one MI355X: [256, 4096] x [4096, 4096] 28 us
+        // against 102 (tiled) and 85 (expanded); [128, 14336] x [14336, 4096] 34 against 331 and 264; [256, 4096] x
+        // [4096, 14336] 54 against 103 and 105; [448, 4544] x [4544, 18176] 138 against 229 and 130; 12 x [384, 1024] x
+        // [1024, 1024] 29.5 against 24.8 (the 384-row kernel).  The estimates below reproduce those within 15 %.
+        const double k_tiles = k / 32, weights = (double)k * n * (b_fmt == TTMI_BFLOAT8_B ? 1.0625 : 0.8);     // BFLOAT4_B: half the bytes, the same instructions
+        const double sets = (double)batch * (((m + 31) / 32 + 1) / 2);
+        const double streamed_us = 8.0 + sets * weights / 4.7e6;
+        double blocked_us;
+        if (m >= 512) {
+            const double blocks = (double)batch * ((m + 255) / 256) * ((n + 255) / 256);
+            blocked_us = 4.0 + (double)k * n * 3.0625 / 6.0e6 + std::ceil(blocks / 256.0) * k_tiles * 0.72;      // expansion pass + bf16 GEMM
+        } else {
+            const double blocks = (double)batch * ((m + 127) / 128) * ((n + 255) / 256);
+            blocked_us = std::ceil(blocks / 256.0) * k_tiles * 0.78;
+        }
+        if (streamed_us < 0.9 * blocked_us) return Kernel::Wide;
+        return m >= 512 ? Kernel::Expanded : Kernel::Tile;
+    }
     // One band of BFP4_B weights whose 64-column groups are one workgroup per CU, with at most 192 KiB of weights each:
     // the 64-column kernel, which then shares no output and has nothing to hand over.  Measured against the 128-column
     // kernel, same box, M = 32, weights rotated through more than the Infinity Cache holds: [4096, 14336] BFP4_B (Mistral's

@@ -73,7 +73,10 @@ DECODE_MISTRAL = [
     ("mistral_up", 32, 4096, 14336, "bfp4_b", None),
     ("mistral_down", 32, 14336, 4096, "bfp4_b", None),
 ]
-PREFILL = [("prefill_ff1", 2048, 4096, 14336, "bfp8_b", None), ("bert_bmm", 384, 1024, 1024, "bfp8_b", 12)]
+# prefill_ff1_256: the same weights under a short prompt (128 <= M < 512 runs on the fused tiled kernel, which expands the
+# weights in LDS; from 512 rows on they are expanded to bf16 once per launch)
+PREFILL = [("prefill_ff1", 2048, 4096, 14336, "bfp8_b", None), ("bert_bmm", 384, 1024, 1024, "bfp8_b", 12),
+           ("prefill_ff1_256", 256, 4096, 14336, "bfp8_b", None)]
 
 
 def gemm_bytes(m: int, k: int, n: int, fmt: str, batch: int | None = None) -> int:
