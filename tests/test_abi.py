@@ -204,6 +204,25 @@ def test_every_unit_has_exactly_one_workgroup_and_collectors_come_last(shape, wi
             assert min(collectors) > max(contributors)
 
 
+def test_division_by_host_known_divisors():
+    """The kernels divide by numbers the host knows (k ranges per output, groups per band) with a multiplication and a shift;
+    exact for every dividend below 2^31 — checked at the edges of every quotient for a spread of divisors."""
+    L = _test_entries()
+    L.ttmi_test_fast_div.restype = ctypes.c_uint32
+    L.ttmi_test_fast_div.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+    import random
+    rng = random.Random(5)
+    divisors = list(range(1, 70)) + [71, 112, 127, 128, 129, 142, 255, 256, 257, 568, 1000, 4095, 4096, 4097, 65535, 65536, 1 << 20, (1 << 26) - 1, (1 << 30) + 1]
+    for d in divisors:
+        top = (1 << 31) - 1
+        samples = {0, 1, d - 1, d, d + 1, top, top - 1, top // d * d, max(top // d * d - 1, 0)}
+        for _ in range(40):
+            q = rng.randrange(0, top // d + 1)
+            samples.update({min(q * d, top), min(q * d + d - 1, top), max(q * d - 1, 0)})
+        for n in samples:
+            assert L.ttmi_test_fast_div(n, d) == n // d, (n, d)
+
+
 def test_library_scratch_grows_geometrically_and_is_never_shrunk():
     """A buffer that is too small is replaced by one of at least twice its size (the old one is retired, not freed: a
     kernel of another host thread may still be about to use it), so the retired buffers of a stream add up to less than

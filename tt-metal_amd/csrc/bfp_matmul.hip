@@ -33,6 +33,31 @@
 
 namespace ttmi {
 
+// n / d for a divisor known on the host and any n < 2^31, without a division on the device (a 32-bit division is some forty
+// instructions in a dependent chain, and the kernels below divide before they can request their first byte):
+// with s = ceil(log2 d) and M = ceil(2^(32+s) / d) = 2^32 + mul, n / d = (mulhi(n, mul) + n) >> s.
+struct FastDiv {
+    uint32_t mul, shift;
+    __host__ __device__ __forceinline__ uint32_t operator()(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return (__umulhi(n, mul) + n) >> shift;
+#else
+        return (uint32_t)((((uint64_t)n * mul) >> 32) + n) >> shift;
+#endif
+    }
+};
+inline FastDiv fast_div(uint32_t d) {
+    FastDiv f{0, 0};
+    if (d <= 1) return f;
+    uint32_t s = 0;
+    while ((1ull << s) < d) ++s;
+    const unsigned __int128 one = 1;
+    const unsigned __int128 m = ((one << (32 + s)) + d - 1) / d;
+    f.mul = (uint32_t)(m - (one << 32));
+    f.shift = s;
+    return f;
+}
+
 struct MatmulDev {
     const uint8_t *a;        // bf16
     const uint8_t *b;        // packed tiles
@@ -50,6 +75,7 @@ struct MatmulDev {
     uint32_t workgroups;     // P
     uint32_t units;          // U = batch * mt * ngroups * kt
     uint32_t split;          // k ranges per output group (>= 1)
+    FastDiv by_split, by_ngroups, by_mt_sets;     // 128-column kernel: divisions by split, ngroups and mt_sets
     uint32_t xcds;           // 128-column kernel: 8 when workgroups b and b + 8 are known to run on one XCD (the workgroups that share an output are then placed there), else 1
     int a_tiled, c_tiled, c_f32;
     int c_bfp;               // 128-column kernel only: 0, or the mantissa bits (7 | 3) of a block-float output in TILE layout
@@ -466,7 +492,7 @@ constexpr int WIDE_COLS = WIDE_TILES * 32;
 constexpr int WEIGHTS_ONCE = 2;     // cache policy of the weight loads: nt (read once, not to displace the activations in L2); measured 0.4 us per launch
 constexpr int WIDE_WGS_PER_CU = TTMI_WIDE_WGS_PER_CU;
 constexpr int WIDE_STAGES = TTMI_WIDE_STAGES;
-constexpr int WIDE_REDUCE_BYTES = WAVES * 32 * 64 * 4;     // every wavefront lays out half of its 64 accumulator registers
+constexpr int WIDE_REDUCE_BYTES = WAVES * 64 * 64 * 4;     // every wavefront lays out the 64 accumulator registers of one set of sums
 constexpr size_t WIDE_SLOT_BYTES = 32 * WIDE_COLS * sizeof(float);
 
 // NB = 2 is the gated form, C = act(A . B) * (A . B2) (silu(x w1) * (x w3) of a gated MLP in one launch): a unit is then
@@ -477,8 +503,8 @@ constexpr size_t WIDE_SLOT_BYTES = 32 * WIDE_COLS * sizeof(float);
 // X = NB * MB sets of sums (one of NB, MB is 1).
 // 128-column kernel with the output groups dealt out to 8 XCDs: the number (group * split + part) of the workgroup with
 // hardware index b, which runs on XCD (b + c) % 8 and is number b / 8 there: group (b / 8 / split) * 8 + b % 8
-__host__ __device__ __forceinline__ uint32_t wide_workgroup_number(uint32_t b, uint32_t split) {
-    const uint32_t in_xcd = b >> 3, local_group = in_xcd / split;
+__host__ __device__ __forceinline__ uint32_t wide_workgroup_number(uint32_t b, uint32_t split, FastDiv by_split) {
+    const uint32_t in_xcd = b >> 3, local_group = by_split(in_xcd);
     return (local_group * 8 + (b & 7)) * split + (in_xcd - local_group * split);
 }
 
@@ -513,12 +539,12 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     // another XCD's L2: its bounded wait gives up and the launch is reported, it does not return wrong sums.  `me` numbers
     // the workgroups group by group; slots and waits below are told in terms of it.
     const bool in_xcds = p.xcds == 8;
-    const uint32_t me = in_xcds ? wide_workgroup_number(blockIdx.x, p.split) : blockIdx.x;
+    const uint32_t me = in_xcds ? wide_workgroup_number(blockIdx.x, p.split, p.by_split) : blockIdx.x;
     const uint32_t before = in_xcds ? 8 : 1;           // the output group that this workgroup's group collects lies this far back
-    const uint32_t og = me / p.split, part = me - og * p.split;
-    const uint32_t k_begin = (part * p.kt) / p.split, k_end = ((part + 1) * p.kt) / p.split;
-    const uint32_t ng = og % p.ngroups, band = og / p.ngroups;
-    const uint32_t mt = (band % p.mt_sets) * MB, bb = band / p.mt_sets;       // first row band of this workgroup
+    const uint32_t og = p.by_split(me), part = me - og * p.split;
+    const uint32_t k_begin = p.by_split(part * p.kt), k_end = p.by_split((part + 1) * p.kt);
+    const uint32_t band = p.by_ngroups(og), ng = og - band * p.ngroups;
+    const uint32_t bb = p.by_mt_sets(band), mt = (band - bb * p.mt_sets) * MB;       // batch slice, first row band of this workgroup
     const uint32_t nt0 = ng * WIDE_TILES;
     const uint32_t n_valid = min((uint32_t)WIDE_TILES, p.nt - nt0);
 
@@ -681,29 +707,25 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     wait_vmcnt<0>();   // nothing in flight any more (already true; also what the build-time ISA check keys on)
     __builtin_amdgcn_sched_barrier(0);   // and nothing of what follows is scheduled in front of it
     // ---- add the four wavefronts' partial sums through LDS ------------------------------------------------------
-    // In two passes (operands j = 0, 1, then 2, 3; 32 KB each) every wavefront writes its accumulator registers as
-    // float4 (acc[j][4q4 .. 4q4+3]); wavefront w then keeps q4 = w: rows 8w + 4kh + r (r = 0..3), columns 4*c32 + j.
+    // One pass per set of sums (64 KB: the ring is empty by now): every wavefront writes its accumulator registers as float4
+    // (acc[j][4q4 .. 4q4+3]); wavefront w then keeps q4 = w: rows 8w + 4kh + r (r = 0..3), columns 4*c32 + j.
     float4 *red = reinterpret_cast<float4 *>(lds);
     float mine[X][4][4];   // [set of sums][r][j]
 #pragma unroll
-    for (int pass = 0; pass < 2 * X; ++pass) {
-        const int nb = pass >> 1;                         // the set of sums of this pass
+    for (int nb = 0; nb < X; ++nb) {
         __syncthreads();
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                const int j = (pass & 1) * 2 + jj;
-                red[(wave * 8 + jj * 4 + q4) * 64 + lane] = make_float4(acc[nb][j][4 * q4], acc[nb][j][4 * q4 + 1], acc[nb][j][4 * q4 + 2], acc[nb][j][4 * q4 + 3]);
-            }
+            for (int q4 = 0; q4 < 4; ++q4)
+                red[(wave * 16 + j * 4 + q4) * 64 + lane] = make_float4(acc[nb][j][4 * q4], acc[nb][j][4 * q4 + 1], acc[nb][j][4 * q4 + 2], acc[nb][j][4 * q4 + 3]);
         __syncthreads();
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj) {
-            const int j = (pass & 1) * 2 + jj;
+        for (int j = 0; j < 4; ++j) {
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
             for (int sw = 0; sw < WAVES; ++sw) {
-                const float4 x = red[(sw * 8 + jj * 4 + wave) * 64 + lane];
+                const float4 x = red[(sw * 16 + j * 4 + wave) * 64 + lane];
                 v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
             }
             mine[nb][0][j] = v.x; mine[nb][1][j] = v.y; mine[nb][2][j] = v.z; mine[nb][3][j] = v.w;
@@ -718,8 +740,8 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     auto store_band = [&](uint32_t group, uint32_t idx, uint32_t mb, const float (&sums)[NB][4]) __attribute__((always_inline)) {
         const uint32_t lane_of = idx & 63, r_of = (idx >> 6) & 3, w_of = idx >> 8;
         const uint32_t c32_of = lane_of & 31, t_of = c32_of >> 3, fc_of = (c32_of >> 2) & 1, q_of = c32_of & 3;
-        const uint32_t band_of = group / p.ngroups, mt_of = (band_of % p.mt_sets) * MB + mb, bb_of = band_of / p.mt_sets;
-        const uint32_t nt_of = (group % p.ngroups) * WIDE_TILES + t_of;
+        const uint32_t band_of = p.by_ngroups(group), bb_of = p.by_mt_sets(band_of), mt_of = (band_of - bb_of * p.mt_sets) * MB + mb;
+        const uint32_t nt_of = (group - band_of * p.ngroups) * WIDE_TILES + t_of;
         const uint32_t row_in_band = w_of * 8 + (lane_of >> 5) * 4 + r_of, row = mt_of * 32 + row_in_band;
         if (nt_of >= p.nt || row >= p.m) return;
         const uint32_t n_col = nt_of * 32 + fc_of * 16 + q_of * 4;           // first of the 4 columns
@@ -827,7 +849,7 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     if (og < before || og - before >= p.groups) return;
     const uint32_t target = og - before;
     // ranges of whole lane quads: the four chunks of a face row (16 columns) stay with four neighbouring threads
-    const uint32_t lo = ((part * 256u) / p.split) * 4u, hi = (((part + 1) * 256u) / p.split) * 4u;
+    const uint32_t lo = p.by_split(part * 256u) * 4u, hi = p.by_split((part + 1) * 256u) * 4u;
     const u32x4 empty = {SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY, SLOT_EMPTY};
     for (uint32_t idx0 = lo; idx0 < hi; idx0 += 256) {
         const bool active = idx0 + threadIdx.x < hi;                       // idle lanes re-read the last chunk and drop it
@@ -980,6 +1002,7 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
     p.mt = d.mt; p.mt_sets = d.mt_sets; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.groups = (uint32_t)d.groups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
     p.split = d.split;
+    p.by_split = fast_div(d.split); p.by_ngroups = fast_div(d.ngroups); p.by_mt_sets = fast_div(d.mt_sets);
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE;
     p.c_f32 = x.c_dtype == TTMI_FLOAT32;
     p.c_bfp = x.c_dtype == TTMI_BFLOAT8_B ? 7 : x.c_dtype == TTMI_BFLOAT4_B ? 3 : 0;
@@ -1243,6 +1266,8 @@ __attribute__((visibility("default"))) void ttmi_test_wide_layout(int mantissa_b
 }
 __attribute__((visibility("default"))) uint32_t ttmi_test_range_start(uint32_t kt, uint32_t split, uint32_t i) { return ttmi::range_start(kt, split, i); }
 // 128-column kernel, output groups dealt out to 8 XCDs: group * split + part of the workgroup with hardware index b
-__attribute__((visibility("default"))) uint32_t ttmi_test_wide_workgroup_number(uint32_t b, uint32_t split) { return ttmi::wide_workgroup_number(b, split); }
+__attribute__((visibility("default"))) uint32_t ttmi_test_wide_workgroup_number(uint32_t b, uint32_t split) { return ttmi::wide_workgroup_number(b, split, ttmi::fast_div(split)); }
+// n / d as the kernels compute it
+__attribute__((visibility("default"))) uint32_t ttmi_test_fast_div(uint32_t n, uint32_t d) { return ttmi::fast_div(d)(n); }
 __attribute__((visibility("default"))) uint32_t ttmi_test_workgroup_of(uint32_t kt, uint32_t split, uint32_t unit) { return ttmi::workgroup_of(kt, split, unit); }
 }
