@@ -149,12 +149,13 @@ TTMI_API size_t ttmi_matmul_bfp_workspace_bytes(uint32_t batch, uint32_t m, uint
  *   c        c_dtype TTMI_BFLOAT16 (round to nearest even) or TTMI_FLOAT32; c_layout as for a.  Or c_dtype TTMI_BFLOAT8_B |
  *            TTMI_BFLOAT4_B with c_layout TTMI_TILE (output_dtype of tt::operations::primary::matmul, bmm_op.hpp:318-346):
  *            packed tiles of the bf16-rounded result with the host packers' arithmetic (what ttmi_typecast_tiles gives for
- *            the bf16 output) — packed in the epilogue of the decode kernel (up to 32 rows), by one more launch otherwise
+ *            the bf16 output), packed in the epilogue of whichever kernel the shape goes to: one launch, no buffer in between
  *   workspace NULL (the library keeps a buffer of its own per device and stream, allocated on first use) or at least
- *            ttmi_matmul_bfp_workspace_bytes() bytes of device memory, 256-byte aligned.  Up to 127 rows it holds
- *            partial sums of workgroups that share an output (a few MB); from 512 rows on the weights expanded to
- *            bf16 (2 bytes per weight; the size query assumes every batch slice has weights of its own, a call with
- *            b_batch == 1 needs only one slice's worth)
+ *            ttmi_matmul_bfp_workspace_bytes() bytes of device memory, 256-byte aligned.  Where the weights are streamed
+ *            (up to 127 rows, and taller activations whose output has too few blocks to fill the chip) it holds partial
+ *            sums of workgroups that share an output (a few MB); where they are expanded to bf16 first (from 512 rows
+ *            on), the expanded weights (2 bytes per weight; the size query assumes every batch slice has weights of its
+ *            own, a call with b_batch == 1 needs only one slice's worth)
  * fp32 accumulation throughout. */
 TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch,
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
@@ -187,9 +188,11 @@ TTMI_API int ttmi_matmul_bfp_gated(const void *a, int a_layout, const uint32_t *
  * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and results as
  * ttmi_matmul_bfp without the workspace pair; the scratch of the kernels lies in a static device array of
  * TTMI_STATIC_SCRATCH_BYTES (16 MiB) that every GPU the library runs on holds until the process ends, so the call
- * allocates nothing (no hipMalloc, hipFree or hipHostMalloc).  Shapes whose scratch does not fit
+ * allocates nothing (no hipMalloc, hipFree or hipHostMalloc; the first call on a device resolves the array's address,
+ * which is when the runtime places the array).  Shapes whose scratch does not fit
  * (ttmi_matmul_bfp_workspace_bytes() > TTMI_STATIC_SCRATCH_BYTES: in practice GEMMs of 512 rows and more, whose weights
- * are expanded to 2 bytes each) are rejected with TTMI_ERR_UNSUPPORTED.  All calls on one GPU share the one array: calls
+ * are expanded to 2 bytes each) are rejected with TTMI_ERR_UNSUPPORTED; every output dtype that ttmi_matmul_bfp takes
+ * is served.  All calls on one GPU share the one array: calls
  * that overlap in time on one GPU (two streams, two host threads) race and give wrong results — keep them on one
  * stream.  A wait that gives up is reported through ttmi_device_status() only if the device's error word already exists
  * (call ttmi_device_status() once beforehand, where allocating is allowed). */

@@ -624,9 +624,9 @@ def test_library_slots_beyond_the_first_launch_are_empty_too():
                                          (1, 256, 128, 256), (1, 512, 64, 160)])
 def test_block_float_output(oracle, out_fmt, fmt, batch, m, k, n):
     """Output dtype BFLOAT8_B / BFLOAT4_B (TILE layout): the words are those that packing the bf16 output of the same GEMM
-    gives (ttmi_typecast_tiles, itself pinned against the oracle's packer) — in the epilogue of the 128-column kernel,
-    stored directly and through the hand-over of partial sums, with a column group that is not full; through a buffer of
-    the library and one more launch for the other kernels — and unpack to the oracle's unpacking of those words."""
+    gives (ttmi_typecast_tiles, itself pinned against the oracle's packer) — packed in the epilogue of whichever kernel the
+    shape goes to, stored directly and through the hand-over of partial sums, with a column group that is not full — and
+    unpack to the oracle's unpacking of those words."""
     a_bits = workloads.activations_bf16(m, k, seed=400, batch=batch)
     words, _ = pack_weights(oracle, workloads.weights_f32(k, n, seed=401), fmt)
     a_tiles = capi.tilize(bf16_dev(a_bits).reshape(batch, m, k))
@@ -641,6 +641,25 @@ def test_block_float_output(oracle, out_fmt, fmt, batch, m, k, n):
     with pytest.raises(RuntimeError, match="TILE layout"):
         capi.check(capi.lib().ttmi_matmul_bfp(a_tiles.data_ptr(), capi.TILE, words.data_ptr(), fmt, batch, 1, m, k, n, None, 0, got.data_ptr(),
                                               capi.ROW_MAJOR, out_fmt, None, 0, None))
+
+
+@pytest.mark.parametrize("out_fmt", [BFP8, BFP4])
+@pytest.mark.parametrize("kernel", ["wide", "tile", "tile256", "tile4waves", "tile384", "expanded"])
+@pytest.mark.parametrize("batch,b_batch,m,k,n", [(2, 2, 384, 96, 288), (1, 1, 128, 1024, 96), (3, 1, 64, 2048, 160)])
+def test_every_kernel_packs_a_block_float_output_in_its_epilogue(oracle, out_fmt, kernel, batch, b_batch, m, k, n, knobs):
+    """No kernel leaves a block-float output to a second launch: forced onto one shape after the other (ragged column groups,
+    batches, shared outputs), each writes the words that packing its own bf16 output gives, and those are the oracle's."""
+    knobs("kernel", "tile" if kernel.startswith("tile") else kernel)
+    if kernel != "tile" and kernel.startswith("tile"):
+        knobs("block", {"tile256": 256, "tile4waves": 4, "tile384": 384}[kernel])
+    a_bits = workloads.activations_bf16(m, k, seed=410, batch=batch)
+    words, _ = pack_weights(oracle, workloads.weights_f32(k, n, seed=411, batch=b_batch), BFP8)
+    a_tiles = capi.tilize(bf16_dev(a_bits).reshape(batch, m, k))
+    bias = bf16_dev(workloads.f32_to_bf16_bits_rne(workloads.normal_tensor((n,), seed=412)))
+    dense = capi.matmul_bfp(a_tiles, capi.TILE, words, BFP8, batch, b_batch, m, k, n, c_layout=capi.TILE, bias=bias, activation=capi.ACT_SILU)
+    got = capi.matmul_bfp(a_tiles, capi.TILE, words, BFP8, batch, b_batch, m, k, n, c_layout=capi.TILE, out_bfp=out_fmt, bias=bias, activation=capi.ACT_SILU)
+    host = oracle.pack_fp32_vec_as_bfp_tiles(out_fmt, dense.float().cpu().numpy().reshape(-1), False)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), host)
 
 
 @pytest.mark.parametrize("batch,b_batch,m,k,n", [(1, 1, 32, 64, 64), (1, 1, 32, 4544, 256), (2, 2, 40, 160, 96), (3, 1, 300, 96, 288), (1, 1, 512, 256, 544)])

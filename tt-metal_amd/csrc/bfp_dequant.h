@@ -379,6 +379,7 @@ struct StoreTarget {
     uint32_t nt0;            // first packed tile column of the group (the group has 1 or 2 tiles)
     float unscale;
     int c_tiled, c_f32;
+    int c_bfp;               // 0, or the mantissa bits (7 | 3) of a block-float output (TILE layout)
 };
 
 template <int ACT, typename Acc, int RB>
@@ -420,6 +421,43 @@ __device__ __forceinline__ void store_wave_part(const Acc (&acc)[RB][2], const S
         }
     }
     if (o.c_f32) return;
+    if (o.c_bfp) {
+        // Block-float output: the bf16 tiles staged above are packed with the host packers' arithmetic (the sums are rounded
+        // to bf16 first, as for a bf16 output).  A lane takes one face row at a time — 16 bf16, 32 bytes of the stage — finds
+        // the shared exponent, and writes 16 (BFLOAT8_B) or 8 (BFLOAT4_B) code bytes and the exponent byte to their places in
+        // the packed tile (64 exponent bytes, then the faces' code rows: tt_metal/common/bfloat8.hpp:102-173).
+        const uint32_t tile_bytes = o.c_bfp == 7 ? 1088u : 576u, row_bytes = o.c_bfp == 7 ? 16u : 8u;
+#pragma unroll
+        for (int it = 0; it < RB * 2; ++it) {
+            const uint32_t fr = it * 64 + lane;                            // face row of the part: 32-row band, tile, face, row
+            const uint32_t rb = fr >> 7, tt = (fr >> 6) & 1, f = (fr >> 4) & 3, r16 = fr & 15;
+            const uint32_t row = o.row0 + rb * 32;
+            if (row >= o.m || tt >= tiles) continue;
+            const uint8_t *from = lds_wave + rb * 4096 + tt * 2048 + f * 512 + ((r16 * 32) ^ (tt * 32 + (f & 1) * 64));
+            const u32x4 lo8 = *reinterpret_cast<const u32x4 *>(from), hi8 = *reinterpret_cast<const u32x4 *>(from + 16);
+            uint32_t bits[16], shared = 0;
+#pragma unroll
+            for (int w2 = 0; w2 < 4; ++w2) {
+                bits[2 * w2] = lo8[w2] << 16; bits[2 * w2 + 1] = lo8[w2] & 0xffff0000u;
+                bits[8 + 2 * w2] = hi8[w2] << 16; bits[8 + 2 * w2 + 1] = hi8[w2] & 0xffff0000u;
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) shared = max(shared, (bits[e] >> 23) & 0xffu);
+            uint8_t *tile = o.c + ((o.slice * mt + (row >> 5)) * o.nt + o.nt0 + tt) * tile_bytes;
+            uint32_t words[4] = {0, 0, 0, 0};
+            if (o.c_bfp == 7) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) words[e >> 2] |= to_code<7>(bits[e], shared) << (8 * (e & 3));
+                *reinterpret_cast<u32x4 *>(tile + 64 + f * 256 + r16 * row_bytes) = u32x4{words[0], words[1], words[2], words[3]};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) words[e >> 3] |= to_code<3>(bits[e], shared) << (4 * (e & 7));
+                *reinterpret_cast<uint2 *>(tile + 64 + f * 128 + r16 * row_bytes) = make_uint2(words[0], words[1]);
+            }
+            tile[f * 16 + r16] = (uint8_t)shared;
+        }
+        return;
+    }
     if (o.c_tiled) {
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {

@@ -1020,7 +1020,8 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
         if (x.workspace_bytes < need) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace of %zu bytes given, %zu needed", x.workspace_bytes, need);
         if (reinterpret_cast<uintptr_t>(x.workspace) & 255u) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: workspace must be 256-byte aligned");
         slots = x.workspace;
-        fill = true;                                // a caller's buffer may hold anything
+        fill = need > x.workspace_empty_bytes;      // a caller's buffer may hold anything, unless it says how much of it is empty slots
+        if (x.workspace_left_empty_bytes) *x.workspace_left_empty_bytes = std::max(need, x.workspace_empty_bytes);      // a launch that completes leaves its slots empty
     } else if (int rc = scratch_get(SCRATCH_SLOTS, st, need, &slots, &fill, &fill_bytes)) {
         // the library's own slots, one buffer per stream: every word is SLOT_EMPTY once filled, and every launch that
         // completes leaves it that way
@@ -1119,7 +1120,7 @@ static Kernel choose_kernel(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, 
     if (m <= 32 && !c_bfp && b_fmt == TTMI_BFLOAT4_B && group_weights <= 192u * 1024u &&
         one_round_of_groups((uint64_t)batch * ((n / 32 + GROUP_TILES - 1) / GROUP_TILES)))
         return Kernel::Stream;
-    return m <= 32 || ((m + 31) / 32) % 2 == 0 ? Kernel::Wide : Kernel::Stream;
+    return m <= 32 || ((m + 31) / 32) % 2 == 0 || c_bfp ? Kernel::Wide : Kernel::Stream;
 }
 
 size_t matmul_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
@@ -1137,8 +1138,8 @@ size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n
     }
     const bool wide = kernel == Kernel::Wide;
     const size_t need = slot_bytes_needed(decompose(batch, m, k, n, wide), wide, two_bands(m, wide, false));
-    // one band in the 64-column kernel: with a block-float output the same shape goes to the 128-column kernel
-    if (!wide && m <= 32) return std::max(need, slot_bytes_needed(decompose(batch, m, k, n, true), true, false));
+    // 64-column kernel: with a block-float output the same shape goes to the 128-column kernel
+    if (!wide) return std::max(need, slot_bytes_needed(decompose(batch, m, k, n, true), true, two_bands(m, true, false)));
     return need;
 }
 
@@ -1146,21 +1147,9 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
     // what an earlier launch on this device has reported (a wait for partial sums that gave up) surfaces here
     if (!x.no_alloc || error_word_if_exists(nullptr, nullptr))
         if (int rc = ttmi_device_status()) return rc;
+    // every kernel but the 64-column one packs a block-float output in its epilogue (choose_kernel keeps that one out of it)
     const bool c_bfp = x.c_dtype == TTMI_BFLOAT8_B || x.c_dtype == TTMI_BFLOAT4_B;
     const Kernel kernel = choose_kernel(x.batch, x.m, x.k, x.n, x.b_fmt, c_bfp);
-    if (c_bfp && kernel != Kernel::Wide) {
-        // Only the 128-column kernel packs in its epilogue.  The others write bf16 tiles into a buffer of the library (one
-        // per stream) and one typecast pass packs them: the same bits, one more launch.
-        if (x.no_alloc) return fail(TTMI_ERR_UNSUPPORTED, "matmul: a block-float output of this shape needs a buffer that this entry point may not allocate");
-        void *tiles = nullptr;
-        bool fresh;
-        const size_t n_tiles = (size_t)x.batch * ((x.m + 31) / 32) * (x.n / 32);
-        if (int rc = scratch_get(SCRATCH_OUTPUT, st, n_tiles * 2048, &tiles, &fresh)) return rc;
-        MatmulArgs y = x;
-        y.c = tiles; y.c_dtype = TTMI_BFLOAT16;
-        if (int rc = matmul_bfp(y, st)) return rc;
-        return codec_typecast_tiles(tiles, TTMI_BFLOAT16, x.c, x.c_dtype, n_tiles, st);
-    }
     switch (kernel) {
         case Kernel::Expanded: return matmul_bfp_expanded(x, st);
         case Kernel::Tile: return matmul_bfp_tiled(x, st);
@@ -1170,19 +1159,10 @@ int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
 }
 
 // bf16 x bf16: the weights are brought into the operand layout of the expanding GEMM's second pass (a re-layout instead of
-// an expansion), whatever the number of rows; a block-float output goes through the library's output buffer.
+// an expansion), whatever the number of rows.
 int matmul_bf16(const MatmulArgs &x, hipStream_t st) {
     if (int rc = ttmi_device_status()) return rc;
-    const bool c_bfp = x.c_dtype == TTMI_BFLOAT8_B || x.c_dtype == TTMI_BFLOAT4_B;
-    if (!c_bfp) return matmul_bfp_expanded(x, st);
-    void *tiles = nullptr;
-    bool fresh;
-    const size_t n_tiles = (size_t)x.batch * ((x.m + 31) / 32) * (x.n / 32);
-    if (int rc = scratch_get(SCRATCH_OUTPUT, st, n_tiles * 2048, &tiles, &fresh)) return rc;
-    MatmulArgs y = x;
-    y.c = tiles; y.c_dtype = TTMI_BFLOAT16;
-    if (int rc = matmul_bfp_expanded(y, st)) return rc;
-    return codec_typecast_tiles(tiles, TTMI_BFLOAT16, x.c, x.c_dtype, n_tiles, st);
+    return matmul_bfp_expanded(x, st);
 }
 
 // c = act(a . b + bias) * (a . b2) in one launch of the 128-column kernel (any number of rows: the weights are streamed
@@ -1202,6 +1182,11 @@ int matmul_bfp_gated(const MatmulArgs &x, hipStream_t st) {
 // ---------------------------------------------------------------------------------------------------------
 static __device__ __align__(256) uint8_t scratch[TTMI_STATIC_SCRATCH_BYTES + 256];      // + 256: stand-in for the error word
 static void *g_scratch_at[64];       // device address of `scratch` per device (the array's name is no device address on the host)
+// How many leading bytes of the array hold nothing but empty partial-sum slots, per device (a launch that shares outputs
+// then needs no fill launch in front of it), as of which generation of the library's slot buffers (a reported give-up
+// invalidates them all).  Kernels that put expanded weights into the array set it back to 0.
+static size_t g_scratch_empty_bytes[64];
+static uint64_t g_scratch_generation[64];
 static std::mutex g_scratch_guard;
 
 static int static_scratch(void **ptr) {
@@ -1231,7 +1216,23 @@ extern "C" int ttmi_matmul_bfp_static(const void *a, int a_layout, const uint32_
         if (int rc = static_scratch(&at)) return rc;
     ttmi::MatmulArgs args{a, a_layout, b, b_fmt, batch, b_batch, m, k, n, bias, activation, c, c_layout, c_dtype, at, need ? (size_t)TTMI_STATIC_SCRATCH_BYTES + 256 : 0};
     args.no_alloc = true;
-    return ttmi::matmul_bfp(args, (hipStream_t)stream);
+    int dev = 0;
+    if (int rc = ttmi::check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    size_t left_empty = 0;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_guard);
+        const uint64_t generation = ttmi::scratch_generation(ttmi::SCRATCH_SLOTS);
+        args.workspace_empty_bytes = g_scratch_generation[dev] == generation ? g_scratch_empty_bytes[dev] : 0;
+        g_scratch_generation[dev] = generation;
+        g_scratch_empty_bytes[dev] = 0;     // until this call has gone through: it may put expanded weights there instead
+    }
+    args.workspace_left_empty_bytes = &left_empty;
+    const int rc = ttmi::matmul_bfp(args, (hipStream_t)stream);
+    if (rc == TTMI_OK && left_empty) {
+        std::lock_guard<std::mutex> lock(g_scratch_guard);
+        g_scratch_empty_bytes[dev] = left_empty;
+    }
+    return rc;
 }
 
 // Test entry points (not declared in include/ttmi.h): the decomposition the host chooses for a shape, and the two index

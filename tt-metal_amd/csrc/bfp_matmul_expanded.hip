@@ -139,6 +139,7 @@ struct ExpandedDev {
     uint32_t kt, nt, groups, tiles_m, tiles_n, tiles_n8;
     float unscale;
     int a_tiled, c_tiled, c_f32;
+    int c_bfp;               // 0, or the mantissa bits (7 | 3) of a block-float output in TILE layout
 };
 
 constexpr int EXP_STAGES = 4;
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(512, 1) void matmul_expanded_kernel(const ExpandedD
     StoreTarget o;
     o.c = p.c; o.bias = p.bias; o.m = p.m; o.n = p.n; o.nt = p.nt; o.slice = bb;
     o.row0 = m0 + wr * 128; o.nt0 = (tn * 4 + wc) * 2;
-    o.unscale = p.unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32;
+    o.unscale = p.unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32; o.c_bfp = p.c_bfp;
     store_wave_part<ACT>(acc, o, lds + wave * 16384, lane);
 }
 
@@ -292,6 +293,7 @@ int matmul_bfp_expanded(const MatmulArgs &x, hipStream_t st) {
     p.tiles_m = (x.m + 255) / 256; p.tiles_n = (x.n + 255) / 256; p.tiles_n8 = (p.tiles_n + 7) / 8;
     p.unscale = x.b_fmt == TTMI_BFLOAT8_B ? Wfmt<7>::unscale : x.b_fmt == TTMI_BFLOAT4_B ? Wfmt<3>::unscale : 1.0f;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE; p.c_f32 = x.c_dtype == TTMI_FLOAT32;
+    p.c_bfp = x.c_dtype == TTMI_BFLOAT8_B ? 7 : x.c_dtype == TTMI_BFLOAT4_B ? 3 : 0;
     const uint64_t blocks = (uint64_t)x.batch * p.tiles_m * p.tiles_n8 * 8;
     const uint64_t items = (uint64_t)x.b_batch * p.kt * p.groups;
     if (blocks > 0x7fffffffull || items > 0x7fffffffull) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: problem too large for one launch");

@@ -39,6 +39,7 @@ struct TileDev {
     uint32_t batch, b_batch, m, k, n;
     uint32_t kt, nt, tiles_m, tiles_n;
     int a_tiled, c_tiled, c_f32;
+    int c_bfp;               // 0, or the mantissa bits (7 | 3) of a block-float output in TILE layout
 };
 
 constexpr int TILE_STAGES = 4;
@@ -258,7 +259,7 @@ __global__ __launch_bounds__(256, 1) void matmul_tile_kernel(const TileDev p) {
     StoreTarget o;
     o.c = p.c; o.bias = p.bias; o.m = p.m; o.n = p.n; o.nt = p.nt; o.slice = bb;
     o.row0 = m0; o.nt0 = nt0;
-    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32;
+    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32; o.c_bfp = p.c_bfp;
     static_assert(MB == 4 && TILE_STAGES * STAGE_BYTES >= 4 * 16384, "the epilogue stages 128 rows x 64 columns per wavefront in the ring");
     store_wave_part<ACT>(acc, o, lds + wave * 16384, lane);
 }
@@ -453,7 +454,7 @@ __global__ __launch_bounds__(512, 1) void matmul_tile8_kernel(const TileDev p) {
     StoreTarget o;
     o.c = p.c; o.bias = p.bias; o.m = p.m; o.n = p.n; o.nt = p.nt; o.slice = bb;
     o.row0 = m0 + wr * 32 * MB; o.nt0 = nt0;
-    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32;
+    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32; o.c_bfp = p.c_bfp;
     static_assert(OPS_BASE + 2 * OPS_BYTES >= 8 * MB * 4096, "staging of the epilogue does not fit into LDS");
     store_wave_part<ACT>(acc, o, lds + wave * (MB * 4096), lane);
 }
@@ -691,7 +692,7 @@ __global__ __launch_bounds__(64 * NW, 1) void matmul_tall_kernel(const TileDev p
     StoreTarget o;
     o.c = p.c; o.bias = p.bias; o.m = p.m; o.n = p.n; o.nt = p.nt; o.slice = bb;
     o.row0 = m0 + wave * 32; o.nt0 = nt0;
-    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32;
+    o.unscale = F::unscale; o.c_tiled = p.c_tiled; o.c_f32 = p.c_f32; o.c_bfp = p.c_bfp;
     static_assert(LDS_BYTES >= NW * 4096, "staging of the epilogue does not fit into LDS");
     store_wave_part<ACT>(acc, o, lds + wave * 4096, lane);
 }
@@ -737,6 +738,7 @@ int matmul_bfp_tiled(const MatmulArgs &x, hipStream_t st) {
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
     p.kt = x.k / 32; p.nt = x.n / 32;
     p.a_tiled = x.a_layout == TTMI_TILE; p.c_tiled = x.c_layout == TTMI_TILE; p.c_f32 = x.c_dtype == TTMI_FLOAT32;
+    p.c_bfp = x.c_dtype == TTMI_BFLOAT8_B ? 7 : x.c_dtype == TTMI_BFLOAT4_B ? 3 : 0;
     // 256-row blocks when they fill the chip, 128-row blocks otherwise (fewer idle CUs, half the accumulators).
     // The test entry point can force a form (TTMI_KNOB_MATMUL_BLOCK): 256, 128 (eight wavefronts), 4 (128 rows, four wavefronts) or 384 (384 x 64).
     const uint32_t tiles_n = (x.n + TILE_COLS - 1) / TILE_COLS;

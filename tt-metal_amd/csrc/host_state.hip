@@ -28,6 +28,7 @@ struct Key {
     }
 };
 std::mutex g_guard;
+std::atomic<uint64_t> g_allocations{0};          // hipMalloc / hipHostMalloc calls this library has made (a test reads it)
 std::map<Key, Buffer> g_live;
 std::vector<void *> g_retired;
 uint64_t g_generation[SCRATCH_KINDS] = {};       // raised by scratch_invalidate: contents of every buffer of that kind are suspect
@@ -50,6 +51,7 @@ int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fr
         const size_t size = scratch_grown_size(b.bytes, bytes);
         void *p = nullptr;
         if (int rc = check_hip(hipMalloc(&p, size), "hipMalloc(library scratch)")) return rc;
+        ++g_allocations;
         if (b.ptr) g_retired.push_back(b.ptr);
         b.ptr = p; b.bytes = size;
         *fresh = true;
@@ -58,6 +60,11 @@ int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fr
     *ptr = b.ptr;
     if (capacity) *capacity = b.bytes;
     return TTMI_OK;
+}
+
+uint64_t scratch_generation(int kind) {
+    std::lock_guard<std::mutex> lock(g_guard);
+    return g_generation[kind];
 }
 
 // after this, scratch_get reports every buffer of that kind as fresh once (its owner initialises it again)
@@ -85,6 +92,7 @@ int error_word(uint32_t **device_ptr, volatile uint32_t **host_ptr) {
     if (!w.host) {
         void *h = nullptr, *d = nullptr;
         if (int rc = check_hip(hipHostMalloc(&h, 64, hipHostMallocMapped), "hipHostMalloc(error word)")) return rc;
+        ++g_allocations;
         *reinterpret_cast<volatile uint32_t *>(h) = 0;
         if (int rc = check_hip(hipHostGetDevicePointer(&d, h, 0), "hipHostGetDevicePointer(error word)")) return rc;
         w.host = reinterpret_cast<volatile uint32_t *>(h);
@@ -152,6 +160,9 @@ int ttmi_device_status(void) {
     scratch_invalidate(SCRATCH_SLOTS);
     return fail(TTMI_ERR_HIP, "a matmul kernel gave up waiting for the partial sums of another workgroup (code %u): its output is invalid", raised);
 }
+
+// Test entry point: how many allocations (device scratch, the pinned error word) the library has made in this process.
+__attribute__((visibility("default"))) uint64_t ttmi_test_allocations(void) { return g_allocations.load(); }
 
 // Test entry point: the size a library buffer of `have` bytes grows to when `need` bytes are asked for.
 __attribute__((visibility("default"))) size_t ttmi_test_scratch_grown_size(size_t have, size_t need) { return scratch_grown_size(have, need); }

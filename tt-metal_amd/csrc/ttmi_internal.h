@@ -15,12 +15,13 @@ int check_launch(const char *what);
 int check_hip(hipError_t e, const char *what);
 
 // ---- host state (host_state.hip) --------------------------------------------------------------------------------------
-enum { SCRATCH_SLOTS = 0, SCRATCH_EXPANDED = 1, SCRATCH_OUTPUT = 2, SCRATCH_KINDS = 3 };
+enum { SCRATCH_SLOTS = 0, SCRATCH_EXPANDED = 1, SCRATCH_KINDS = 2 };
 // The library's own device buffer of at least `bytes` for this purpose on the current device and this stream.  *fresh is
 // set when the contents are undefined (a new buffer, or one invalidated since): the caller initialises ALL of it on `stream`
 // (*capacity bytes: buffers grow geometrically, so a later, larger request may be served without being fresh).
 int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fresh, size_t *capacity = nullptr);
 void scratch_invalidate(int kind);
+uint64_t scratch_generation(int kind);      // raised by scratch_invalidate
 size_t scratch_grown_size(size_t have, size_t need);
 // Device and host address of the current device's error word (either may be null).
 int error_word(uint32_t **device_ptr, volatile uint32_t **host_ptr);
@@ -64,6 +65,8 @@ struct MatmulArgs {
     void *c; int c_layout, c_dtype;
     void *workspace; size_t workspace_bytes;
     const uint32_t *b2 = nullptr;   // gated form (128-column kernel only): c = act(a . b) * (a . b2)
+    size_t workspace_empty_bytes = 0;            // this many leading bytes of the workspace are known to hold nothing but empty slots
+    size_t *workspace_left_empty_bytes = nullptr;   // out: as above, after a launch that keeps its partial sums there (untouched otherwise)
     bool no_alloc = false;          // the call may not allocate: `workspace` is all the scratch there is, its last 256 bytes stand
                                     // in for the error word when the device has none yet
 };
