@@ -51,11 +51,23 @@ TTMI_API const char *ttmi_last_error(void);
 TTMI_API const char *ttmi_version(void);
 
 /* What kernels on the current device have reported since the last query: TTMI_OK, or TTMI_ERR_HIP (message in
- * ttmi_last_error()) when a matmul kernel gave up waiting for another workgroup's partial sums — its output is invalid.
+ * ttmi_last_error()) when a matmul kernel gave up waiting for another workgroup's partial sums — the output of every
+ * matmul launched on this device since the last query is then suspect (launches queued behind the one that gave up ran
+ * on slots it left in disorder).
  * Reads a word of pinned host memory, no synchronisation; the report becomes visible once the kernel has run, and
  * ttmi_matmul_bfp makes the same check on entry.  The reference learns of a stuck kernel from its watcher thread
  * (tt_metal/impl/debug/watcher_server.cpp) or never; there is no call of this kind in it. */
 TTMI_API int ttmi_device_status(void);
+
+/* The library's own device memory.  A matmul called without a workspace takes its scratch — partial-sum slots, or the
+ * weights expanded to bf16 (2 bytes per weight) — from a buffer that the library allocates on first use and keeps, one per
+ * purpose, device and stream (launches on different streams may overlap and never share one); a buffer that has become
+ * too small is replaced by one at least twice its size and kept aside until now.  Nothing is freed while the process runs
+ * unless this is called: it waits for the current device to go idle (hipDeviceSynchronize) and frees every buffer that the
+ * library holds on it, so a caller that has created many streams, or is done with large shapes, gets the memory back; the
+ * next call without a workspace allocates again.  Returns the number of bytes freed through *freed_bytes (may be NULL).
+ * No counterpart in the reference, whose allocator owns all device memory (tt_metal/impl/allocator). */
+TTMI_API int ttmi_release_scratch(size_t *freed_bytes);
 
 /* tt_metal/common/tt_backend_api_types.hpp:109-132 tile_size(DataFormat): bytes of one 32x32 tile
  * (1088 bfloat8_b, 576 bfloat4_b, 2048 bfloat16/uint16, 4096 float32/uint32); 0 for an unknown dtype. */

@@ -27,14 +27,29 @@ KERNEL_CODE = {"stream": 1, "wide": 2, "tile": 3, "expanded": 4}
 
 
 @pytest.fixture
-def knobs():
+def test_library():
+    """The test runs on libttmi_test.so / _ttmi_test: the product sources built with -DTTMI_TEST_HOOKS, which adds the
+    ttmi_test_* entry points (the product library has none of them)."""
+    import tt_lib.tensor
+
+    tt_lib.tensor.use_test_library(True)
+    try:
+        from ttmi import capi
+
+        yield capi.lib()
+    finally:
+        tt_lib.tensor.use_test_library(False)
+
+
+@pytest.fixture
+def knobs(test_library):
     """knobs(name, value) on the library's test entry point (name: kernel = stream | wide | tile | expanded, workgroups,
     block = 256 | 128 | 4 | 384, spin_limit, drop_partial_sums, xcds = 1 | 8); everything set is cleared again after the test."""
     import ctypes
 
     from ttmi import capi
 
-    L = capi.lib()
+    L = test_library
     L.ttmi_test_set_knob.restype = ctypes.c_int
     L.ttmi_test_set_knob.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_int]
     touched = []

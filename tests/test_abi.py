@@ -26,6 +26,21 @@ def test_header_symbols_are_exported():
         assert hasattr(L, n), n
 
 
+def test_the_product_library_has_no_test_hooks():
+    """The ttmi_test_* entry points (forcing a kernel, dropping partial sums ...) exist in libttmi_test.so only."""
+    import subprocess
+
+    from ttmi import capi
+
+    if not os.path.exists(capi.LIB_PATH) or not os.path.exists(capi.LIB_TEST_PATH):
+        pytest.skip("libraries not built")
+    exported = lambda path: {line.split()[-1] for line in subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout.splitlines() if line.strip()}
+    product, test = exported(capi.LIB_PATH), exported(capi.LIB_TEST_PATH)
+    assert not [s for s in product if "ttmi_test" in s]
+    assert {"ttmi_test_set_knob", "ttmi_test_kernel_choice", "ttmi_test_allocations"} <= test
+    assert {s for s in product if s.startswith("ttmi_")} == {s for s in test if s.startswith("ttmi_") and not s.startswith("ttmi_test_")}
+
+
 def test_size_helpers_need_no_gpu():
     from ttmi import capi
 
@@ -100,9 +115,9 @@ def test_missing_library_fails_loudly(monkeypatch):
 def _test_entries():
     from ttmi import capi
 
-    if not os.path.exists(capi.LIB_PATH):
-        pytest.skip("libttmi.so not built")
-    L = capi.lib()
+    if not os.path.exists(capi.LIB_TEST_PATH):
+        pytest.skip("libttmi_test.so not built")
+    L = capi._load(capi.LIB_TEST_PATH)          # the build with the ttmi_test_* entry points; the product library has none
     u32 = ctypes.c_uint32
     L.ttmi_test_stream_decomposition.restype = None
     L.ttmi_test_stream_decomposition.argtypes = [u32, u32, u32, u32, ctypes.c_int, ctypes.POINTER(u32)]
@@ -265,9 +280,7 @@ def test_lds_stage_of_the_wide_kernel(bits, tile_bytes):
     lanes of a load fetch one aligned 64-byte piece of memory (what the vector memory pipe coalesces)."""
     from ttmi import capi
 
-    if not os.path.exists(capi.LIB_PATH):
-        pytest.skip("libttmi.so not built")
-    L = capi.lib()
+    L = _test_entries()
     L.ttmi_test_wide_layout.restype = None
     L.ttmi_test_wide_layout.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_uint32)]
     lanes = []

@@ -7,6 +7,8 @@ subtract the face row's power of two with every weight, so for them the summatio
 |w| of the 16-column face row (check_against_reference(face_row_scale=True), test_face_rows_with_outliers); with weights
 whose face rows hold comparable magnitudes, as everywhere else in this file, they meet the bound above as well.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -567,6 +569,34 @@ def test_a_wait_that_gives_up_is_raised_where_the_result_is_read(oracle, knobs):
         with pytest.raises(RuntimeError, match="gave up waiting"):
             read(bad)
         assert torch.equal(ttnn.to_torch(ttnn.matmul(tx, tw)), good)        # reported once; the slots are refilled
+
+
+def test_library_scratch_can_be_released(oracle, test_library):
+    """ttmi_release_scratch frees what the library holds on the device (buffers per stream, and those it had outgrown) once
+    the device is idle; the next call allocates again and gives the same bits."""
+    m, k, n = 32, 4096, 512
+    a = bf16_dev(workloads.activations_bf16(m, k, seed=124))
+    words, _ = pack_weights(oracle, workloads.weights_f32(k, n, seed=125), BFP8)
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    outs = []
+    for stream in streams:
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            outs.append(capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n))
+    torch.cuda.synchronize()
+    L = capi.lib()
+    L.ttmi_test_allocations.restype = ctypes.c_uint64
+    free_before, made_before = torch.cuda.mem_get_info()[0], L.ttmi_test_allocations()
+    freed = capi.release_scratch()
+    assert freed >= 3 * capi.lib().ttmi_matmul_bfp_workspace_bytes(1, m, k, n, BFP8) > 0       # a buffer per stream, at least
+    assert torch.cuda.mem_get_info()[0] >= free_before + freed // 2                              # back with the device (allocation granularity aside)
+    assert capi.release_scratch() == 0
+    with torch.cuda.stream(streams[0]):
+        again = capi.matmul_bfp(a, capi.ROW_MAJOR, words, BFP8, 1, 1, m, k, n)
+    torch.cuda.synchronize()
+    capi.device_status()
+    assert L.ttmi_test_allocations() > made_before
+    assert all(torch.equal(again.view(torch.int16), c.view(torch.int16)) for c in outs)
 
 
 def test_library_scratch_is_per_stream(oracle):

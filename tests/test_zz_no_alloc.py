@@ -64,7 +64,7 @@ def both_entry_points(fmt, batch, b_batch, m, k, n, seed, bias=False, activation
     assert torch.equal(outs[0], outs[1]), (fmt, batch, m, k, n)
 
 
-def test_static_scratch_matches_the_allocating_entry_point():
+def test_static_scratch_matches_the_allocating_entry_point(test_library):        # the test build: it counts the library's allocations
     # outputs shared between workgroups (partial-sum slots in the static array), first the larger input, then a smaller one
     both_entry_points(BFP8, 1, 1, 32, 4544, 4608, seed=200, layout=capi.TILE)
     both_entry_points(BFP8, 1, 1, 32, 1024, 288, seed=203)

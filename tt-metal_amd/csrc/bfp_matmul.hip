@@ -1045,7 +1045,7 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
         return rc;
     }
     p.spin_limit = knob_or(TTMI_KNOB_SPIN_LIMIT, SLOT_SPIN_LIMIT);
-    p.drop_partial_sums = (int)knob_or(TTMI_KNOB_DROP_PARTIAL_SUMS, 0);
+    p.drop_partial_sums = (int)knob_or(TTMI_KNOB_DROP_PARTIAL_SUMS, 0);      // always 0 in the product library
     // 128-column kernel with shared outputs: one more round of `split` workgroups per XCD collects the XCD's last groups
     p.xcds = 1;
     if (wide && d.split > 1 && p.error)
@@ -1235,6 +1235,7 @@ extern "C" int ttmi_matmul_bfp_static(const void *a, int a_layout, const uint32_
     return rc;
 }
 
+#ifdef TTMI_TEST_HOOKS
 // Test entry points (not declared in include/ttmi.h): the decomposition the host chooses for a shape, and the two index
 // functions the kernels cut the work with, so that their invariants can be checked without a GPU.
 // Test entry point: the LDS stage of the 128-column kernel as its code computes it, for lane `lane` of a wavefront.
@@ -1272,3 +1273,4 @@ __attribute__((visibility("default"))) uint32_t ttmi_test_wide_workgroup_number(
 __attribute__((visibility("default"))) uint32_t ttmi_test_fast_div(uint32_t n, uint32_t d) { return ttmi::fast_div(d)(n); }
 __attribute__((visibility("default"))) uint32_t ttmi_test_workgroup_of(uint32_t kt, uint32_t split, uint32_t unit) { return ttmi::workgroup_of(kt, split, unit); }
 }
+#endif

@@ -30,7 +30,8 @@ struct Key {
 std::mutex g_guard;
 std::atomic<uint64_t> g_allocations{0};          // hipMalloc / hipHostMalloc calls this library has made (a test reads it)
 std::map<Key, Buffer> g_live;
-std::vector<void *> g_retired;
+struct Retired { void *ptr; size_t bytes; int device; };
+std::vector<Retired> g_retired;
 uint64_t g_generation[SCRATCH_KINDS] = {};       // raised by scratch_invalidate: contents of every buffer of that kind are suspect
 }  // namespace
 
@@ -52,7 +53,7 @@ int scratch_get(int kind, hipStream_t stream, size_t bytes, void **ptr, bool *fr
         void *p = nullptr;
         if (int rc = check_hip(hipMalloc(&p, size), "hipMalloc(library scratch)")) return rc;
         ++g_allocations;
-        if (b.ptr) g_retired.push_back(b.ptr);
+        if (b.ptr) g_retired.push_back(Retired{b.ptr, b.bytes, dev});
         b.ptr = p; b.bytes = size;
         *fresh = true;
     }
@@ -115,6 +116,7 @@ bool error_word_if_exists(uint32_t **device_ptr, volatile uint32_t **host_ptr) {
     return true;
 }
 
+#ifdef TTMI_TEST_HOOKS
 // ---------------------------------------------------------------------------------------------------------
 // Test knobs (ttmi_test_set_knob): which kernel, how many workgroups, which block form, the spin limit of the bounded
 // waits, and whether producers keep their partial sums to themselves.  Product code never sets them.
@@ -135,12 +137,15 @@ uint32_t knob_or(int which, uint32_t fallback) {
     return knob(which, &v) ? v : fallback;
 }
 
+#endif
+
 }  // namespace ttmi
 
 using namespace ttmi;
 
 extern "C" {
 
+#ifdef TTMI_TEST_HOOKS
 // Test entry point (not declared in include/ttmi.h): sets knob `which` to `value`, or clears it when `set` is 0.
 __attribute__((visibility("default"))) int ttmi_test_set_knob(int which, uint32_t value, int set) {
     if (which < 0 || which >= TTMI_KNOB_COUNT) return fail(TTMI_ERR_INVALID_ARGUMENT, "unknown test knob %d", which);
@@ -148,6 +153,7 @@ __attribute__((visibility("default"))) int ttmi_test_set_knob(int which, uint32_
     g_knob_set[which].store(set != 0, std::memory_order_relaxed);
     return TTMI_OK;
 }
+#endif
 
 // What a kernel has reported since the last query on the current device: TTMI_OK, or TTMI_ERR_HIP with the message in
 // ttmi_last_error().  Clears the report.
@@ -158,13 +164,42 @@ int ttmi_device_status(void) {
     if (!raised) return TTMI_OK;
     *host = 0;
     scratch_invalidate(SCRATCH_SLOTS);
-    return fail(TTMI_ERR_HIP, "a matmul kernel gave up waiting for the partial sums of another workgroup (code %u): its output is invalid", raised);
+    return fail(TTMI_ERR_HIP, "a matmul kernel gave up waiting for the partial sums of another workgroup (code %u): the output of every matmul "
+                "launched on this device since the last status check is suspect", raised);
 }
 
+int ttmi_release_scratch(size_t *freed_bytes) {
+    int dev = 0;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (int rc = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize")) return rc;      // nothing queued may still be about to use a buffer
+    size_t freed = 0;
+    std::lock_guard<std::mutex> lock(g_guard);
+    for (auto it = g_live.begin(); it != g_live.end();) {
+        if (it->first.device == dev) {
+            if (it->second.ptr) { (void)hipFree(it->second.ptr); freed += it->second.bytes; }
+            it = g_live.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    for (size_t i = 0; i < g_retired.size();) {
+        if (g_retired[i].device == dev) {
+            (void)hipFree(g_retired[i].ptr); freed += g_retired[i].bytes;
+            g_retired[i] = g_retired.back(); g_retired.pop_back();
+        } else {
+            ++i;
+        }
+    }
+    if (freed_bytes) *freed_bytes = freed;
+    return TTMI_OK;
+}
+
+#ifdef TTMI_TEST_HOOKS
 // Test entry point: how many allocations (device scratch, the pinned error word) the library has made in this process.
 __attribute__((visibility("default"))) uint64_t ttmi_test_allocations(void) { return g_allocations.load(); }
 
 // Test entry point: the size a library buffer of `have` bytes grows to when `need` bytes are asked for.
 __attribute__((visibility("default"))) size_t ttmi_test_scratch_grown_size(size_t have, size_t need) { return scratch_grown_size(have, need); }
+#endif
 
 }  // extern "C"

@@ -26,7 +26,8 @@ size_t scratch_grown_size(size_t have, size_t need);
 // Device and host address of the current device's error word (either may be null).
 int error_word(uint32_t **device_ptr, volatile uint32_t **host_ptr);
 bool error_word_if_exists(uint32_t **device_ptr, volatile uint32_t **host_ptr);     // never allocates
-// Knobs of the test entry point ttmi_test_set_knob(which, value, set); product code never sets them.
+// Knobs of the test entry point ttmi_test_set_knob(which, value, set), which only the test build of the library has
+// (-DTTMI_TEST_HOOKS: libttmi_test.so); in the product library every knob reads as unset.
 enum {
     TTMI_KNOB_MATMUL_KERNEL = 0,      // 1 stream (64 columns), 2 wide (128 columns), 3 tiled, 4 expanded
     TTMI_KNOB_MATMUL_WORKGROUPS = 1,  // workgroups the streaming kernels aim for
@@ -36,8 +37,14 @@ enum {
     TTMI_KNOB_XCDS = 5,               // 1: the 128-column kernel assumes nothing about where workgroups run (device-scope hand-over)
     TTMI_KNOB_COUNT = 6
 };
+#ifdef TTMI_TEST_HOOKS
 bool knob(int which, uint32_t *value);
 uint32_t knob_or(int which, uint32_t fallback);
+#else
+// the product library has no knobs and no test entry points: they exist in libttmi_test.so only (build.py)
+inline bool knob(int, uint32_t *) { return false; }
+inline uint32_t knob_or(int, uint32_t fallback) { return fallback; }
+#endif
 
 int codec_pack_chunks(int fmt, const float *src, size_t n_tiles, int row_major_input, uint32_t *dst, hipStream_t st);
 int codec_unpack_chunks(int fmt, const uint32_t *words, size_t n_tiles, int row_major_output, float *dst, hipStream_t st);

@@ -68,7 +68,7 @@ template <typename F> auto unlocked(F &&f) {
 const host::Tensor *optional_tensor(const py::object &t) { return t.is_none() ? nullptr : &py::cast<const host::Tensor &>(t); }
 
 void bind_tensor_layer(py::module_ &m) {
-    py::class_<host::Tensor>(m, "Tensor", "Shape with and without tile padding, data type, layout and a buffer on the host or on a GPU")
+    py::class_<host::Tensor>(m, "Tensor", py::module_local(), "Shape with and without tile padding, data type, layout and a buffer on the host or on a GPU")
         .def_property_readonly("shape", [](const host::Tensor &t) { return py::tuple(py::cast(t.shape)); })
         .def_property_readonly("padded_shape", [](const host::Tensor &t) { return py::tuple(py::cast(t.padded)); })
         .def_property_readonly("dtype", [](const host::Tensor &t) { return (int)t.dtype; })
@@ -182,7 +182,10 @@ void bind_tensor_layer(py::module_ &m) {
     m.def("load_tensor", &host::load_tensor, no_gil);
 }
 
-PYBIND11_MODULE(_ttmi, m) {
+#ifndef TTMI_PYBIND_NAME
+#define TTMI_PYBIND_NAME _ttmi      // the test build (against libttmi_test.so) is _ttmi_test
+#endif
+PYBIND11_MODULE(TTMI_PYBIND_NAME, m) {
     m.doc() = "Block-float tensors of tt-metal / TT-NN on MI355X: the host layer (Tensor and its operations) and the C ABI (include/ttmi.h)";
     bind_tensor_layer(m);
 

@@ -74,16 +74,24 @@ class MemoryConfig:
         return f"MemoryConfig({self.memory_layout.name}, {self.buffer_type.name})"
 
 
-_module = None
+_modules = {}
+_module_name = "_ttmi"
+
+
+def use_test_library(on: bool) -> None:
+    """Tests only: the mirror runs on _ttmi_test / libttmi_test.so (the build with the ttmi_test_* hooks) until switched back.
+    Tensors made under one of the two do not pass to the other."""
+    global _module_name
+    _module_name = "_ttmi_test" if on else "_ttmi"
+    capi.use_test_library(on)
 
 
 def _m():
     """The C++ host layer, with torch installed as its runtime: memory from torch's allocator (flat uint8 tensors own every
     buffer), launches on torch's current stream."""
-    global _module
-    if _module is None:
+    if _module_name not in _modules:
         capi.lib()                                     # fail loudly when the HIP library is not built
-        mod = pybind.module()
+        mod = pybind.module(_module_name)
 
         def allocate(nbytes, device):
             if device < 0:
@@ -91,8 +99,8 @@ def _m():
             return torch.empty(nbytes, dtype=torch.uint8, device=torch.device("cuda", device))
 
         mod.set_runtime(allocate, lambda device: torch.cuda.current_stream(device).cuda_stream, torch.cuda.is_available)
-        _module = mod
-    return _module
+        _modules[_module_name] = mod
+    return _modules[_module_name]
 
 
 class Device:

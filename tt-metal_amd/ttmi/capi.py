@@ -10,6 +10,8 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libttmi.so")
+# the test build of the same sources (-DTTMI_TEST_HOOKS): the product library plus the ttmi_test_* entry points; tests only
+LIB_TEST_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libttmi_test.so")
 
 BFLOAT16, FLOAT32, UINT32, BFLOAT8_B, BFLOAT4_B, UINT16 = 0, 1, 2, 3, 4, 6
 ROW_MAJOR, TILE = 0, 1
@@ -25,19 +27,35 @@ SYMBOLS = (
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
     "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_typecast_tiles", "ttmi_device_status", "ttmi_matmul_bfp_static",
     "ttmi_matmul_bfp_gated_workspace_bytes", "ttmi_matmul_bfp_gated", "ttmi_matmul_bf16_workspace_bytes", "ttmi_matmul_bf16",
+    "ttmi_release_scratch",
 )
 
 _lib = None
+_loaded = {}
+
+
+def use_test_library(on: bool) -> None:
+    """Tests only: every call below goes to libttmi_test.so (the library with the ttmi_test_* hooks) until switched back."""
+    global _lib
+    _lib = None
+    if on:
+        _lib = _load(LIB_TEST_PATH)
 
 
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
+        _lib = _load(LIB_PATH)
+    return _lib
+
+
+def _load(path: str) -> ctypes.CDLL:
+    if path not in _loaded:
+        if not os.path.exists(path):
             raise RuntimeError(
-                f"{LIB_PATH} is not built: run `python tt-metal_amd/build.py` (needs hipcc); there is no CPU fallback"
+                f"{path} is not built: run `python tt-metal_amd/build.py` (needs hipcc); there is no CPU fallback"
             )
-        L = ctypes.CDLL(LIB_PATH)
+        L = ctypes.CDLL(path)
         vp, u32, i32, sz = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int, ctypes.c_size_t
         L.ttmi_last_error.restype = ctypes.c_char_p
         L.ttmi_last_error.argtypes = []
@@ -81,10 +99,12 @@ def lib() -> ctypes.CDLL:
         L.ttmi_typecast_tiles.argtypes = [vp, i32, vp, i32, sz, vp]
         L.ttmi_device_status.restype = i32
         L.ttmi_device_status.argtypes = []
+        L.ttmi_release_scratch.restype = i32
+        L.ttmi_release_scratch.argtypes = [ctypes.POINTER(ctypes.c_size_t)]
         L.ttmi_eltwise_bf16.restype = i32
         L.ttmi_eltwise_bf16.argtypes = [i32, vp, vp, ctypes.c_float, vp, sz, vp]
-        _lib = L
-    return _lib
+        _loaded[path] = L
+    return _loaded[path]
 
 
 def check(status: int) -> None:
@@ -302,6 +322,13 @@ def unpad_tiles(dtype: int, tiles, src_tiles, start_tile, dst_tiles):
     check(lib().ttmi_unpad_tiles(dtype, _dev(tiles.contiguous()), u4(*[int(x) for x in src_tiles]), _dev(out), u4(*[int(x) for x in start_tile]),
                                  u4(*[int(x) for x in dst_tiles]), _stream()))
     return out
+
+
+def release_scratch() -> int:
+    """Frees the library's own device buffers on the current device (after the device has gone idle); returns the bytes freed."""
+    freed = ctypes.c_size_t(0)
+    check(lib().ttmi_release_scratch(ctypes.byref(freed)))
+    return int(freed.value)
 
 
 def device_status() -> None:

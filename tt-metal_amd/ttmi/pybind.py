@@ -7,17 +7,18 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_DIR = os.path.join(os.path.dirname(_HERE), "lib")
-_mod = None
+_mods = {}
 
 
-def module():
-    """Returns the loaded extension module; raises RuntimeError when it has not been built."""
-    global _mod
-    if _mod is None:
-        found = sorted(glob.glob(os.path.join(_LIB_DIR, "_ttmi*.so")))
+def module(name: str = "_ttmi"):
+    """Returns the loaded extension module; raises RuntimeError when it has not been built.  `_ttmi_test` is the same
+    bindings over libttmi_test.so (the library with the test hooks): tests only."""
+    if name not in _mods:
+        found = sorted(glob.glob(os.path.join(_LIB_DIR, name + ".*.so")))
         if not found:
-            raise RuntimeError(f"pybind11 module _ttmi not built in {_LIB_DIR} (run `python tt-metal_amd/build.py`)")
-        spec = importlib.util.spec_from_file_location("_ttmi", found[0])
-        _mod = importlib.util.module_from_spec(spec)
-        spec.loader.exec_module(_mod)
-    return _mod
+            raise RuntimeError(f"pybind11 module {name} not built in {_LIB_DIR} (run `python tt-metal_amd/build.py`)")
+        spec = importlib.util.spec_from_file_location(name, found[0])
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _mods[name] = mod
+    return _mods[name]
