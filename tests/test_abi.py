@@ -138,7 +138,7 @@ def test_kernel_choice_by_shape():
     """Which kernel a GEMM goes to: one band streams in 128-column units, unless its 64-column groups are one workgroup per CU
     (200 to 256 of them) of at most 192 KiB of BFP4_B weights each and the output is not block-float — then the 64-column kernel
     takes it with one workgroup per group and nothing shared; two and four bands in the two-band form, three in 64-column
-    units; from 128 rows on tiled (up to 511 rows) or expanded where the output has blocks enough to fill the chip, else
+    units when the GEMM has more columns than rows of weights; from 128 rows on tiled (up to 511 rows) or expanded where the output has blocks enough to fill the chip, else
     streamed in the two-band form."""
     from ttmi import capi
 
@@ -152,7 +152,7 @@ def test_kernel_choice_by_shape():
              ((1, 32, 4096, 14336, B4, BF16), STREAM), ((1, 32, 4096, 14336, B4, B8), WIDE), ((1, 32, 4096, 14336, B8, BF16), WIDE),
              ((1, 32, 4096, 16384, B4, BF16), STREAM), ((1, 32, 4096, 16448, B4, BF16), WIDE), ((1, 32, 4096, 12736, B4, BF16), WIDE),
              ((1, 32, 14336, 4096, B4, BF16), WIDE), ((2, 20, 1024, 7168, B8, BF16), WIDE), ((2, 20, 1024, 7168, B4, BF16), STREAM), ((1, 32, 8192, 14336, B4, BF16), WIDE), ((1, 64, 4096, 14336, B4, BF16), WIDE),
-             ((1, 96, 4096, 4096, B8, BF16), STREAM), ((1, 2048, 4096, 14336, B8, BF16), EXPANDED),
+             ((1, 96, 4096, 4096, B8, BF16), WIDE), ((1, 96, 4096, 14336, B4, BF16), STREAM), ((1, 96, 14336, 4096, B4, BF16), WIDE), ((1, 2048, 4096, 14336, B8, BF16), EXPANDED),
              # from 128 rows on: blocks of the output where there are enough of them to fill the chip, else the weights are streamed
              ((1, 128, 4096, 4096, B8, BF16), WIDE), ((1, 256, 4096, 14336, B8, BF16), WIDE), ((1, 128, 14336, 4096, B8, BF16), WIDE),
              ((12, 384, 1024, 1024, B8, BF16), TILE), ((1, 256, 512, 32768, B8, BF16), TILE), ((4, 256, 1024, 8192, B8, BF16), TILE),

@@ -78,8 +78,10 @@ def test_sd_matmul(oracle, device, batch_size, channel_a, channel_b, m, k, n, na
     out = ttnn.matmul(a, b, core_grid=ttnn.CoreGrid(x=8, y=8), dtype=ttnn.bfloat16)
     assert out.shape == (batch_size, channel_a, m, n) and out.layout == ttnn.TILE_LAYOUT and out.dtype == ttnn.bfloat16
     got = ttnn.to_torch(out).double()
-    aq = ttnn.to_torch(a).double()
-    bq = ttnn.to_torch(b).double()
+    # the quantised operands come from the CPU oracle (the host sequences of from_torch and to_torch), not from this library
+    quantise = lambda t: torch.from_numpy(oracle.to_torch_bfp_tiles(int(dtype), oracle.from_torch_bfp_tiles(int(dtype), t.float().numpy()), tuple(t.shape))).double()
+    aq, bq = quantise(ta), quantise(tb)
+    assert torch.equal(ttnn.to_torch(a).double(), aq) and torch.equal(ttnn.to_torch(b).double(), bq)
     ref = aq @ bq
     bound = 2.0 ** -8 * ref.abs() + 2.0 * k * 2.0 ** -24 * (aq.abs() @ bq.abs()) + 1e-30
     assert bool(((got - ref).abs() <= bound).all())

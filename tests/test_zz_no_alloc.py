@@ -71,7 +71,7 @@ def test_static_scratch_matches_the_allocating_entry_point(test_library):       
     both_entry_points(BFP4, 2, 2, 24, 2048, 160, seed=206, bias=True, activation=capi.ACT_SILU)
     # two bands of rows per workgroup (two slots each), three bands (64-column kernel), then a single small band again
     both_entry_points(BFP8, 1, 1, 64, 4096, 512, seed=209)
-    both_entry_points(BFP8, 1, 1, 96, 4096, 512, seed=210)
+    both_entry_points(BFP8, 1, 1, 96, 1024, 2048, seed=210)
     both_entry_points(BFP4, 1, 1, 8, 512, 64, seed=212)
     # no scratch at all (fused tiled kernels), a shape whose expanded weights (2 bytes each) fit the array — they overwrite
     # the slots, which the next launch that shares outputs has to find empty again

@@ -1078,8 +1078,10 @@ int matmul_bfp_wide(const MatmulArgs &x, hipStream_t st) { return launch_streami
 // Which kernel a shape goes to.  Up to 127 rows the weights are streamed (HBM-bound): one 32-row band in 128-column units;
 // two or four bands in the two-band form of the same kernel, which streams the weights once per 64 rows (measured at 64
 // rows, TILE layout: 32.8 against 44.1 us for the Falcon h_to_4h shape, 29.8 against 41.4 us for 4h_to_h, no difference for
-// Mistral's shapes); three bands in 64-column units, once per band (the two-band form would compute a fourth band for
-// nothing: 57 against 53 us).  Taller activations are MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows
+// Mistral's shapes); three bands in 64-column units, once per band, when the GEMM has more columns than rows of weights,
+// else in the two-band form, whose fourth band is computed for nothing but which cuts a long k range finer (measured at 96
+// rows, 64-column against two-band: [4544, 18176] BFP8_B 56.5 against 73.2 us, [4096, 14336] BFP4_B 32.0 against 33.7; but
+// [18176, 4544] BFP8_B 58.1 against 54.0, [4096, 4096] BFP8_B 17.6 against 15.6, [14336, 4096] BFP4_B 37.0 against 30.3).  Taller activations are MFMA-bound: the fused tiled kernels up to 511 rows, and from 512 rows
 // on (two or more 256-row blocks share every weight) the weights are expanded to bf16 once and a plain bf16 GEMM follows.
 // The test entry point can force a kernel (TTMI_KNOB_MATMUL_KERNEL).
 enum class Kernel { Stream = 1, Wide = 2, Tile = 3, Expanded = 4 };
@@ -1120,7 +1122,7 @@ static Kernel choose_kernel(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, 
     if (m <= 32 && !c_bfp && b_fmt == TTMI_BFLOAT4_B && group_weights <= 192u * 1024u &&
         one_round_of_groups((uint64_t)batch * ((n / 32 + GROUP_TILES - 1) / GROUP_TILES)))
         return Kernel::Stream;
-    return m <= 32 || ((m + 31) / 32) % 2 == 0 || c_bfp ? Kernel::Wide : Kernel::Stream;
+    return m <= 32 || ((m + 31) / 32) % 2 == 0 || c_bfp || k >= n ? Kernel::Wide : Kernel::Stream;
 }
 
 size_t matmul_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n) {
