@@ -173,6 +173,21 @@ TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int
                     uint32_t m, uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout,
                     int c_dtype, void *workspace, size_t workspace_bytes, void *stream);
 
+/* The same GEMM with block-float ACTIVATIONS (tt_eager/tt_dnn/op_library/bmm/bmm_op.cpp:531,839 accept BFLOAT8_B for input a;
+ * tests/ttnn/unit_tests/operations/test_matmul.py:561-620 multiplies two BFLOAT8_B tensors):
+ *   a        packed BFLOAT8_B tiles, tile (mt, kt) of slice s at index (s*Mt + mt)*Kt + kt; m a multiple of 32
+ * The kernel that streams the weights expands the activations itself — exactly, to the bf16 values ttmi_typecast_tiles gives —
+ * so the result is bit for bit that of ttmi_typecast_tiles(a -> BFLOAT16) followed by ttmi_matmul_bfp, in one launch and
+ * with no bf16 copy of A (Falcon-7B 4h_to_h, M = 32: 23.4 us against 29.6 us for the two calls).  Only that kernel's
+ * one-band form takes them: ttmi_matmul_bfp_ab_supported() says (1 / 0) whether a shape goes there (m == 32 per batch
+ * slice: decode); for other shapes, and for BFLOAT4_B activations, the call returns TTMI_ERR_UNSUPPORTED and the caller
+ * expands A first (one pass over A, as the GEMMs for tall shapes expand the weights in a pass of their own).
+ * Workspace: ttmi_matmul_bfp_workspace_bytes(). */
+TTMI_API int ttmi_matmul_bfp_ab_supported(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int a_fmt, int b_fmt);
+TTMI_API int ttmi_matmul_bfp_ab(const uint32_t *a, int a_fmt, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch, uint32_t m,
+                       uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout, int c_dtype, void *workspace,
+                       size_t workspace_bytes, void *stream);
+
 /* ttnn.matmul / tt_lib.tensor.matmul / bmm with two bf16 operands (ttnn/cpp/ttnn/operations/matmul.hpp:39-42,
  * tt_eager/tt_dnn/op_library/bmm/bmm_op.hpp:388-456):  C[b, m, n] = act(A[b, m, k] . B[(b | 0), k, n] + bias[n]).
  *   b        bf16 in TILE layout (4-face tiles of 2048 bytes, tile (kt, nt) of slice s at index (s*Kt + kt)*Nt + nt), k and n

@@ -741,3 +741,53 @@ def test_face_rows_with_outliers(oracle, fmt, kernel, knobs):
     check_against_reference(c, a, w_ref, k, bf16_out=False, face_row_scale=kernel in ("wide", "stream"))
     ref = a.astype(np.float64) @ w_ref.astype(np.float64)
     assert np.sqrt(((c - ref) ** 2).mean() / (ref ** 2).mean()) < 1e-6
+
+
+@pytest.mark.parametrize("fmt,batch,b_batch,m,k,n", [
+    (BFP8, 1, 1, 32, 4544, 4608), (BFP8, 1, 1, 32, 1024, 288), (BFP4, 1, 1, 32, 4096, 14336), (BFP4, 2, 2, 32, 2048, 160),
+    (BFP8, 3, 1, 32, 512, 96), (BFP4, 1, 1, 32, 14336, 4096), (BFP8, 1, 1, 32, 64, 32)])
+def test_block_float_activations_are_expanded_inside_the_streaming_kernel(oracle, fmt, batch, b_batch, m, k, n):
+    """ttmi_matmul_bfp_ab: packed BFLOAT8_B activations go into the kernel that streams the weights as they are (one band of
+    rows per batch slice: BFP4_B and BFP8_B weights, batches, shared outputs, ragged column groups).  The result is bit for bit
+    what expanding them first (ttmi_typecast_tiles) and calling ttmi_matmul_bfp gives — bf16, fp32 and block-float outputs,
+    bias and activation — and it meets the element-wise bound against a float64 product of the oracle-unpacked operands."""
+    L = capi.lib()
+    assert L.ttmi_matmul_bfp_ab_supported(batch, m, k, n, BFP8, fmt) == 1
+    a_f32 = workloads.bf16_bits_to_f32(workloads.activations_bf16(m, k, seed=600, batch=batch)).reshape(batch, m, k)
+    a_f32 = a_f32 * np.exp2(np.arange(m) % 7 - 3).astype(np.float32)[None, :, None]       # face rows of different exponents
+    a_words = capi.pack_tensor(BFP8, dev(a_f32))
+    a_host = oracle.from_torch_bfp_tiles(BFP8, a_f32)
+    assert np.array_equal(a_words.cpu().numpy().view(np.uint32), a_host)
+    a_q = oracle.to_torch_bfp_tiles(BFP8, a_host, a_f32.shape)
+    w = workloads.weights_f32(k, n, seed=601, batch=b_batch)
+    words, w_q = pack_weights(oracle, w, fmt)
+    w_q = w_q.reshape(b_batch, k, n)
+    a_tiles = capi.typecast_tiles(a_words, BFP8, capi.BFLOAT16)
+    bias = bf16_dev(workloads.f32_to_bf16_bits_rne(workloads.normal_tensor((n,), seed=602)))
+    for kwargs in ({}, {"out_dtype": torch.float32}, {"bias": bias, "activation": capi.ACT_GELU}, {"c_layout": capi.TILE, "out_bfp": BFP8}):
+        kwargs = {"c_layout": capi.TILE, **kwargs}
+        two = capi.matmul_bfp(a_tiles, capi.TILE, words, fmt, batch, b_batch, m, k, n, **kwargs)
+        one = capi.matmul_bfp_ab(a_words, BFP8, words, fmt, batch, b_batch, m, k, n, **kwargs)
+        assert torch.equal(one.view(torch.int16), two.view(torch.int16)), kwargs
+    c = capi.matmul_bfp_ab(a_words, BFP8, words, fmt, batch, b_batch, m, k, n, out_dtype=torch.float32)
+    capi.device_status()
+    for b in range(batch):
+        check_against_reference(c[b].cpu().numpy(), a_q[b], w_q[b if b_batch > 1 else 0], k, bf16_out=False, face_row_scale=True)
+
+
+def test_block_float_activations_where_no_kernel_takes_them():
+    """Shapes that go to the MFMA-bound kernels, and BFLOAT4_B activations: refused with TTMI_ERR_UNSUPPORTED before any
+    launch; the host layer expands such activations first (tests/test_gpu_ttnn.py multiplies two BFLOAT8_B tensors)."""
+    L = capi.lib()
+    one = ctypes.c_void_p(256)
+    assert L.ttmi_matmul_bfp_ab_supported(1, 2048, 4096, 14336, BFP8, BFP8) == 0
+    assert L.ttmi_matmul_bfp_ab_supported(12, 384, 1024, 1024, BFP8, BFP8) == 0
+    assert L.ttmi_matmul_bfp_ab_supported(1, 32, 4096, 4096, BFP4, BFP8) == 0
+    assert L.ttmi_matmul_bfp_ab_supported(1, 40, 4096, 4096, BFP8, BFP8) == 0           # whole tiles of A only
+    assert L.ttmi_matmul_bfp_ab_supported(1, 64, 4096, 4096, BFP8, BFP8) == 0           # one band of rows only
+    assert L.ttmi_matmul_bfp_ab(one, BFP8, one, BFP8, 1, 1, 64, 4096, 4096, None, 0, one, capi.TILE, capi.BFLOAT16, None, 0, None) == 3
+    assert L.ttmi_matmul_bfp_ab(one, BFP8, one, BFP8, 1, 1, 2048, 4096, 14336, None, 0, one, capi.TILE, capi.BFLOAT16, None, 0, None) == 3
+    assert b"ttmi_typecast_tiles" in L.ttmi_last_error()
+    assert L.ttmi_matmul_bfp_ab(one, BFP4, one, BFP8, 1, 1, 32, 4096, 4096, None, 0, one, capi.TILE, capi.BFLOAT16, None, 0, None) == 3
+    assert L.ttmi_matmul_bfp_ab(one, capi.BFLOAT16, one, BFP8, 1, 1, 32, 4096, 4096, None, 0, one, capi.TILE, capi.BFLOAT16, None, 0, None) == 1
+    assert L.ttmi_matmul_bfp_ab(one, BFP8, one, BFP8, 1, 1, 40, 4096, 4096, None, 0, one, capi.ROW_MAJOR, capi.BFLOAT16, None, 0, None) == 1

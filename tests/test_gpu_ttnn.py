@@ -78,6 +78,13 @@ def test_sd_matmul(oracle, device, batch_size, channel_a, channel_b, m, k, n, na
     out = ttnn.matmul(a, b, core_grid=ttnn.CoreGrid(x=8, y=8), dtype=ttnn.bfloat16)
     assert out.shape == (batch_size, channel_a, m, n) and out.layout == ttnn.TILE_LAYOUT and out.dtype == ttnn.bfloat16
     got = ttnn.to_torch(out).double()
+    if m == 32 and name == "bfloat8_b":
+        # one band of rows: the kernel that streams the weights took the packed activations as they are; expanding them
+        # first gives the same bits
+        import tt_lib
+
+        a16 = tt_lib.tensor.typecast(a, ttnn.bfloat16)
+        assert torch.equal(ttnn.to_torch(ttnn.matmul(a16, b, dtype=ttnn.bfloat16)), ttnn.to_torch(out))
     # the quantised operands come from the CPU oracle (the host sequences of from_torch and to_torch), not from this library
     quantise = lambda t: torch.from_numpy(oracle.to_torch_bfp_tiles(int(dtype), oracle.from_torch_bfp_tiles(int(dtype), t.float().numpy()), tuple(t.shape))).double()
     aq, bq = quantise(ta), quantise(tb)

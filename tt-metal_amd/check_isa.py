@@ -6,7 +6,8 @@ value as soon as the load has issued.  That is only safe if it never copies, mov
 between the load and the point where the data is taken over.  This script reads the device assembly of the file,
 builds the control-flow graph of each streaming kernel (64- and 128-column) and propagates the set of registers with a load in flight:
 
-  ring loads   (inline global_load_dwordx4 without sc1: activations in flight across loop iterations) are in flight
+  ring loads   (inline global_load_dwordx4 / global_load_ubyte without sc1: activations, and the exponent bytes of block-float
+               ones, in flight across loop iterations) are in flight
                until an inline `v_mov_b32 vX, vN` reads register N
   slot loads   (inline global_load_dwordx4 ... sc1: partial sums of other workgroups) are in flight until the next
                `s_waitcnt vmcnt(0)`
@@ -121,7 +122,7 @@ def _check_kernel(name, body, problems, release_on_mfma=False):
             if text.startswith("s_waitcnt") and "lgkmcnt(0)" in text:           # every LDS read has returned
                 lds.clear()
             if asm:
-                if text.startswith("global_load_dwordx4"):
+                if text.startswith(("global_load_dwordx4", "global_load_ubyte")):
                     dest = _regs(text.split(",")[0])
                     (slot if "sc1" in text else ring).update(dest)
                 elif text.startswith("ds_read"):

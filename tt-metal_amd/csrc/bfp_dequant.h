@@ -163,6 +163,27 @@ __device__ __forceinline__ bf16x8 weights_operand8(const uint32_t (&words)[8], c
     return __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
 }
 
+// Eight BFLOAT8_B activations of one face row (codes in `w0`, `w1` in memory order, shared exponent byte `e`) as the bf16 A
+// operand of an MFMA, 64 times too large: mantissa x 2^(max(E, 1) - 127), exact (a 7-bit mantissa fits a bf16), where the
+// reference unpacker gives mantissa x 2^(E - 127 - 6) (bfloat8.hpp:229-249).  Whoever stores the sums takes the 64 out.
+template <int LO> __device__ __forceinline__ uint32_t activations_pair(uint32_t w, uint32_t mags, float scale) {
+    const uint32_t v0 = __float_as_uint(byte_to_float<LO>(mags) * scale);
+    const uint32_t v1 = __float_as_uint(byte_to_float<LO + 1>(mags) * scale);
+    const uint32_t both = __builtin_amdgcn_perm(v1, v0, 0x07060302u);                         // the upper halves: exact bf16
+    constexpr uint32_t sign_sel = ((uint32_t)(LO + 1) << 24) | (0x0cu << 16) | ((uint32_t)LO << 8) | 0x0cu;
+    return (__builtin_amdgcn_perm(w, w, sign_sel) & 0x80008000u) | both;
+}
+__device__ __forceinline__ u32x4 activations_operand8(uint32_t w0, uint32_t w1, uint32_t e) {
+    const float scale = row_scale(e & 0xffu);
+    const uint32_t m0 = w0 & 0x7f7f7f7fu, m1 = w1 & 0x7f7f7f7fu;
+    u32x4 out;
+    out[0] = activations_pair<0>(w0, m0, scale);
+    out[1] = activations_pair<2>(w0, m0, scale);
+    out[2] = activations_pair<0>(w1, m1, scale);
+    out[3] = activations_pair<2>(w1, m1, scale);
+    return out;
+}
+
 // Fills `chunk_of[l]` with the global chunk (16 bytes, counted from the start of a 2-tile run) that lands in this
 // lane's slot of direct-to-LDS load l, for the stage layout described at Wfmt.
 template <int W> __device__ __forceinline__ void stage_chunks(int lane, uint32_t (&chunk_of)[Wfmt<W>::loads]) {

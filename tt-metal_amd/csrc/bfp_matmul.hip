@@ -508,16 +508,17 @@ __host__ __device__ __forceinline__ uint32_t wide_workgroup_number(uint32_t b, u
     return (local_group * 8 + (b & 7)) * split + (in_xcd - local_group * split);
 }
 
-template <int W, int ACT, int NB, int MB>
+template <int W, int ACT, int NB, int MB, bool A8 = false>
 __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wide_kernel(const MatmulDev p) {
     using F = WideFmt<W>;
     constexpr int X = NB * MB;
     static_assert(X <= 2, "one of NB, MB is 1");
+    static_assert(!A8 || NB == 1, "block-float activations: one weight matrix");
     constexpr int UNIT_BYTES = NB * F::unit_bytes;     // a stage holds the unit's tiles of every weight matrix
     constexpr int WAVE_LDS = WIDE_STAGES * UNIT_BYTES;
     constexpr int LDS_BYTES = WIDE_REDUCE_BYTES > WAVES * WAVE_LDS ? WIDE_REDUCE_BYTES : WAVES * WAVE_LDS;
     constexpr int NLOAD = F::loads;
-    constexpr int PER = NB * NLOAD + 2 * MB;           // vector-memory requests per unit
+    constexpr int PER = NB * NLOAD + (A8 ? 4 : 2) * MB;   // vector-memory requests per unit
     __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
 
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
@@ -561,19 +562,27 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
     // activations of one unit for this lane: row c32 of the band, k = kt*32 + 16s + 8kh .. + 7 for s = 0, 1;
     // rows past M read row M-1 and are never stored
     // (a second band past the last one repeats the last one and is never stored)
-    const uint8_t *aptr[MB];
+    // Block-float activations (A8: packed BFLOAT8_B tiles): the lane's 8 codes are half of a 16-byte face row — face
+    // 2 (c32 / 16) + s of the tile, row c32 % 16 — which both lanes of the row load whole, and the row's exponent byte
+    // comes by a load of its own (eptr).
+    const uint8_t *aptr[MB], *eptr[MB];
     uint32_t a_second, a_step;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const uint32_t band_mt = min(mt + mb, p.mt - 1);
-        if (p.a_tiled) {
+        eptr[mb] = nullptr;
+        if (A8) {
+            const uint8_t *tile = p.a + (((uint64_t)bb * p.mt + band_mt) * p.kt + k_begin + wave) * 1088;
+            aptr[mb] = tile + 64 + (c32 >> 4) * 512 + (c32 & 15) * 16;
+            eptr[mb] = tile + (c32 >> 4) * 32 + (c32 & 15);
+        } else if (p.a_tiled) {
             aptr[mb] = p.a + (((uint64_t)bb * p.mt + band_mt) * p.kt + k_begin + wave) * 2048 + (c32 >> 4) * 1024 + (c32 & 15) * 32 + kh * 16;
         } else {
             const uint32_t r0 = min(band_mt * 32 + c32, p.m - 1);
             aptr[mb] = p.a + (((uint64_t)bb * p.m + r0) * p.k + (k_begin + wave) * 32 + kh * 8) * 2;
         }
     }
-    if (p.a_tiled) { a_second = 512; a_step = WAVES * 2048; } else { a_second = 32; a_step = WAVES * 64; }
+    if (A8) { a_second = 256; a_step = WAVES * 1088; } else if (p.a_tiled) { a_second = 512; a_step = WAVES * 2048; } else { a_second = 32; a_step = WAVES * 64; }
 
     f32x16 acc[X][4];
 #pragma unroll
@@ -595,6 +604,17 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
                 asm volatile("v_mov_b32 %0, 0" : "=v"(zero));
                 a_ring[s][h][e] = zero;
             }
+    uint32_t e_ring[WIDE_STAGES][2 * MB];               // A8: the exponent bytes of those rows
+    if constexpr (A8) {
+#pragma unroll
+        for (int s = 0; s < WIDE_STAGES; ++s)
+#pragma unroll
+            for (int h = 0; h < 2 * MB; ++h) {
+                uint32_t zero;
+                asm volatile("v_mov_b32 %0, 0" : "=v"(zero));
+                e_ring[s][h] = zero;
+            }
+    }
 
     // Requests one unit: its 4 packed tiles straight into LDS stage S, its activations into a_ring[S] (inline assembly
     // for the loads and their waits, as in the 64-column kernel).
@@ -614,6 +634,11 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
             asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][2 * mb]) : "v"(aptr[mb]) : "memory");
             asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(a_ring[S][2 * mb + 1]) : "v"(aptr[mb] + a_second) : "memory");
             aptr[mb] += a_step;
+            if constexpr (A8) {
+                asm volatile("global_load_ubyte %0, %1, off" : "+v"(e_ring[S][2 * mb]) : "v"(eptr[mb]) : "memory");
+                asm volatile("global_load_ubyte %0, %1, off" : "+v"(e_ring[S][2 * mb + 1]) : "v"(eptr[mb] + 16) : "memory");
+                eptr[mb] += a_step;
+            }
         }
     };
     auto work = [&](auto stage_tag, auto younger_tag, bool refill) __attribute__((always_inline)) {
@@ -622,6 +647,10 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
         if (YOUNGER >= 0) wait_vmcnt<(YOUNGER < 0 ? 0 : YOUNGER) * PER>();   // < 0: the caller has waited
         if constexpr (MB == 2) asm volatile("" : "+v"(a_ring[S][0]), "+v"(a_ring[S][1]), "+v"(a_ring[S][2 * MB - 2]), "+v"(a_ring[S][2 * MB - 1]) :: "memory");
         else asm volatile("" : "+v"(a_ring[S][0]), "+v"(a_ring[S][1]) :: "memory");
+        if constexpr (A8) {
+#pragma unroll
+            for (int s = 0; s < 2 * MB; ++s) asm volatile("" : "+v"(e_ring[S][s]) :: "memory");
+        }
         u32x4 a_now[2 * MB];
 #pragma unroll
         for (int s = 0; s < 2 * MB; ++s)
@@ -631,6 +660,15 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
                 asm volatile("v_mov_b32 %0, %1" : "=v"(moved) : "v"(a_ring[S][s][e]));
                 a_now[s][e] = moved;
             }
+        if constexpr (A8) {
+            // codes and exponent -> 8 exact bf16 values, 64 times the activations (the factor leaves with the sums)
+#pragma unroll
+            for (int s = 0; s < 2 * MB; ++s) {
+                uint32_t exponent;
+                asm volatile("v_mov_b32 %0, %1" : "=v"(exponent) : "v"(e_ring[S][s]));
+                a_now[s] = activations_operand8(kh ? a_now[s][2] : a_now[s][0], kh ? a_now[s][3] : a_now[s][1], exponent);
+            }
+        }
         // hidden-one form (bfp_dequant.h): A.W = 2 (A.hi - A.lo); the subtraction is an MFMA with the negated activations
         u32x4 a_neg[2 * MB];
 #pragma unroll
@@ -748,7 +786,7 @@ __global__ __launch_bounds__(256, NB == 2 ? 1 : WIDE_WGS_PER_CU) void matmul_wid
         float v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            float x = sums[0][j] * decode_unscale<W, MB>();
+            float x = sums[0][j] * (decode_unscale<W, MB>() * (A8 ? 0.015625f : 1.f));
             if (p.bias) x += __uint_as_float((uint32_t)p.bias[n_col + j] << 16);
             v[j] = apply_activation<ACT>(x);
             if (NB == 2) v[j] *= sums[NB - 1][j] * decode_unscale<W, MB>();
@@ -999,6 +1037,8 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     p.a = (const uint8_t *)x.a; p.b = (const uint8_t *)x.b; p.b2 = (const uint8_t *)x.b2; p.bias = (const uint16_t *)x.bias; p.c = (uint8_t *)x.c;
     const bool gated = x.b2 != nullptr;
     if (gated && !wide) return fail(TTMI_ERR_UNSUPPORTED, "matmul: the gated form runs on the 128-column kernel only");
+    const bool a8 = x.a_dtype == TTMI_BFLOAT8_B;
+    if (a8 && !(wide && !gated && x.m <= 32 && x.a_layout == TTMI_TILE)) return fail(TTMI_ERR_UNSUPPORTED, "matmul: this kernel takes no block-float activations");
     p.batch = x.batch; p.b_batch = x.b_batch; p.m = x.m; p.k = x.k; p.n = x.n;
     p.mt = d.mt; p.mt_sets = d.mt_sets; p.kt = d.kt; p.nt = d.nt; p.ngroups = d.ngroups; p.groups = (uint32_t)d.groups; p.workgroups = d.workgroups; p.units = (uint32_t)d.units;
     p.split = d.split;
@@ -1056,6 +1096,7 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     const uint32_t wide_grid = d.split == 1 ? d.workgroups : p.xcds == 8 ? 8 * (((uint32_t)d.groups + 7) / 8 + 1) * d.split : d.workgroups + d.split;
 #define TTMI_LAUNCH(W, ACT)                                                                                     \
     if (wide && gated) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 2, 1>), dim3(wide_grid), dim3(256), 0, st, p); \
+    else if (wide && a8) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 1, true>), dim3(wide_grid), dim3(256), 0, st, p); \
     else if (wide && bands2) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 2>), dim3(wide_grid), dim3(256), 0, st, p); \
     else if (wide) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 1>), dim3(wide_grid), dim3(256), 0, st, p); \
     else hipLaunchKernelGGL((matmul_stream_kernel<W, ACT>), dim3(d.workgroups), dim3(256), 0, st, p)
@@ -1145,13 +1186,23 @@ size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n
     return need;
 }
 
+bool matmul_takes_bfp_activations(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt) {
+    // One band of rows: with two, the expansion of four slabs of activations per unit no longer fits the registers beside
+    // two sets of sums (measured with it: [64, 18176] x [18176, 4544] 45.5 us against 38.3 for expanding A first).
+    return batch && m == 32 && k && n && choose_kernel(batch, m, k, n, b_fmt, true) == Kernel::Wide;
+}
+
 int matmul_bfp(const MatmulArgs &x, hipStream_t st) {
     // what an earlier launch on this device has reported (a wait for partial sums that gave up) surfaces here
     if (!x.no_alloc || error_word_if_exists(nullptr, nullptr))
         if (int rc = ttmi_device_status()) return rc;
     // every kernel but the 64-column one packs a block-float output in its epilogue (choose_kernel keeps that one out of it)
     const bool c_bfp = x.c_dtype == TTMI_BFLOAT8_B || x.c_dtype == TTMI_BFLOAT4_B;
-    const Kernel kernel = choose_kernel(x.batch, x.m, x.k, x.n, x.b_fmt, c_bfp);
+    const bool a8 = x.a_dtype == TTMI_BFLOAT8_B;      // block-float activations: the 128-column kernel alone takes them
+    const Kernel kernel = choose_kernel(x.batch, x.m, x.k, x.n, x.b_fmt, c_bfp || a8);
+    if (a8 && !matmul_takes_bfp_activations(x.batch, x.m, x.k, x.n, x.b_fmt))
+        return fail(TTMI_ERR_UNSUPPORTED, "matmul: block-float activations are taken by the one-band streaming kernel only, which this shape does "
+                    "not go to (ttmi_matmul_bfp_ab_supported): expand them with ttmi_typecast_tiles first");
     switch (kernel) {
         case Kernel::Expanded: return matmul_bfp_expanded(x, st);
         case Kernel::Tile: return matmul_bfp_tiled(x, st);

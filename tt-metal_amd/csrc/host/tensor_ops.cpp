@@ -446,15 +446,21 @@ Tensor matmul(const Tensor &a, const Tensor &b, bool bcast_batch, const Tensor *
     }
     const uint64_t a_elements = (uint64_t)batch_a * m * k, c_elements = (uint64_t)batch_a * m * n;
     // block-float activations are expanded (exactly) to bf16 tiles by one kernel in front of the GEMM; a block-float output is
-    // packed by the GEMM itself — in the epilogue of the decode kernel, behind the others by one more launch inside the
-    // library (the host packers' arithmetic on the bf16-rounded sums: parity with the Tensix packer unpinned)
-    Buffer a_tiles = is_block_float(a.dtype) ? typecast_tiles(a.buffer, a.dtype, DataType::BFLOAT16, a_elements, device) : a.buffer;
+    // packed by the GEMM itself, in its epilogue (the host packers' arithmetic on the bf16-rounded sums: parity with the
+    // Tensix packer unpinned)
+    // ... unless the shape goes to the kernel that streams the weights, which takes BFLOAT8_B activations as they are
+    const bool a_in_kernel = is_block_float(b.dtype) && ttmi_matmul_bfp_ab_supported(batch_a, m, k, n, (int)a.dtype, (int)b.dtype);
+    Buffer a_tiles = is_block_float(a.dtype) && !a_in_kernel ? typecast_tiles(a.buffer, a.dtype, DataType::BFLOAT16, a_elements, device) : a.buffer;
     const bool packed_out = is_block_float(out_dtype);
     const int c_layout = untilize_out ? TTMI_ROW_MAJOR : TTMI_TILE;                                     // bmm_op.cpp:1069
     Buffer c = allocate(packed_out ? storage_bytes(out_dtype, Layout::TILE, {batch_a, m, n}) : c_elements * 2, device);
     if (b.dtype == DataType::BFLOAT16)      // two bf16 operands: not the tuned path (the weights are re-laid-out on every call), but the same surface
         check(ttmi_matmul_bf16(a_tiles.data, TTMI_TILE, b.buffer.data, batch_a, batch_b, m, k, n, bias ? bias_row.data : nullptr, activation, c.data,
                                c_layout, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0, stream_of(device)));
+    else if (a_in_kernel)
+        check(ttmi_matmul_bfp_ab((const uint32_t *)a_tiles.data, (int)a.dtype, (const uint32_t *)b.buffer.data, (int)b.dtype, batch_a, batch_b, m, k, n,
+                                 bias ? bias_row.data : nullptr, activation, c.data, c_layout, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0,
+                                 stream_of(device)));
     else
         check(ttmi_matmul_bfp(a_tiles.data, TTMI_TILE, (const uint32_t *)b.buffer.data, (int)b.dtype, batch_a, batch_b, m, k, n,
                               bias ? bias_row.data : nullptr, activation, c.data, c_layout, packed_out ? (int)out_dtype : TTMI_BFLOAT16, nullptr, 0,

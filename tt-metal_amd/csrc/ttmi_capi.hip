@@ -165,6 +165,22 @@ int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, u
     return matmul_bfp(args, (hipStream_t)stream);
 }
 
+int ttmi_matmul_bfp_ab_supported(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int a_fmt, int b_fmt) {
+    return a_fmt == TTMI_BFLOAT8_B && is_bfp(b_fmt) && (k & 31) == 0 && (n & 31) == 0 && matmul_takes_bfp_activations(batch, m, k, n, b_fmt) ? 1 : 0;
+}
+
+int ttmi_matmul_bfp_ab(const uint32_t *a, int a_fmt, const uint32_t *b, int b_fmt, uint32_t batch, uint32_t b_batch, uint32_t m, uint32_t k,
+                       uint32_t n, const void *bias, int activation, void *c, int c_layout, int c_dtype, void *workspace,
+                       size_t workspace_bytes, void *stream) {
+    if (!is_bfp(a_fmt)) return fail(TTMI_ERR_INVALID_ARGUMENT, "matmul: activation dtype must be BFLOAT8_B or BFLOAT4_B here, got %d", a_fmt);
+    if (int rc = validate_matmul(a, TTMI_TILE, b, b_fmt, batch, b_batch, m, k, n, activation, c, c_layout, c_dtype)) return rc;
+    if (a_fmt != TTMI_BFLOAT8_B)
+        return fail(TTMI_ERR_UNSUPPORTED, "matmul: BFLOAT4_B activations are not taken by any kernel: expand them with ttmi_typecast_tiles first");
+    MatmulArgs args{a, TTMI_TILE, b, b_fmt, batch, b_batch, m, k, n, bias, activation, c, c_layout, c_dtype, workspace, workspace_bytes};
+    args.a_dtype = a_fmt;
+    return matmul_bfp(args, (hipStream_t)stream);
+}
+
 size_t ttmi_matmul_bfp_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt) {
     (void)b_fmt;
     return matmul_gated_workspace_bytes(batch, m, k, n);

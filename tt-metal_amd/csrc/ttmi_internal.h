@@ -74,6 +74,7 @@ struct MatmulArgs {
     const uint32_t *b2 = nullptr;   // gated form (128-column kernel only): c = act(a . b) * (a . b2)
     size_t workspace_empty_bytes = 0;            // this many leading bytes of the workspace are known to hold nothing but empty slots
     size_t *workspace_left_empty_bytes = nullptr;   // out: as above, after a launch that keeps its partial sums there (untouched otherwise)
+    int a_dtype = TTMI_BFLOAT16;    // TTMI_BFLOAT8_B: `a` holds packed tiles (TILE layout), which the 128-column kernel expands itself
     bool no_alloc = false;          // the call may not allocate: `workspace` is all the scratch there is, its last 256 bytes stand
                                     // in for the error word when the device has none yet
 };
@@ -83,6 +84,7 @@ int validate_matmul(const void *a, int a_layout, const uint32_t *b, int b_fmt, u
                     uint32_t n, int activation, const void *c, int c_layout, int c_dtype, bool allow_bf16_weights = false);
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
 int matmul_bfp(const MatmulArgs &args, hipStream_t st);         // streaming kernel (decode shapes) or the tiled one
+bool matmul_takes_bfp_activations(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);   // args.a_dtype = TTMI_BFLOAT8_B goes through for this shape
 int matmul_bfp_stream(const MatmulArgs &args, hipStream_t st);
 int matmul_bfp_wide(const MatmulArgs &args, hipStream_t st);     // the streaming kernel with 128-column units
 size_t matmul_gated_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n);

@@ -27,7 +27,7 @@ SYMBOLS = (
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
     "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_typecast_tiles", "ttmi_device_status", "ttmi_matmul_bfp_static",
     "ttmi_matmul_bfp_gated_workspace_bytes", "ttmi_matmul_bfp_gated", "ttmi_matmul_bf16_workspace_bytes", "ttmi_matmul_bf16",
-    "ttmi_release_scratch",
+    "ttmi_release_scratch", "ttmi_matmul_bfp_ab_supported", "ttmi_matmul_bfp_ab",
 )
 
 _lib = None
@@ -81,6 +81,10 @@ def _load(path: str) -> ctypes.CDLL:
         L.ttmi_matmul_bfp_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
         L.ttmi_matmul_bfp.restype = i32
         L.ttmi_matmul_bfp.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, sz, vp]
+        L.ttmi_matmul_bfp_ab_supported.restype = i32
+        L.ttmi_matmul_bfp_ab_supported.argtypes = [u32, u32, u32, u32, i32, i32]
+        L.ttmi_matmul_bfp_ab.restype = i32
+        L.ttmi_matmul_bfp_ab.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, sz, vp]
         L.ttmi_copy_window.restype = i32
         L.ttmi_copy_window.argtypes = [i32, vp, ctypes.POINTER(u32), vp, ctypes.POINTER(u32), ctypes.POINTER(ctypes.c_int32), ctypes.c_float, vp]
         L.ttmi_unpad_tiles.restype = i32
@@ -234,6 +238,26 @@ def matmul_bfp(a, a_layout: int, b_words, b_fmt: int, batch: int, b_batch: int, 
     if c_layout == ROW_MAJOR:
         return c.view(batch, m, n)
     return c
+
+
+def matmul_bfp_ab(a_words, a_fmt: int, b_words, b_fmt: int, batch: int, b_batch: int, m: int, k: int, n: int, *,
+                  bias=None, activation: int = ACT_NONE, c_layout: int = ROW_MAJOR, out_dtype=None, workspace=None, out_bfp: int | None = None):
+    """Block-float activations (ttmi_matmul_bfp_ab): a_words = packed tiles of A; the rest as for matmul_bfp."""
+    import torch
+
+    out_dtype = out_dtype or torch.bfloat16
+    if out_bfp is not None:
+        c = torch.empty(batch * (m // 32) * (n // 32) * TILE_BYTES[out_bfp] // 4, dtype=torch.int32, device=a_words.device)
+    else:
+        c = torch.empty(batch * m * n, dtype=out_dtype, device=a_words.device)
+    ws_ptr, ws_bytes = None, 0
+    if workspace is not None:
+        ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
+    check(lib().ttmi_matmul_bfp_ab(
+        _dev(a_words), a_fmt, _dev(b_words), b_fmt, batch, b_batch, m, k, n,
+        _dev(bias) if bias is not None else None, activation, _dev(c), c_layout, out_bfp if out_bfp is not None else _torch_dtype_code(c),
+        ws_ptr, ws_bytes, _stream()))
+    return c.view(batch, m, n) if c_layout == ROW_MAJOR else c
 
 
 def matmul_bf16(a, a_layout: int, b_tiles, batch: int, b_batch: int, m: int, k: int, n: int, *, bias=None, activation: int = ACT_NONE,
