@@ -183,7 +183,7 @@ def main():
         L = capi.lib()
         stream = torch.cuda.current_stream().cuda_stream
         m = 32
-        if name == "falcon_mlp_block":
+        if name.startswith("falcon_mlp_block"):
             gemms = [("w1", 4544, 18176, "bfp8_b", capi.ACT_GELU), ("w2", 18176, 4544, "bfp8_b", capi.ACT_NONE)]
         else:
             gemms = [("w1", 4096, 14336, "bfp4_b", capi.ACT_SILU), ("w3", 4096, 14336, "bfp4_b", capi.ACT_NONE),
@@ -203,7 +203,7 @@ def main():
 
         plans = []
         for cp in copies:
-            if name == "falcon_mlp_block":
+            if name.startswith("falcon_mlp_block"):
                 plans.append([("mm", mm(x, cp["w1"], 4544, 18176, "bfp8_b", capi.ACT_GELU, h1)),
                               ("mm", mm(h1, cp["w2"], 18176, 4544, "bfp8_b", capi.ACT_NONE, out))])
             else:
@@ -211,6 +211,16 @@ def main():
                               ("mm", mm(x, cp["w3"], 4096, 14336, "bfp4_b", capi.ACT_NONE, h3)),
                               ("el", (capi.OP_MUL, h1.data_ptr(), h3.data_ptr(), 0.0, h1.data_ptr(), h1.numel(), stream)),
                               ("mm", mm(h1, cp["w2"], 14336, 4096, "bfp4_b", capi.ACT_NONE, out))])
+
+        if name == "falcon_mlp_block_bfp8_act":
+            # the same block with a BFLOAT8_B intermediate, as Falcon-40B's BFLOAT8_B configuration issues it
+            # (models/demos/falcon40b/tt/falcon_mlp.py:97-135, output_dtype of dense_h_to_4h): packed in the epilogue of the
+            # first GEMM, expanded inside the second (ttmi_matmul_bfp_ab) - two launches, no bf16 copy of the intermediate
+            h8 = torch.empty(m * hidden // 1024 * 1088 // 4, dtype=torch.int32, device="cuda")
+            plans = [[("mm", (x.data_ptr(), capi.TILE, cp["w1"].data_ptr(), FMT["bfp8_b"], 1, 1, m, 4544, 18176, None, capi.ACT_GELU, h8.data_ptr(),
+                              capi.TILE, capi.BFLOAT8_B, None, 0, stream)),
+                      ("ab", (h8.data_ptr(), capi.BFLOAT8_B, cp["w2"].data_ptr(), FMT["bfp8_b"], 1, 1, m, 18176, 4544, None, capi.ACT_NONE, out.data_ptr(),
+                              capi.TILE, capi.BFLOAT16, None, 0, stream))] for cp in copies]
 
         if name == "mistral_mlp_block_fused":
             # the same block with silu(x w1) * (x w3) as ONE launch (ttmi_matmul_bfp_gated), then w2: two launches instead of four
@@ -220,10 +230,13 @@ def main():
 
         def run(i):
             for kind, call in plans[i % ncopies]:
-                capi.check(L.ttmi_matmul_bfp(*call) if kind == "mm" else L.ttmi_matmul_bfp_gated(*call) if kind == "gated" else L.ttmi_eltwise_bf16(*call))
+                capi.check(L.ttmi_matmul_bfp(*call) if kind == "mm" else L.ttmi_matmul_bfp_gated(*call) if kind == "gated" else
+                           L.ttmi_matmul_bfp_ab(*call) if kind == "ab" else L.ttmi_eltwise_bf16(*call))
 
         ms = time_loop(run, steps, warmup)
         nbytes = sum(workloads.gemm_bytes(m, g[1], g[2], g[3], None) for g in gemms) + (3 * m * hidden * 2 if len(gemms) == 3 else 0)
+        if name == "falcon_mlp_block_bfp8_act":    # the intermediate is written and read as packed tiles
+            nbytes -= 2 * (m * hidden * 2 - m * hidden // 1024 * 1088)
         if name == "mistral_mlp_block_fused":      # x once, no [32, 14336] intermediates but the one that feeds w2
             nbytes = sum((g[1] // 32) * (g[2] // 32) * 576 for g in gemms) + m * 4096 * 2 + 2 * m * hidden * 2 + m * 4096 * 2
         flops = sum(workloads.gemm_flops(m, g[1], g[2], None) for g in gemms)
@@ -358,6 +371,9 @@ def main():
                     torch.cuda.empty_cache()
                     if wl == "decode_mistral":
                         sub.append(block_leg("mistral_mlp_block_fused", sub_steps, warmup, 4321))
+                        torch.cuda.empty_cache()
+                    if wl == "decode_falcon":
+                        sub.append(block_leg("falcon_mlp_block_bfp8_act", sub_steps, warmup, 4321))
                         torch.cuda.empty_cache()
             results[wl] = sub
         else:

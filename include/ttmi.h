@@ -188,6 +188,14 @@ TTMI_API int ttmi_matmul_bfp_ab(const uint32_t *a, int a_fmt, const uint32_t *b,
                        uint32_t k, uint32_t n, const void *bias, int activation, void *c, int c_layout, int c_dtype, void *workspace,
                        size_t workspace_bytes, void *stream);
 
+/* Which kernel a block-float GEMM of this shape and these dtypes goes to, for whoever reads a profiler trace (no counterpart
+ * in the reference, whose program factories log their choice; needs no GPU):
+ *   out[0]  1 = 64-column streaming kernel, 2 = 128-column streaming kernel, 3 = fused tiled kernels, 4 = expansion + bf16 GEMM
+ *   out[1]  k ranges per output (workgroups that share an output), streaming kernels only, else 0
+ *   out[2]  workgroups launched where the library knows nothing about workgroup placement
+ *   out[3]  workgroups launched on a device whose consecutive workgroups go to 8 XCDs in turn (MI355X) */
+TTMI_API void ttmi_matmul_bfp_plan(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int a_dtype, int b_fmt, int c_dtype, uint32_t out[4]);
+
 /* ttnn.matmul / tt_lib.tensor.matmul / bmm with two bf16 operands (ttnn/cpp/ttnn/operations/matmul.hpp:39-42,
  * tt_eager/tt_dnn/op_library/bmm/bmm_op.hpp:388-456):  C[b, m, n] = act(A[b, m, k] . B[(b | 0), k, n] + bias[n]).
  *   b        bf16 in TILE layout (4-face tiles of 2048 bytes, tile (kt, nt) of slice s at index (s*Kt + kt)*Nt + nt), k and n

@@ -159,6 +159,29 @@ def test_kernel_choice_by_shape():
              ((1, 1024, 4096, 14336, B8, BF16), EXPANDED), ((1, 512, 4096, 1024, B8, BF16), WIDE)]
     for args, want in cases:
         assert L.ttmi_test_kernel_choice(*args) == want, args
+    # the public form of the same answer (for reading profiler traces): kernel, k ranges per output, grid with and without
+    # the output groups dealt out to 8 XCDs
+    L.ttmi_test_stream_decomposition.restype = None
+    L.ttmi_test_stream_decomposition.argtypes = [u32, u32, u32, u32, ctypes.c_int, ctypes.POINTER(u32)]
+    P = capi.lib()
+    for args, want in cases:
+        plan, dec = (u32 * 4)(), (u32 * 4)()
+        P.ttmi_matmul_bfp_plan(*args[:4], BF16, args[4], args[5], plan)
+        assert plan[0] == want, args
+        if want in (STREAM, WIDE):
+            L.ttmi_test_stream_decomposition(*args[:4], int(want == WIDE), dec)
+            groups, split, workgroups = dec[0], dec[2], dec[3]
+            assert plan[1] == split
+            assert plan[2] == (workgroups + (split if want == WIDE and split > 1 else 0))
+            dealt = want == WIDE and split > 1 and ((groups + 7) // 8) * 8 * 32 <= groups * 33
+            assert plan[3] == (8 * ((groups + 7) // 8 + 1) * split if dealt else plan[2]), args
+        else:
+            assert list(plan[1:]) == [0, 0, 0]
+    plan = (u32 * 4)()
+    P.ttmi_matmul_bfp_plan(1, 32, 4544, 18176, BF16, B8, BF16, plan)
+    assert list(plan) == [WIDE, 3, 429, 456]                                # Falcon h_to_4h: 142 groups x 3, + 3 collectors | 8 x 19 x 3
+    P.ttmi_matmul_bfp_plan(1, 32, 4096, 14336, B8, B4, BF16, plan)          # block-float activations keep the 64-column kernel out
+    assert plan[0] == WIDE
     # the one-round form: one workgroup per group, no partial sums, no workspace
     out = (u32 * 4)()
     L.ttmi_test_stream_decomposition(1, 32, 4096, 14336, 0, out)

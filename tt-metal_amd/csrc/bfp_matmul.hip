@@ -1031,6 +1031,13 @@ static int device_xcds(uint32_t *xcds) {
     return TTMI_OK;
 }
 
+// Dealing the output groups out to 8 XCDs leaves some XCDs a group short when their number is no multiple of 8: only where
+// that costs little (at most 1/32 of a round).
+static bool deal_to_xcds(const Decomposition &d) { return d.split > 1 && (((uint32_t)d.groups + 7) / 8) * 8 * 32 <= (uint32_t)d.groups * 33; }
+static uint32_t wide_grid_size(const Decomposition &d, bool in_xcds) {
+    return d.split == 1 ? d.workgroups : in_xcds ? 8 * (((uint32_t)d.groups + 7) / 8 + 1) * d.split : d.workgroups + d.split;
+}
+
 static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     const Decomposition d = decompose(x.batch, x.m, x.k, x.n, wide, x.b2 != nullptr);
     MatmulDev p{};
@@ -1090,10 +1097,9 @@ static int launch_streaming(const MatmulArgs &x, hipStream_t st, bool wide) {
     p.xcds = 1;
     if (wide && d.split > 1 && p.error)
         if (int rc = device_xcds(&p.xcds)) return rc;
-    // dealing the groups out to 8 XCDs leaves some XCDs a group short when their number is no multiple of 8: only where that costs little
-    if (p.xcds == 8 && (((uint32_t)d.groups + 7) / 8) * 8 * 32 > (uint32_t)d.groups * 33) p.xcds = 1;
+    if (p.xcds == 8 && !deal_to_xcds(d)) p.xcds = 1;
     p.xcds = knob_or(TTMI_KNOB_XCDS, p.xcds) == 8 ? p.xcds : 1;      // a test can ask for the placement-agnostic form
-    const uint32_t wide_grid = d.split == 1 ? d.workgroups : p.xcds == 8 ? 8 * (((uint32_t)d.groups + 7) / 8 + 1) * d.split : d.workgroups + d.split;
+    const uint32_t wide_grid = wide_grid_size(d, p.xcds == 8);
 #define TTMI_LAUNCH(W, ACT)                                                                                     \
     if (wide && gated) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 2, 1>), dim3(wide_grid), dim3(256), 0, st, p); \
     else if (wide && a8) hipLaunchKernelGGL((matmul_wide_kernel<W, ACT, 1, 1, true>), dim3(wide_grid), dim3(256), 0, st, p); \
@@ -1184,6 +1190,20 @@ size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n
     // 64-column kernel: with a block-float output the same shape goes to the 128-column kernel
     if (!wide) return std::max(need, slot_bytes_needed(decompose(batch, m, k, n, true), true, two_bands(m, true, false)));
     return need;
+}
+
+// What a shape gets: the kernel, the k ranges per output and the grid (for reading profiler output; no GPU needed).
+void matmul_plan(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt, bool a_or_c_bfp, uint32_t out[4]) {
+    out[0] = out[1] = out[2] = out[3] = 0;
+    if (!batch || !m || !k || !n) return;
+    const Kernel kernel = choose_kernel(batch, m, k, n, b_fmt, a_or_c_bfp);
+    out[0] = (uint32_t)kernel;
+    if (kernel != Kernel::Wide && kernel != Kernel::Stream) return;
+    const bool wide = kernel == Kernel::Wide;
+    const Decomposition d = decompose(batch, m, k, n, wide);
+    out[1] = d.split;
+    out[2] = wide ? wide_grid_size(d, false) : d.workgroups;
+    out[3] = wide && deal_to_xcds(d) ? wide_grid_size(d, true) : out[2];
 }
 
 bool matmul_takes_bfp_activations(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt) {

@@ -165,6 +165,10 @@ int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int b_fmt, u
     return matmul_bfp(args, (hipStream_t)stream);
 }
 
+void ttmi_matmul_bfp_plan(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int a_dtype, int b_fmt, int c_dtype, uint32_t out[4]) {
+    matmul_plan(batch, m, k, n, b_fmt, is_bfp(a_dtype) || is_bfp(c_dtype), out);
+}
+
 int ttmi_matmul_bfp_ab_supported(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int a_fmt, int b_fmt) {
     return a_fmt == TTMI_BFLOAT8_B && is_bfp(b_fmt) && (k & 31) == 0 && (n & 31) == 0 && matmul_takes_bfp_activations(batch, m, k, n, b_fmt) ? 1 : 0;
 }

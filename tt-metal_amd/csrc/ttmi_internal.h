@@ -84,6 +84,7 @@ int validate_matmul(const void *a, int a_layout, const uint32_t *b, int b_fmt, u
                     uint32_t n, int activation, const void *c, int c_layout, int c_dtype, bool allow_bf16_weights = false);
 size_t matmul_workspace_bytes(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);
 int matmul_bfp(const MatmulArgs &args, hipStream_t st);         // streaming kernel (decode shapes) or the tiled one
+void matmul_plan(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt, bool a_or_c_bfp, uint32_t out[4]);
 bool matmul_takes_bfp_activations(uint32_t batch, uint32_t m, uint32_t k, uint32_t n, int b_fmt);   // args.a_dtype = TTMI_BFLOAT8_B goes through for this shape
 int matmul_bfp_stream(const MatmulArgs &args, hipStream_t st);
 int matmul_bfp_wide(const MatmulArgs &args, hipStream_t st);     // the streaming kernel with 128-column units

@@ -27,7 +27,7 @@ SYMBOLS = (
     "ttmi_tilize", "ttmi_untilize", "ttmi_matmul_bfp_workspace_bytes", "ttmi_matmul_bfp",
     "ttmi_eltwise_bf16", "ttmi_copy_window", "ttmi_unpad_tiles", "ttmi_typecast_tiles", "ttmi_device_status", "ttmi_matmul_bfp_static",
     "ttmi_matmul_bfp_gated_workspace_bytes", "ttmi_matmul_bfp_gated", "ttmi_matmul_bf16_workspace_bytes", "ttmi_matmul_bf16",
-    "ttmi_release_scratch", "ttmi_matmul_bfp_ab_supported", "ttmi_matmul_bfp_ab",
+    "ttmi_release_scratch", "ttmi_matmul_bfp_ab_supported", "ttmi_matmul_bfp_ab", "ttmi_matmul_bfp_plan",
 )
 
 _lib = None
@@ -81,6 +81,8 @@ def _load(path: str) -> ctypes.CDLL:
         L.ttmi_matmul_bfp_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
         L.ttmi_matmul_bfp.restype = i32
         L.ttmi_matmul_bfp.argtypes = [vp, i32, vp, i32, u32, u32, u32, u32, u32, vp, i32, vp, i32, i32, vp, sz, vp]
+        L.ttmi_matmul_bfp_plan.restype = None
+        L.ttmi_matmul_bfp_plan.argtypes = [u32, u32, u32, u32, i32, i32, i32, ctypes.POINTER(u32)]
         L.ttmi_matmul_bfp_ab_supported.restype = i32
         L.ttmi_matmul_bfp_ab_supported.argtypes = [u32, u32, u32, u32, i32, i32]
         L.ttmi_matmul_bfp_ab.restype = i32

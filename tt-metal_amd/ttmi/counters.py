@@ -56,23 +56,15 @@ def leg_kernels():
     from . import capi, workloads
 
     L = capi.lib()
-    u32 = ctypes.c_uint32
-    L.ttmi_test_stream_decomposition.restype = None
-    L.ttmi_test_stream_decomposition.argtypes = [u32, u32, u32, u32, ctypes.c_int, ctypes.POINTER(u32)]
     legs = {}
-    L.ttmi_test_kernel_choice.restype = ctypes.c_int
-    L.ttmi_test_kernel_choice.argtypes = [u32, u32, u32, u32, ctypes.c_int, ctypes.c_int]
     for name, m, k, n, fmt, batch in workloads.DECODE_FALCON + workloads.DECODE_MISTRAL:
-        out = (u32 * 4)()
-        wide = L.ttmi_test_kernel_choice(batch or 1, m, k, n, capi.BFLOAT8_B if fmt == "bfp8_b" else capi.BFLOAT4_B, capi.BFLOAT16) == 2
-        L.ttmi_test_stream_decomposition(batch or 1, m, k, n, int(wide), out)
-        split, workgroups = int(out[2]), int(out[3])
+        plan = (ctypes.c_uint32 * 4)()
+        L.ttmi_matmul_bfp_plan(batch or 1, m, k, n, capi.BFLOAT16, capi.BFLOAT8_B if fmt == "bfp8_b" else capi.BFLOAT4_B, capi.BFLOAT16, plan)
         w = 7 if fmt == "bfp8_b" else 3
-        if wide:
-            legs[name] = [(f"matmul_wide_kernel<{w}, 0, 1, 1>", workgroups + (split if split > 1 else 0))]
-        else:
-            legs[name] = [(f"matmul_stream_kernel<{w}, 0>", workgroups)]
+        # the grid of an MI355X (output groups dealt out to its XCDs)
+        legs[name] = [(f"matmul_wide_kernel<{w}, 0, 1, 1, false>" if plan[0] == 2 else f"matmul_stream_kernel<{w}, 0>", int(plan[3]))]
     legs["prefill_ff1"] = [("expand_kernel<7>", None), ("matmul_expanded_kernel<0>", None)]
+    legs["prefill_ff1_256"] = [("matmul_wide_kernel<7, 0, 1, 2, false>", None)]
     legs["bert_bmm"] = [("matmul_tall_kernel<7, 0", None)]
     legs["pack_bfp4_4k_pack"] = [("pack_whole_kernel<3,", None)]
     legs["pack_bfp4_4k_unpack"] = [("unpack_whole_kernel<3,", None)]
@@ -99,14 +91,17 @@ def traffic_lines(fetch_csv: str, write_csv: str) -> str:
     fetch, write = counter_rows(fetch_csv), counter_rows(write_csv)
 
     def calibration(rows, counter):
-        avg, key = _average_for(rows, counter, "at::native::vectorized_elementwise_kernel", None)
-        cands = {k: v for k, v in rows.items() if k[2] == counter and "MulFunctor" in k[0]}
-        if cands:
-            key = max(cands, key=lambda k: len(cands[k]))
-            avg = sum(cands[key]) / len(cands[key])
-        if not avg:
+        # torch.mul(src, 1.0, out=dst) on fp32: vectorized_elementwise_kernel<4, AUnaryFunctor<.. MulFunctor ..>>, every workgroup
+        # of which reads 4 KiB and writes 4 KiB (the calibration copy of 256 MiB is 65536 of them); bench.py's copy-ceiling
+        # leg launches the same kernel on 512 MiB and calibrates as well
+        moved = raw = 0.0
+        for k, v in rows.items():
+            if k[2] == counter and "vectorized_elementwise_kernel<4" in k[0] and "AUnaryFunctor" in k[0] and k[1] >= 65536:
+                moved += 4.0 * k[1] * len(v)
+                raw += sum(v)
+        if not raw:
             raise SystemExit(f"no calibration launch (torch.mul on 256 MiB) found for {counter}: run bench.py with --counter-calibration")
-        return CALIBRATION_KIB / avg
+        return moved / raw
 
     f_scale, w_scale = calibration(fetch, "FETCH_SIZE"), calibration(write, "WRITE_SIZE")
     out = [f"scale FETCH_SIZE x{f_scale:.3f}  WRITE_SIZE x{w_scale:.3f}  (calibration copy = {CALIBRATION_KIB:.0f} KiB each way)"]
