@@ -177,7 +177,9 @@ TTMI_API int ttmi_matmul_bfp(const void *a, int a_layout, const uint32_t *b, int
  * tests/ttnn/unit_tests/operations/test_matmul.py:561-620 multiplies two BFLOAT8_B tensors):
  *   a        packed BFLOAT8_B tiles, tile (mt, kt) of slice s at index (s*Mt + mt)*Kt + kt; m a multiple of 32
  * The kernel that streams the weights expands the activations itself — exactly, to the bf16 values ttmi_typecast_tiles gives —
- * so the result is bit for bit that of ttmi_typecast_tiles(a -> BFLOAT16) followed by ttmi_matmul_bfp, in one launch and
+ * so the result is bit for bit that of ttmi_typecast_tiles(a -> BFLOAT16) followed by ttmi_matmul_bfp (but for face rows
+ * of A with exponent byte 0, values below 2^-126, which the kernel reads with the scale of exponent 1 as it reads such
+ * rows of the weights), in one launch and
  * with no bf16 copy of A (Falcon-7B 4h_to_h, M = 32: 23.4 us against 29.6 us for the two calls).  Only that kernel's
  * one-band form takes them: ttmi_matmul_bfp_ab_supported() says (1 / 0) whether a shape goes there (m == 32 per batch
  * slice: decode); for other shapes, and for BFLOAT4_B activations, the call returns TTMI_ERR_UNSUPPORTED and the caller
