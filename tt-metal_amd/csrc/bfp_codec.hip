@@ -284,7 +284,13 @@ __global__ __launch_bounds__(256) void pack_whole_kernel(const uint8_t *__restri
 
     uint4 raw[ITS];
 #pragma unroll
-    for (int it = 0; it < ITS; ++it) raw[it] = *reinterpret_cast<const uint4 *>(p + (uint64_t)it * s.row_stride * ELEM);
+    for (int it = 0; it < ITS; ++it) {
+        // read once: the non-temporal policy keeps the 64 MiB of a large source from displacing what the caches hold
+        // (measured on fp32 4096 x 4096 -> BFLOAT4_B: 13.6 against 14.1 us)
+        typedef uint32_t v4 __attribute__((ext_vector_type(4)));
+        const v4 v = __builtin_nontemporal_load(reinterpret_cast<const v4 *>(p + (uint64_t)it * s.row_stride * ELEM));
+        raw[it] = make_uint4(v.x, v.y, v.z, v.w);
+    }
 
     const int t = lane / (2 * LPR), fc = (lane / LPR) & 1, q = lane % LPR;
     const int face = (wave >> 1) * 2 + fc, i0 = (wave & 1) * 8;
@@ -471,7 +477,11 @@ __global__ __launch_bounds__(256) void unpack_whole_kernel(const uint8_t *__rest
         const uint4 *in = reinterpret_cast<const uint4 *>(src + tile0 * F::tile_bytes);
         uint4 *out = reinterpret_cast<uint4 *>(stage);
 #pragma unroll
-        for (uint32_t k = threadIdx.x; k < n16; k += 256) out[k] = in[k];
+        for (uint32_t k = threadIdx.x; k < n16; k += 256) {      // read once: non-temporal (13.0 against 13.4 us for BFLOAT4_B -> fp32 4096 x 4096)
+            typedef uint32_t v4 __attribute__((ext_vector_type(4)));
+            const v4 v = __builtin_nontemporal_load(reinterpret_cast<const v4 *>(in + k));
+            out[k] = make_uint4(v.x, v.y, v.z, v.w);
+        }
     }
     __syncthreads();
 
@@ -523,7 +533,7 @@ __global__ __launch_bounds__(256) void unpack_whole_kernel(const uint8_t *__rest
         if (ELEM == 4) v = make_uint4(bits[0], bits[1], bits[2], bits[3]);
         else v = make_uint4((bits[0] >> 16) | (bits[1 % EPL] & 0xffff0000u), (bits[2 % EPL] >> 16) | (bits[3 % EPL] & 0xffff0000u),
                             (bits[4 % EPL] >> 16) | (bits[5 % EPL] & 0xffff0000u), (bits[6 % EPL] >> 16) | (bits[7 % EPL] & 0xffff0000u));
-        *reinterpret_cast<uint4 *>(p + (uint64_t)it * s.row_stride * ELEM) = v;
+        *reinterpret_cast<uint4 *>(p + (uint64_t)it * s.row_stride * ELEM) = v;      // (non-temporal stores here: 14.6 against 13.0 us)
     }
 }
 
