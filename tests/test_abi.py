@@ -69,7 +69,7 @@ def test_matmul_workspace_sizes_follow_the_decomposition():
     assert ws(1, 64, 4544, 18176, 3) == 142 * 3 * 2 * 16384    # two bands per workgroup of the 128-column kernel: two slots each
     assert ws(1, 96, 4544, 18176, 3) == 0                      # three bands, 64-column kernel: 3 x 284 groups fill the chip
     assert ws(12, 384, 1024, 1024, 3) == 0                     # fused tiled kernels
-    assert ws(1, 256, 4096, 4096, 3) == 128 * 3 * 2 * 16384    # too few blocks for the tiled kernels: streamed, 4 pairs of bands x 32 groups, 3 k ranges each, two slots per workgroup
+    assert ws(1, 256, 4096, 4096, 3) == 128 * 4 * 2 * 16384    # too few blocks for the tiled kernels: streamed, 4 pairs of bands x 32 groups, 4 k ranges each (512 workgroups; those that only collect come on top), two slots per workgroup
     assert ws(1, 2048, 4096, 14336, 3) == 4096 * 14336 * 2     # expanded weights
     assert ws(0, 32, 64, 64, 3) == 0
 

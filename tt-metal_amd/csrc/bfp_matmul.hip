@@ -981,6 +981,14 @@ static Decomposition decompose(uint32_t batch, uint32_t m, uint32_t k, uint32_t 
     const bool few = d.groups < 100 || gated;
     const uint64_t resident = knob_or(TTMI_KNOB_MATMUL_WORKGROUPS, wide ? (few ? 256 : 256 * WIDE_WGS_PER_CU) : d.groups >= 256 ? 768 : 512);
     uint64_t parts = d.groups >= resident ? 1 : wide && !few ? resident / (d.groups + 1) : resident / d.groups;
+    // The round of workgroups that only collect may come late (they are the last of the launch and wait for everybody
+    // anyway): where counting them in leaves a quarter of the places empty and one more k range per output fills them
+    // exactly, take it, if every wavefront still keeps 8 k-tiles.  Measured: [32, 4544] x [4544, 16384] (128 groups)
+    // 20.8-21.3 us with 4 ranges against 23.6-24.0 with 3; [4544, 21760] (170 groups) 25.8-26.1 with 3 against 30.9-31.6
+    // with 2; [8192, 16384] 30.7-31.5 against 36.3-36.9.  (More ranges than that cost more than they fill:
+    // [4544, 13056], 102 groups, 22.2-22.9 us with 5 against 19.2-19.7 with 4.)
+    if (wide && !few && d.groups < resident && d.groups * parts * 100 < resident * 78 && d.groups * (parts + 1) <= resident && d.kt >= 8u * WAVES * (parts + 1))
+        ++parts;
     uint32_t asked;
     if (!wide && one_round_of_groups(d.groups) && !knob(TTMI_KNOB_MATMUL_WORKGROUPS, &asked)) parts = 1;
     if (parts == 0) parts = 1;
