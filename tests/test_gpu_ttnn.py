@@ -222,6 +222,44 @@ def test_tt_lib_matmul_and_bmm(device):
     assert torch.equal(out2.cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch(), out.cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch())
 
 
+def test_primary_matmul_1d_with_program_config_and_block_float_chain(device):
+    """tt_lib.operations.primary.matmul_1d (module.hpp:373-406) as Falcon-40B's MLP issues it
+    (models/demos/falcon40b/tt/falcon_mlp.py:97-135): a 1D program config that carries the fused GELU, a BFLOAT8_B output
+    of the first GEMM feeding the second as its activations.  The program config objects are plain holders (keyword-only
+    constructors as in module.hpp:53-122); the fused activation is honoured."""
+    import tt_lib as ttl
+
+    P = ttl.operations.primary
+    torch.manual_seed(9)
+    h, f = 256, 1024
+    x = torch.randn((1, 1, 32, h), dtype=torch.bfloat16) * 0.5
+    w1, w2 = torch.randn((1, 1, h, f)) * 0.05, torch.randn((1, 1, f, h)) * 0.05
+    tx = ttl.tensor.Tensor(x, ttl.tensor.DataType.BFLOAT16).to(ttl.tensor.Layout.TILE).to(device)
+    t1 = ttl.tensor.Tensor(w1, ttl.tensor.DataType.BFLOAT8_B).to(ttl.tensor.Layout.TILE).to(device)
+    t2 = ttl.tensor.Tensor(w2, ttl.tensor.DataType.BFLOAT8_B).to(ttl.tensor.Layout.TILE).to(device)
+    config = P.MatmulMultiCoreReuseMultiCast1DProgramConfig(
+        compute_with_storage_grid_size=(8, 4), in0_block_w=2, out_subblock_h=1, out_subblock_w=4, per_core_M=1, per_core_N=1,
+        fuse_batch=True, fused_activation=[ttl.tensor.FusibleActivation.GELU, True], mcast_in0=True)
+    assert "in0_block_w=2" in repr(config)
+    with pytest.raises(TypeError):
+        P.MatmulMultiCoreReuseMultiCast1DProgramConfig(in0_block_w=2)
+    hidden = P.matmul_1d(tx, t1, program_config=config, output_dtype=ttl.tensor.DataType.BFLOAT8_B)
+    assert hidden.get_dtype() == ttl.tensor.DataType.BFLOAT8_B and tuple(hidden.get_legacy_shape()) == (1, 1, 32, f)
+    out = P.matmul_1d(hidden, t2, output_dtype=ttl.tensor.DataType.BFLOAT16)
+    back = lambda t: t.cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch().double()
+    h_ref = torch.nn.functional.gelu(x.double() @ back(t1))
+    assert np.corrcoef(back(hidden).numpy().ravel(), h_ref.numpy().ravel())[0, 1] >= 0.999
+    ref = back(hidden) @ back(t2)                                  # from the quantised intermediate the device holds
+    got = back(out)
+    bound = 2.0 ** -8 * ref.abs() + 2.0 * f * 2.0 ** -24 * (back(hidden).abs() @ (5.0 * back(t2).abs().amax(dim=-1, keepdim=True).expand_as(back(t2)))) + 1e-30
+    assert bool(((got - ref).abs() <= bound).all())
+    # the same chain op by op with a bf16 intermediate typecast to BFLOAT8_B gives the same hidden tensor
+    plain = P.matmul(tx, t1, program_config=config)
+    assert torch.equal(back(ttl.tensor.typecast(plain, ttl.tensor.DataType.BFLOAT8_B)), back(hidden))
+    with pytest.raises(RuntimeError, match="not supported as activation"):
+        P.matmul(tx, t1, activation="tanh")
+
+
 @pytest.mark.parametrize("m", [32, 64, 96, 160, 544])        # every GEMM kernel: one band, two bands, three bands, tiled, expanded
 def test_untilize_out_gives_the_tile_result_row_major(device, m):
     """bmm_op.cpp:1069: with untilize_out the output tensor is ROW_MAJOR; :536-538, :865-867: bfloat16 only.  The values are
