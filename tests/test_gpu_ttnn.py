@@ -222,6 +222,34 @@ def test_tt_lib_matmul_and_bmm(device):
     assert torch.equal(out2.cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch(), out.cpu().to(ttl.tensor.Layout.ROW_MAJOR).to_torch())
 
 
+@pytest.mark.parametrize("batch_size,m_size,k_size,n_size", [(1, 31, 1024, 1023), (3, 63, 512, 2047)])
+def test_matmul_by_passing_in_1d_systolic_array_program_config(device, batch_size, m_size, k_size, n_size):
+    """tests/ttnn/unit_tests/operations/test_matmul.py:460-486: ttnn.create_matmul_1d_systolic_array_program_config from the
+    padded shapes, passed to ttnn.matmul; here also with block-float weights and with an activation carried by the config."""
+    import ttnn
+
+    torch.manual_seed(0)
+    ta = torch.randn((batch_size, m_size, k_size), dtype=torch.bfloat16)
+    tb = torch.randn((k_size, n_size), dtype=torch.bfloat16)
+    a = ttnn.from_torch(ta, layout=ttnn.TILE_LAYOUT, device=device)
+    for dtype in (ttnn.bfloat16, ttnn.bfloat8_b):
+        b = ttnn.from_torch(tb, layout=ttnn.TILE_LAYOUT, device=device, dtype=dtype)
+        config = ttnn.create_matmul_1d_systolic_array_program_config(
+            input_shape_a=a.shape.with_tile_padding(), input_shape_b=b.shape.with_tile_padding(), core_grid=ttnn.CoreGrid(y=8, x=8))
+        assert config.fused_activation is None and config.fuse_batch is True
+        out = ttnn.to_torch(ttnn.matmul(a, b, program_config=config))
+        ref = ta.double() @ ttnn.to_torch(b).double()
+        assert out.shape == (batch_size, m_size, n_size)
+        assert np.corrcoef(out.double().numpy().ravel(), ref.numpy().ravel())[0, 1] >= 0.9999
+        relu = ttnn.create_matmul_1d_systolic_array_program_config(
+            input_shape_a=a.shape.with_tile_padding(), input_shape_b=b.shape.with_tile_padding(), activation="relu")
+        assert torch.equal(ttnn.to_torch(ttnn.matmul(a, b, program_config=relu)), torch.relu(out))
+    with pytest.raises(RuntimeError):
+        ttnn.create_matmul_1d_systolic_array_program_config(input_shape_a=(32, 64), input_shape_b=(96, 32))
+    with pytest.raises(RuntimeError):
+        ttnn.create_matmul_1d_systolic_array_program_config(input_shape_a=(32, 64), input_shape_b=(64, 32), activation="tanh")
+
+
 def test_primary_matmul_1d_with_program_config_and_block_float_chain(device):
     """tt_lib.operations.primary.matmul_1d (module.hpp:373-406) as Falcon-40B's MLP issues it
     (models/demos/falcon40b/tt/falcon_mlp.py:97-135): a 1D program config that carries the fused GELU, a BFLOAT8_B output

@@ -117,7 +117,7 @@ def is_tensor_storage_on_device(tensor: Tensor) -> bool:
 
 
 from .core import from_torch, to_torch, to_layout, to_device, from_device, reshape, deallocate, unsqueeze_to_4D, clone  # noqa: E402
-from .matmul import matmul, linear  # noqa: E402
+from .matmul import matmul, linear, create_matmul_1d_systolic_array_program_config  # noqa: E402
 from . import experimental  # noqa: E402
 from .elementwise import mul, multiply, add, sub, subtract, gelu, relu, silu  # noqa: E402
 from .files import load_tensor, dump_tensor, as_tensor, get_memory_config  # noqa: E402
