@@ -141,3 +141,18 @@ def test_as_tensor_and_clone_argument_checks():
         ttnn.to_layout(ttnn.from_torch(torch.zeros(32, 32, dtype=torch.bfloat16)), ttnn.TILE_LAYOUT, dtype=ttnn.bfloat8_b)
     with pytest.raises(RuntimeError, match="cannot slice"):
         ttnn.from_torch(torch.zeros(4, 4))[:2]
+
+
+def test_tensix_only_objects_exist_and_are_inert():
+    """Objects that model code constructs for a Tensix device — compute kernel configs, core grids, interleaved memory
+    configs — exist with the reference's constructor arguments (tt_lib_bindings_tensor.cpp:325-348) and steer nothing."""
+    import ttnn
+
+    cfg = ttnn.WormholeComputeKernelConfig(math_fidelity=ttnn.MathFidelity.HiFi4, math_approx_mode=False, fp32_dest_acc_en=True, packer_l1_acc=True)
+    assert (cfg.math_fidelity, cfg.math_approx_mode, cfg.fp32_dest_acc_en, cfg.packer_l1_acc) == (ttnn.MathFidelity.HiFi4, False, True, True)
+    assert ttnn.GrayskullComputeKernelConfig(math_fidelity=ttnn.MathFidelity.LoFi).math_approx_mode is True
+    with pytest.raises(TypeError):
+        ttnn.WormholeComputeKernelConfig(ttnn.MathFidelity.HiFi4)          # keyword-only, as bound
+    marker = object()
+    assert ttnn.to_memory_config(marker, ttnn.DRAM_MEMORY_CONFIG) is marker and ttnn.to_memory_config(marker, ttnn.L1_MEMORY_CONFIG) is marker
+    assert ttnn.CoreGrid(y=8, x=8).num_cores == 64

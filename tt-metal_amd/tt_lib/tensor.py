@@ -387,6 +387,21 @@ def bert_large_post_softmax_bmm(input_a: Tensor, input_b: Tensor, output_mem_con
     return _matmul(input_a, input_b, bcast_batch=False, output_dtype=output_dtype, op="bert_large_post_softmax_bmm")
 
 
+# ---- compute kernel configs (tt_lib_bindings_tensor.cpp:325-348) ----------------------------------------------------
+class GrayskullComputeKernelConfig:
+    """Fidelity phases of the Tensix matrix unit: nothing of it applies here (the GEMMs multiply exact bf16 operands and add in
+    fp32 whatever it says); model code constructs it and passes it as ``compute_kernel_config``, so the object exists."""
+
+    def __init__(self, *, math_fidelity=None, math_approx_mode: bool = True):
+        self.math_fidelity, self.math_approx_mode = math_fidelity, math_approx_mode
+
+
+class WormholeComputeKernelConfig:
+    def __init__(self, *, math_fidelity=None, math_approx_mode: bool = True, fp32_dest_acc_en: bool = False, packer_l1_acc: bool = False):
+        self.math_fidelity, self.math_approx_mode = math_fidelity, math_approx_mode
+        self.fp32_dest_acc_en, self.packer_l1_acc = fp32_dest_acc_en, packer_l1_acc
+
+
 # ---- fused activations and the Falcon matmuls (bmm_op.cpp:747-807) -------------------------------------------------
 class FusibleActivation(enum.IntEnum):  # UnaryOpType, tt_eager/tt_dnn/op_library/eltwise_unary/eltwise_unary_op.hpp:17-78
     GELU = 2

@@ -14,6 +14,7 @@ from typing import Optional, Tuple, Union
 import tt_lib as ttl
 
 from tt_lib.tensor import DataType, Layout, StorageType, MemoryConfig, BufferType, TensorMemoryLayout, MathFidelity, Device, Tensor
+from tt_lib.tensor import GrayskullComputeKernelConfig, WormholeComputeKernelConfig  # noqa: F401  (accepted by matmul / linear and ignored)
 from ttmi import capi as _capi
 
 # ---- ttnn/ttnn/types.py ----------------------------------------------------------------------------------
@@ -110,6 +111,16 @@ def synchronize_device(device: Optional[Device] = None) -> None:
     import torch
 
     torch.cuda.synchronize()
+
+
+def to_memory_config(tensor: Tensor, memory_config=None) -> Tensor:
+    """ttnn/ttnn/operations/core.py:484-606 moves a tensor between DRAM, L1 and sharded layouts of a Tensix device.  One GPU has
+    one memory, HBM, and every tensor is interleaved in it: an interleaved target is where the tensor already is; a sharded
+    one has no meaning here and raises."""
+    layout = getattr(memory_config, "memory_layout", None)
+    if layout is not None and layout != TensorMemoryLayout.INTERLEAVED:
+        raise RuntimeError("ttnn.to_memory_config: sharded memory configs describe Tensix L1 and are not supported on this device")
+    return tensor
 
 
 def is_tensor_storage_on_device(tensor: Tensor) -> bool:
