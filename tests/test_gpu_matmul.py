@@ -400,6 +400,22 @@ def test_decode_shapes_full_size(oracle, name, m, k, n, fmt, batch, layout):
     print(name, "pcc", pcc)
 
 
+@pytest.mark.parametrize("m,k,n,fmt", [(32, 4096, 16384, "bfp8_b"), (32, 4096, 21760, "bfp4_b"), (256, 4096, 4096, "bfp8_b")])
+def test_shapes_whose_collecting_workgroups_come_on_top(oracle, m, k, n, fmt):
+    """128 and 170 output groups (and 4 pairs of row bands x 32): one more k range per output fills the places that the
+    workgroups which only collect would have been given, so those come on top of a full chip and start late.  Every
+    output element against the float64 product with the oracle-unpacked weights."""
+    plan = (ctypes.c_uint32 * 4)()
+    capi.lib().ttmi_matmul_bfp_plan(1, m, k, n, capi.BFLOAT16, FMT[fmt], capi.BFLOAT16, plan)
+    assert plan[0] == 2 and plan[2] > 512, list(plan)                    # 128-column kernel, more workgroups than places
+    a_bits = workloads.activations_bf16(m, k, seed=86)
+    words = capi.pack_tensor(FMT[fmt], dev(workloads.weights_f32(k, n, seed=87)))
+    w_unpacked = oracle_unpacked(oracle, FMT[fmt], words, k, n)[0]
+    c = capi.matmul_bfp(bf16_dev(a_bits), capi.ROW_MAJOR, words, FMT[fmt], 1, 1, m, k, n)
+    capi.device_status()
+    check_on_gpu(c[0], a_bits, w_unpacked, k)
+
+
 @pytest.mark.parametrize("m", [64, 128 - 3])
 @pytest.mark.parametrize("name,k,n,fmt", [("falcon_h_to_4h", 4544, 18176, "bfp8_b"), ("falcon_4h_to_h", 18176, 4544, "bfp8_b"), ("mistral_gate", 4096, 14336, "bfp4_b")])
 def test_two_and_four_row_bands_full_size(oracle, name, m, k, n, fmt):
